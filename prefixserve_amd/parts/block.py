@@ -1,0 +1,37 @@
+"""How a layer's parts are arranged."""
+
+from __future__ import annotations
+
+from typing import TYPE_CHECKING, Any
+
+import torch
+
+from .base import FeedForward, Mixer, Norm, Part, register_block
+
+if TYPE_CHECKING:
+    from prefixserve_amd.engine.batch import StepContext
+
+
+class PreNormBlock:
+    """norm -> mixer -> add, norm -> feed-forward -> add (prefixserve/model/llama.py:111-121).
+
+    The residual stream is float32. Each sub-layer's output is not added at once: it is
+    handed on as ``pending`` and summed into the residual by the next norm's fused
+    add+norm, so the stream is read and written once per sub-layer."""
+
+    def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm, feed_forward_norm: Norm) -> None:
+        self.mixer, self.feed_forward = mixer, feed_forward
+        self.mixer_norm, self.feed_forward_norm = mixer_norm, feed_forward_norm
+
+    def parts(self) -> list[Part]:
+        return [self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward]
+
+    def forward(self, residual: torch.Tensor, pending: torch.Tensor | None, ctx: "StepContext", cache: Any,
+                state: torch.Tensor | None, writes_cache: bool) -> torch.Tensor:
+        x = self.mixer_norm.add_norm(residual, pending, "block.x")
+        mixed = self.mixer.forward(x, ctx, cache, state, writes_cache)
+        x = self.feed_forward_norm.add_norm(residual, mixed, "block.x")
+        return self.feed_forward.forward(x, ctx)
+
+
+register_block("prenorm", PreNormBlock)
