@@ -1,0 +1,64 @@
+// C interface of the kernel library (libpsamd_kernels.so). Every function launches on the
+// given HIP stream, takes raw device pointers, returns 0 on success and otherwise leaves a
+// message for psamd_last_error(). dtype codes: 0 = float32, 1 = bfloat16. Shapes are checked
+// on the host before a launch; a shape a kernel does not take is an error, never a wrong
+// result.
+#pragma once
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* psamd_last_error(void);
+
+// out[t, :] = float(table[ids[t], :])
+int psamd_embed(void* stream, const int32_t* ids, const void* table, int table_dtype, float* out, int64_t tokens,
+                int hidden);
+
+// rows == NULL: residual[r] += delta[r] (if delta), out[r] = weight * rmsnorm(residual[r]) for r < out_rows.
+// rows != NULL: out[i] = weight * rmsnorm(residual[rows[i]] + delta[rows[i]]); residual untouched.
+int psamd_add_rmsnorm(void* stream, float* residual, const void* delta, const int32_t* rows, const void* weight,
+                      int weight_dtype, float eps, void* out, int act_dtype, int64_t out_rows, int hidden);
+
+// out[t, c] = silu(gate_up[t, c]) * gate_up[t, inter + c]
+int psamd_swiglu(void* stream, const void* gate_up, void* out, int act_dtype, int64_t tokens, int inter);
+
+// Rotates the q and k heads of qkv[t] in place by table[positions[t]] (NULL table: no rotation) and, if kv
+// is given, writes k and v of token t to page slot write_slot[t] (= page * 16 + offset).
+int psamd_rope_kv_append(void* stream, void* qkv, int act_dtype, int64_t tokens, int hq, int hkv, int head_dim,
+                         const int32_t* positions, const float* table, void* kv, const int32_t* write_slot);
+
+// out[M, N] = x[M, K] * w[N, K]^T with float accumulation (LDS-tiled FMA; exact path and fallback).
+int psamd_linear(void* stream, const void* x, int x_dtype, const void* w, int w_dtype, void* out, int out_dtype,
+                 int64_t M, int N, int K);
+
+// bfloat16 product for M <= 64 on the matrix cores. epilogue 1: w = [gate; up], out = silu(gate) * up.
+int psamd_linear_skinny(void* stream, const void* x, const void* w, void* out, int out_dtype, int M, int n_out, int K,
+                        int epilogue);
+
+int psamd_attention_generic(void* stream, const void* qkv, int q_stride, void* out, const void* kv, int act_dtype,
+                            int64_t tokens, const int32_t* positions, const int32_t* tok_item,
+                            const int32_t* table_off, const int32_t* block_ids, int hq, int hkv, int head_dim,
+                            float scale, int window);
+
+int psamd_attention_mfma_supports(int hq, int hkv, int head_dim);
+
+int psamd_attention_prefill(void* stream, const void* qkv, int q_stride, void* out, const void* kv,
+                            const int32_t* pf_tiles, int n_tiles, const int32_t* item_start, const int32_t* item_pos0,
+                            const int32_t* table_off, const int32_t* block_ids, int hq, int hkv, int head_dim,
+                            float scale, int window);
+
+int psamd_attention_decode(void* stream, const void* qkv, int q_stride, void* out, const void* kv, float* part_o,
+                           float* part_ml, const int32_t* dec_items, int n_dec, const int32_t* item_start,
+                           const int32_t* item_end, const int32_t* table_off, const int32_t* block_ids, int hq,
+                           int hkv, int head_dim, int nsplit, float scale, int window);
+
+// out[r] = argmax (temperature[r] <= 0) or the inverse-CDF draw with uniform[r] in [0, 1).
+int psamd_sample(void* stream, const float* logits, const float* temperature, const float* uniform, int32_t* out,
+                 int rows, int vocab);
+
+#ifdef __cplusplus
+}
+#endif

@@ -1,0 +1,462 @@
+// bfloat16 causal grouped-query attention over the paged cache on the CDNA4 matrix cores.
+//
+// Both kernels compute the score tile TRANSPOSED, S^T = K * Q^T (keys are rows), because the
+// accumulator layout of S^T is, lane for lane, the B-operand layout of the next product
+// O^T = V^T * P^T: probabilities go from the first product's registers straight into the
+// second without passing through LDS. The cache stores values transposed per page
+// ([D][16], see elementwise.hip) so that V^T rows are contiguous 8-byte runs.
+//
+//  * prefill: one wave per (32 new tokens, query head); v_mfma_f32_32x32x16_bf16; online
+//    softmax per query column held redundantly in lanes l and l^32.
+//  * decode: one workgroup per (request, kv head, split of the key range); the `group`
+//    query heads sharing the kv head are the columns of a 16x16x32 tile, so every key and
+//    value byte is read once for all of them; 4 waves interleave 32-key tiles and merge by
+//    log-sum-exp in LDS; a second small kernel merges the splits.
+//
+// Softmax statistics, scaling and masks are float. Page layout per layer:
+// [num_blocks][2][kv_heads][16 * D], half 0 keys [16][D], half 1 values [D][16].
+
+#include "api.h"
+#include "common.h"
+
+namespace psamd {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+__device__ __forceinline__ bf16x8 ld8(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
+__device__ __forceinline__ bf16x4 ld4(const bf16_t* p) { return *reinterpret_cast<const bf16x4*>(p); }
+
+__device__ __forceinline__ bf16x8 zeros8() {
+  bf16x8 z;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = static_cast<__bf16>(0.f);
+  return z;
+}
+
+__device__ __forceinline__ bf16x8 join(bf16x4 a, bf16x4 b) {
+  bf16x8 r;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    r[i] = a[i];
+    r[i + 4] = b[i];
+  }
+  return r;
+}
+
+// ------------------------------------------------------------------ prefill
+
+// NS = D / 16. Block = 4 waves = 128 consecutive queries of one item, one query head.
+template <int NS>
+__global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
+    const bf16_t* __restrict__ qkv, int q_stride, bf16_t* __restrict__ out, const bf16_t* __restrict__ kv,
+    const int32_t* __restrict__ pf_tiles, const int32_t* __restrict__ item_start,
+    const int32_t* __restrict__ item_pos0, const int32_t* __restrict__ table_off,
+    const int32_t* __restrict__ block_ids, int hq, int hkv, float scale, int window) {
+  constexpr int D = 16 * NS;
+  constexpr int DT = (D + 31) / 32;
+  const int tile = blockIdx.x, h = blockIdx.y;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int item = pf_tiles[2 * tile];
+  const int q_off = pf_tiles[2 * tile + 1] + wave * 32;
+  const int t0 = item_start[item];
+  const int n = item_start[item + 1] - t0;
+  if (q_off >= n) return;
+  const int pos0 = item_pos0[item];
+  const int kvh = h / (hq / hkv);
+  const int32_t* table = block_ids + table_off[item];
+  const int col = lane & 31, hi = lane >> 5;
+
+  const int qi = min(q_off + col, n - 1);          // lanes past the end repeat the last query
+  const bool q_valid = q_off + col < n;
+  const int q_pos = pos0 + qi;
+  const int first_pos = pos0 + q_off;
+  const int last_pos = pos0 + min(q_off + 31, n - 1);
+  const int max_key = pos0 + n - 1;
+  const int k_lo_q = window > 0 ? max(0, q_pos - window + 1) : 0;
+  const int k_begin = window > 0 ? (max(0, first_pos - window + 1) & ~31) : 0;
+
+  bf16x8 qf[NS];
+  {
+    const bf16_t* qp = qkv + static_cast<int64_t>(t0 + qi) * q_stride + h * D + 8 * hi;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) qf[s] = ld8(qp + 16 * s);
+  }
+
+  f32x16 o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) o[dt][v] = 0.f;
+  float m = -INFINITY, l = 0.f;
+
+  const int64_t page_elems = 2LL * hkv * kPage * D;
+  const int64_t khead = static_cast<int64_t>(kvh) * kPage * D;
+  const int64_t vhead = static_cast<int64_t>(hkv) * kPage * D + static_cast<int64_t>(kvh) * D * kPage;
+
+  for (int k0 = k_begin; k0 <= last_pos; k0 += 32) {
+    // ---- S^T[key][query] = K . Q^T : lane supplies key row (k0 + col) of K
+    const int key_a = min(k0 + col, max_key);
+    const bf16_t* kp = kv + static_cast<int64_t>(table[key_a >> 4]) * page_elems + khead + (key_a & 15) * D + 8 * hi;
+    f32x16 s;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) s[v] = 0.f;
+#pragma unroll
+    for (int i = 0; i < NS; ++i) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ld8(kp + 16 * i), qf[i], s, 0, 0, 0);
+
+    // ---- mask, scale, online softmax for query column `col`
+    float sv[16];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int key = k0 + 8 * (v >> 2) + 4 * hi + (v & 3);
+      const bool ok = key <= q_pos && key >= k_lo_q;
+      sv[v] = ok ? s[v] * scale : -INFINITY;
+      mx = fmaxf(mx, sv[v]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+    const float m_new = fmaxf(m, mx);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = __expf(m - m_use);
+    float rowsum = 0.f;
+    bf16x8 pb[2];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const float p = __expf(sv[v] - m_use);
+      rowsum += p;
+      pb[v >> 3][v & 7] = static_cast<__bf16>(p);
+    }
+    rowsum += __shfl_xor(rowsum, 32, kWave);
+    l = l * alpha + rowsum;
+    m = m_new;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) o[dt][v] *= alpha;
+
+    // ---- O^T[d][query] += V^T . P^T : half c of the tile is page c; lane supplies V^T row d
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      const int key_p = min(k0 + 16 * c, max_key);
+      const bf16_t* vp = kv + static_cast<int64_t>(table[key_p >> 4]) * page_elems + vhead + 4 * hi;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        const int drow = min(32 * dt + col, D - 1);
+        const bf16_t* vr = vp + drow * kPage;
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(join(ld4(vr), ld4(vr + 8)), pb[c], o[dt], 0, 0, 0);
+      }
+    }
+  }
+
+  if (!q_valid) return;
+  const float inv = 1.f / l;
+  bf16_t* op = out + static_cast<int64_t>(t0 + qi) * (static_cast<int64_t>(hq) * D) + h * D;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+    for (int v4 = 0; v4 < 4; ++v4) {
+      const int d = 32 * dt + 8 * v4 + 4 * hi;
+      if (d < D) {
+        ushort4 pk;
+        pk.x = float_to_bf16(o[dt][4 * v4 + 0] * inv);
+        pk.y = float_to_bf16(o[dt][4 * v4 + 1] * inv);
+        pk.z = float_to_bf16(o[dt][4 * v4 + 2] * inv);
+        pk.w = float_to_bf16(o[dt][4 * v4 + 3] * inv);
+        *reinterpret_cast<ushort4*>(op + d) = pk;
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------ decode (split keys)
+
+// NS = D / 16, CT = ceil(group / 16) column tiles of query heads.
+// part_o[dec][head][split][D], part_ml[dec][head][split][2] = (max, sum).
+template <int NS, int CT>
+__global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
+    const bf16_t* __restrict__ qkv, int q_stride, const bf16_t* __restrict__ kv, float* __restrict__ part_o,
+    float* __restrict__ part_ml, const int32_t* __restrict__ dec_items, const int32_t* __restrict__ item_start,
+    const int32_t* __restrict__ item_end, const int32_t* __restrict__ table_off,
+    const int32_t* __restrict__ block_ids, int hq, int hkv, int nsplit, float scale, int window) {
+  constexpr int D = 16 * NS;
+  constexpr int KS = (D + 31) / 32;
+  extern __shared__ float smem[];
+  const int di = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r = lane & 15, g4 = lane >> 4;
+  const int item = dec_items[di];
+  const int64_t t = item_start[item];
+  const int pos = item_end[item] - 1;
+  const int group = hq / hkv;
+  const int32_t* table = block_ids + table_off[item];
+  const int k_lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int tile_lo = k_lo >> 5, tile_hi = pos >> 5;
+  const int tps = (tile_hi - tile_lo + nsplit) / nsplit;   // ceil(ntiles / nsplit)
+  const int my_lo = tile_lo + split * tps;
+  const int my_hi = min(my_lo + tps, tile_hi + 1);
+
+  const int64_t page_elems = 2LL * hkv * kPage * D;
+  const int64_t khead = static_cast<int64_t>(kvh) * kPage * D;
+  const int64_t vhead = static_cast<int64_t>(hkv) * kPage * D + static_cast<int64_t>(kvh) * D * kPage;
+
+  bf16x8 qf[CT][KS];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const int hh = ct * 16 + r;
+    const bf16_t* qp = qkv + t * q_stride + static_cast<int64_t>(kvh * group + min(hh, group - 1)) * D + 8 * g4;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const bool in = hh < group && 32 * ks + 8 * g4 < D;
+      qf[ct][ks] = in ? ld8(qp + 32 * ks) : zeros8();
+    }
+  }
+
+  f32x4 o[CT][NS];
+  float m[CT], l[CT];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    m[ct] = -INFINITY;
+    l[ct] = 0.f;
+#pragma unroll
+    for (int ds = 0; ds < NS; ++ds) o[ct][ds] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  for (int tile = my_lo + wave; tile < my_hi; tile += 4) {
+    const int k0 = tile << 5;
+    // Each 16-key half of the tile is exactly one page.
+    const int64_t page0 = table[min(k0, pos) >> 4];
+    const int64_t page1 = table[min(k0 + 16, pos) >> 4];
+    const bf16_t* kp0 = kv + page0 * page_elems + khead + r * D + 8 * g4;
+    const bf16_t* kp1 = kv + page1 * page_elems + khead + r * D + 8 * g4;
+    bf16x8 ka0[KS], ka1[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const bool in = 32 * ks + 8 * g4 < D;
+      ka0[ks] = in ? ld8(kp0 + 32 * ks) : zeros8();
+      ka1[ks] = in ? ld8(kp1 + 32 * ks) : zeros8();
+    }
+    const bf16_t* vp0 = kv + page0 * page_elems + vhead + 4 * g4;
+    const bf16_t* vp1 = kv + page1 * page_elems + vhead + 4 * g4;
+    bf16x8 va[NS];
+#pragma unroll
+    for (int ds = 0; ds < NS; ++ds) {
+      const int drow = 16 * ds + r;
+      va[ds] = join(ld4(vp0 + drow * kPage), ld4(vp1 + drow * kPage));
+    }
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+      f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka0[ks], qf[ct][ks], s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka1[ks], qf[ct][ks], s1, 0, 0, 0);
+      }
+      float sv[8];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int key0 = k0 + 4 * g4 + v, key1 = key0 + 16;
+        sv[v] = (key0 <= pos && key0 >= k_lo) ? s0[v] * scale : -INFINITY;
+        sv[v + 4] = (key1 <= pos && key1 >= k_lo) ? s1[v] * scale : -INFINITY;
+        mx = fmaxf(mx, fmaxf(sv[v], sv[v + 4]));
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+      const float m_new = fmaxf(m[ct], mx);
+      const float m_use = m_new == -INFINITY ? 0.f : m_new;
+      const float alpha = __expf(m[ct] - m_use);
+      float rowsum = 0.f;
+      bf16x8 pb;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float p = __expf(sv[e] - m_use);
+        rowsum += p;
+        pb[e] = static_cast<__bf16>(p);
+      }
+      rowsum += __shfl_xor(rowsum, 16, kWave);
+      rowsum += __shfl_xor(rowsum, 32, kWave);
+      l[ct] = l[ct] * alpha + rowsum;
+      m[ct] = m_new;
+#pragma unroll
+      for (int ds = 0; ds < NS; ++ds) {
+        o[ct][ds] *= alpha;
+        o[ct][ds] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[ds], pb, o[ct][ds], 0, 0, 0);
+      }
+    }
+  }
+
+  // ---- merge the 4 waves: smem = m[4][group], l[4][group], o[4][group][D]
+  float* sm_m = smem;
+  float* sm_l = smem + 4 * group;
+  float* sm_o = smem + 8 * group;
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const int hh = ct * 16 + r;
+    if (hh < group) {
+      if (g4 == 0) {
+        sm_m[wave * group + hh] = m[ct];
+        sm_l[wave * group + hh] = l[ct];
+      }
+#pragma unroll
+      for (int ds = 0; ds < NS; ++ds)
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+          sm_o[(static_cast<int64_t>(wave) * group + hh) * D + 16 * ds + 4 * g4 + v] = o[ct][ds][v];
+    }
+  }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < group * D; idx += blockDim.x) {
+    const int hh = idx / D, d = idx - hh * D;
+    float mm = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) mm = fmaxf(mm, sm_m[w * group + hh]);
+    float acc = 0.f, ll = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float mw = sm_m[w * group + hh];
+      const float wgt = mw == -INFINITY ? 0.f : __expf(mw - mm);
+      acc += wgt * sm_o[(static_cast<int64_t>(w) * group + hh) * D + d];
+      ll += wgt * sm_l[w * group + hh];
+    }
+    const int64_t slot = (static_cast<int64_t>(di) * hq + kvh * group + hh) * nsplit + split;
+    part_o[slot * D + d] = acc;
+    if (d == 0) {
+      part_ml[slot * 2 + 0] = mm;
+      part_ml[slot * 2 + 1] = ll;
+    }
+  }
+}
+
+// One block per (decode item, head): merges the splits and writes bfloat16.
+__global__ void attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                         bf16_t* __restrict__ out, const int32_t* __restrict__ dec_items,
+                                         const int32_t* __restrict__ item_start, int hq, int d, int nsplit) {
+  const int di = blockIdx.x, h = blockIdx.y;
+  const int64_t t = item_start[dec_items[di]];
+  const int64_t base = (static_cast<int64_t>(di) * hq + h) * nsplit;
+  float mm = -INFINITY;
+  for (int s = 0; s < nsplit; ++s) mm = fmaxf(mm, part_ml[(base + s) * 2]);
+  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    float acc = 0.f, ll = 0.f;
+    for (int s = 0; s < nsplit; ++s) {
+      const float ms = part_ml[(base + s) * 2];
+      const float wgt = ms == -INFINITY ? 0.f : __expf(ms - mm);
+      acc += wgt * part_o[(base + s) * d + i];
+      ll += wgt * part_ml[(base + s) * 2 + 1];
+    }
+    out[t * (static_cast<int64_t>(hq) * d) + h * d + i] = float_to_bf16(acc / ll);
+  }
+}
+
+template <int NS>
+static int launch_prefill(hipStream_t s, const void* qkv, int q_stride, void* out, const void* kv,
+                          const int32_t* pf_tiles, int n_tiles, const int32_t* item_start, const int32_t* item_pos0,
+                          const int32_t* table_off, const int32_t* block_ids, int hq, int hkv, float scale, int window) {
+  attn_prefill_mfma_kernel<NS><<<dim3(n_tiles, hq), dim3(256), 0, s>>>(
+      static_cast<const bf16_t*>(qkv), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(kv), pf_tiles,
+      item_start, item_pos0, table_off, block_ids, hq, hkv, scale, window);
+  return check_launch("psamd_attention_prefill");
+}
+
+template <int NS, int CT>
+static int launch_decode(hipStream_t s, const void* qkv, int q_stride, const void* kv, float* part_o, float* part_ml,
+                         const int32_t* dec_items, int n_dec, const int32_t* item_start, const int32_t* item_end,
+                         const int32_t* table_off, const int32_t* block_ids, int hq, int hkv, int nsplit, float scale,
+                         int window) {
+  const int group = hq / hkv;
+  const size_t smem = sizeof(float) * (8 * group + 4 * static_cast<size_t>(group) * 16 * NS);
+  attn_decode_mfma_kernel<NS, CT><<<dim3(n_dec, hkv, nsplit), dim3(256), smem, s>>>(
+      static_cast<const bf16_t*>(qkv), q_stride, static_cast<const bf16_t*>(kv), part_o, part_ml, dec_items,
+      item_start, item_end, table_off, block_ids, hq, hkv, nsplit, scale, window);
+  return check_launch("psamd_attention_decode");
+}
+
+template <int NS>
+static int dispatch_decode_ct(int ct, hipStream_t s, const void* qkv, int q_stride, const void* kv, float* part_o,
+                              float* part_ml, const int32_t* dec_items, int n_dec, const int32_t* item_start,
+                              const int32_t* item_end, const int32_t* table_off, const int32_t* block_ids, int hq,
+                              int hkv, int nsplit, float scale, int window) {
+#define PSAMD_DEC(CT_)                                                                                             \
+  return launch_decode<NS, CT_>(s, qkv, q_stride, kv, part_o, part_ml, dec_items, n_dec, item_start, item_end, \
+                                table_off, block_ids, hq, hkv, nsplit, scale, window)
+  switch (ct) {
+    case 1: PSAMD_DEC(1);
+    case 2: PSAMD_DEC(2);
+    default: PSAMD_DEC(4);
+  }
+#undef PSAMD_DEC
+}
+
+}  // namespace psamd
+
+using namespace psamd;
+
+extern "C" {
+
+// 1 if the matrix-core kernels take this shape, else 0 (the caller then uses the generic kernel).
+int psamd_attention_mfma_supports(int hq, int hkv, int head_dim) {
+  if (hq <= 0 || hkv <= 0 || hq % hkv) return 0;
+  const int group = hq / hkv;
+  const bool dim_ok = head_dim == 16 || head_dim == 32 || head_dim == 64 || head_dim == 96 || head_dim == 128 ||
+                      head_dim == 256;
+  const size_t smem = sizeof(float) * (8 * group + 4 * static_cast<size_t>(group) * head_dim);
+  return dim_ok && group <= 64 && smem <= 64 * 1024 && hq <= 65535 && hkv <= 65535;
+}
+
+int psamd_attention_prefill(void* stream, const void* qkv, int q_stride, void* out, const void* kv,
+                            const int32_t* pf_tiles, int n_tiles, const int32_t* item_start,
+                            const int32_t* item_pos0, const int32_t* table_off, const int32_t* block_ids, int hq,
+                            int hkv, int head_dim, float scale, int window) {
+  PSAMD_REQUIRE(psamd_attention_mfma_supports(hq, hkv, head_dim), "shape not supported by the matrix-core kernels");
+  PSAMD_REQUIRE(q_stride % 8 == 0, "query row stride must be a multiple of 8 elements");
+  if (n_tiles == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define PSAMD_PF(NS_)                                                                                           \
+  return launch_prefill<NS_>(s, qkv, q_stride, out, kv, pf_tiles, n_tiles, item_start, item_pos0, table_off, \
+                             block_ids, hq, hkv, scale, window)
+  switch (head_dim / 16) {
+    case 1: PSAMD_PF(1);
+    case 2: PSAMD_PF(2);
+    case 4: PSAMD_PF(4);
+    case 6: PSAMD_PF(6);
+    case 8: PSAMD_PF(8);
+    default: PSAMD_PF(16);
+  }
+#undef PSAMD_PF
+}
+
+// part_o needs n_dec * hq * nsplit * head_dim floats, part_ml n_dec * hq * nsplit * 2.
+int psamd_attention_decode(void* stream, const void* qkv, int q_stride, void* out, const void* kv, float* part_o,
+                           float* part_ml, const int32_t* dec_items, int n_dec, const int32_t* item_start,
+                           const int32_t* item_end, const int32_t* table_off, const int32_t* block_ids, int hq,
+                           int hkv, int head_dim, int nsplit, float scale, int window) {
+  PSAMD_REQUIRE(psamd_attention_mfma_supports(hq, hkv, head_dim), "shape not supported by the matrix-core kernels");
+  PSAMD_REQUIRE(q_stride % 8 == 0, "query row stride must be a multiple of 8 elements");
+  PSAMD_REQUIRE(nsplit >= 1 && nsplit <= 65535, "nsplit out of range");
+  if (n_dec == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int group = hq / hkv;
+  const int ct = group <= 16 ? 1 : (group <= 32 ? 2 : 4);
+  int rc;
+#define PSAMD_DEC_NS(NS_)                                                                                          \
+  rc = dispatch_decode_ct<NS_>(ct, s, qkv, q_stride, kv, part_o, part_ml, dec_items, n_dec, item_start, item_end, \
+                               table_off, block_ids, hq, hkv, nsplit, scale, window);                            \
+  break
+  switch (head_dim / 16) {
+    case 1: PSAMD_DEC_NS(1);
+    case 2: PSAMD_DEC_NS(2);
+    case 4: PSAMD_DEC_NS(4);
+    case 6: PSAMD_DEC_NS(6);
+    case 8: PSAMD_DEC_NS(8);
+    default: PSAMD_DEC_NS(16);
+  }
+#undef PSAMD_DEC_NS
+  if (rc != 0) return rc;
+  attn_decode_merge_kernel<<<dim3(n_dec, hq), dim3(64), 0, s>>>(part_o, part_ml, static_cast<bf16_t*>(out), dec_items,
+                                                               item_start, hq, head_dim, nsplit);
+  return check_launch("psamd_attention_decode(merge)");
+}
+
+}  // extern "C"

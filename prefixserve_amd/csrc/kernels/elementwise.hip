@@ -1,0 +1,203 @@
+// Memory-bound kernels around the matrix products: token gather, fused residual-add +
+// RMSNorm, SwiGLU, and rotary encoding fused with the write of keys and values into their
+// cache pages. Each is templated on the activation type (bfloat16 or float); statistics,
+// rotation and the residual sum are always float.
+
+#include "api.h"
+#include "common.h"
+
+namespace psamd {
+
+static thread_local std::string g_error;
+void set_error(const std::string& msg) { g_error = msg; }
+
+// ------------------------------------------------------------------ embed
+
+template <typename W>
+__global__ void embed_kernel(const int32_t* __restrict__ ids, const W* __restrict__ table,
+                             float* __restrict__ out, int hidden) {
+  const int64_t t = blockIdx.x;
+  const W* row = table + static_cast<int64_t>(ids[t]) * hidden;
+  float* o = out + t * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = to_float<W>(row[i]);
+}
+
+// ------------------------------------------------------------------ add + rmsnorm
+
+// One block per output row. residual (float) += delta; out = weight * x * rsqrt(mean(x^2)+eps).
+// With `rows` the block handles residual row rows[blockIdx.x] and leaves the residual as it is.
+template <typename A, int kThreads>
+__global__ void add_rmsnorm_kernel(float* __restrict__ residual, const A* __restrict__ delta,
+                                   const int32_t* __restrict__ rows, const void* __restrict__ weight,
+                                   int weight_dtype, float eps, A* __restrict__ out, int hidden) {
+  __shared__ float scratch[kThreads / kWave];
+  const int64_t src = rows != nullptr ? rows[blockIdx.x] : blockIdx.x;
+  float* r = residual + src * hidden;
+  const A* d = delta != nullptr ? delta + src * hidden : nullptr;
+  A* o = out + static_cast<int64_t>(blockIdx.x) * hidden;
+  const bool store = rows == nullptr && d != nullptr;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += kThreads) {
+    float x = r[i];
+    if (d != nullptr) x += to_float<A>(d[i]);
+    if (store) r[i] = x;
+    ss += x * x;
+  }
+  ss = block_sum(ss, scratch, kThreads / kWave);
+  const float inv = rsqrtf(ss / static_cast<float>(hidden) + eps);
+  for (int i = threadIdx.x; i < hidden; i += kThreads) {
+    float x = r[i];
+    if (!store && d != nullptr) x += to_float<A>(d[i]);
+    o[i] = from_float<A>(load_as_float(weight, weight_dtype, i) * (x * inv));
+  }
+}
+
+// ------------------------------------------------------------------ swiglu
+
+template <typename A>
+__global__ void swiglu_kernel(const A* __restrict__ gate_up, A* __restrict__ out, int64_t tokens, int inter) {
+  const int64_t n = tokens * inter;
+  for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < n;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const int64_t t = i / inter, c = i - t * inter;
+    const float g = to_float<A>(gate_up[t * 2 * inter + c]);
+    const float u = to_float<A>(gate_up[t * 2 * inter + inter + c]);
+    out[i] = from_float<A>(g / (1.f + __expf(-g)) * u);
+  }
+}
+
+// ------------------------------------------------------------------ rope + kv append
+
+// One block per token. q and k heads of the fused qkv row are rotated in place (pair
+// (i, i + D/2), angle table [pos][i] = (cos, sin)); the rotated keys go to their page as
+// [16, D] rows and the values to the page's second half transposed, [D, 16].
+template <typename A>
+__global__ void rope_kv_append_kernel(A* __restrict__ qkv, int hq, int hkv, int d,
+                                      const int32_t* __restrict__ positions,
+                                      const float2* __restrict__ table,
+                                      A* __restrict__ kv, const int32_t* __restrict__ write_slot) {
+  const int64_t t = blockIdx.x;
+  const int half = d / 2;
+  A* row = qkv + t * static_cast<int64_t>((hq + 2 * hkv) * d);
+  const int pos = positions[t];
+  int64_t page = 0;
+  int off = 0;
+  if (kv != nullptr) {
+    const int slot = write_slot[t];
+    page = slot / kPage;
+    off = slot % kPage;
+  }
+  const int64_t page_elems = 2LL * hkv * kPage * d;
+  A* kpage = kv != nullptr ? kv + page * page_elems : nullptr;
+  A* vpage = kv != nullptr ? kpage + static_cast<int64_t>(hkv) * kPage * d : nullptr;
+
+  const int n_rot = (hq + hkv) * half;
+  for (int idx = threadIdx.x; idx < n_rot; idx += blockDim.x) {
+    const int h = idx / half, i = idx - h * half;
+    A* x = row + h * d;
+    float a = to_float<A>(x[i]), b = to_float<A>(x[i + half]);
+    if (table != nullptr) {
+      const float2 cs = table[static_cast<int64_t>(pos) * half + i];
+      const float ra = a * cs.x - b * cs.y;
+      const float rb = b * cs.x + a * cs.y;
+      a = ra;
+      b = rb;
+      x[i] = from_float<A>(a);
+      x[i + half] = from_float<A>(b);
+    }
+    if (kpage != nullptr && h >= hq) {
+      A* dst = kpage + (static_cast<int64_t>(h - hq) * kPage + off) * d;
+      dst[i] = from_float<A>(a);
+      dst[i + half] = from_float<A>(b);
+    }
+  }
+  if (vpage != nullptr) {
+    const A* v = row + (hq + hkv) * d;
+    for (int idx = threadIdx.x; idx < hkv * d; idx += blockDim.x) {
+      const int h = idx / d, c = idx - h * d;
+      vpage[(static_cast<int64_t>(h) * d + c) * kPage + off] = v[idx];
+    }
+  }
+}
+
+}  // namespace psamd
+
+using namespace psamd;
+
+extern "C" {
+
+const char* psamd_last_error(void) { return g_error.c_str(); }
+
+int psamd_embed(void* stream, const int32_t* ids, const void* table, int table_dtype, float* out, int64_t tokens,
+                int hidden) {
+  PSAMD_REQUIRE(tokens >= 0 && hidden > 0, "bad sizes");
+  if (tokens == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (table_dtype == kBF16) {
+    embed_kernel<bf16_t><<<dim3(tokens), dim3(256), 0, s>>>(ids, static_cast<const bf16_t*>(table), out, hidden);
+  } else if (table_dtype == kF32) {
+    embed_kernel<float><<<dim3(tokens), dim3(256), 0, s>>>(ids, static_cast<const float*>(table), out, hidden);
+  } else {
+    return fail("psamd_embed: table dtype must be float32 or bfloat16");
+  }
+  return check_launch("psamd_embed");
+}
+
+int psamd_add_rmsnorm(void* stream, float* residual, const void* delta, const int32_t* rows, const void* weight,
+                      int weight_dtype, float eps, void* out, int act_dtype, int64_t out_rows, int hidden) {
+  PSAMD_REQUIRE(out_rows >= 0 && hidden > 0, "bad sizes");
+  PSAMD_REQUIRE(weight_dtype == kF32 || weight_dtype == kBF16, "weight dtype must be float32 or bfloat16");
+  if (out_rows == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  constexpr int kThreads = 256;
+  if (act_dtype == kBF16) {
+    add_rmsnorm_kernel<bf16_t, kThreads><<<dim3(out_rows), dim3(kThreads), 0, s>>>(
+        residual, static_cast<const bf16_t*>(delta), rows, weight, weight_dtype, eps, static_cast<bf16_t*>(out), hidden);
+  } else if (act_dtype == kF32) {
+    add_rmsnorm_kernel<float, kThreads><<<dim3(out_rows), dim3(kThreads), 0, s>>>(
+        residual, static_cast<const float*>(delta), rows, weight, weight_dtype, eps, static_cast<float*>(out), hidden);
+  } else {
+    return fail("psamd_add_rmsnorm: activation dtype must be float32 or bfloat16");
+  }
+  return check_launch("psamd_add_rmsnorm");
+}
+
+int psamd_swiglu(void* stream, const void* gate_up, void* out, int act_dtype, int64_t tokens, int inter) {
+  PSAMD_REQUIRE(tokens >= 0 && inter > 0, "bad sizes");
+  if (tokens == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int64_t n = tokens * inter;
+  const int blocks = static_cast<int>(std::min<int64_t>(ceil_div(n, 256), 65536));
+  if (act_dtype == kBF16) {
+    swiglu_kernel<bf16_t><<<dim3(blocks), dim3(256), 0, s>>>(static_cast<const bf16_t*>(gate_up),
+                                                            static_cast<bf16_t*>(out), tokens, inter);
+  } else if (act_dtype == kF32) {
+    swiglu_kernel<float><<<dim3(blocks), dim3(256), 0, s>>>(static_cast<const float*>(gate_up),
+                                                           static_cast<float*>(out), tokens, inter);
+  } else {
+    return fail("psamd_swiglu: activation dtype must be float32 or bfloat16");
+  }
+  return check_launch("psamd_swiglu");
+}
+
+int psamd_rope_kv_append(void* stream, void* qkv, int act_dtype, int64_t tokens, int hq, int hkv, int head_dim,
+                         const int32_t* positions, const float* table, void* kv, const int32_t* write_slot) {
+  PSAMD_REQUIRE(tokens >= 0 && hq > 0 && hkv > 0, "bad sizes");
+  PSAMD_REQUIRE(head_dim > 0 && head_dim % 2 == 0, "head_dim must be even");
+  PSAMD_REQUIRE(kv == nullptr || write_slot != nullptr, "a cache needs write slots");
+  if (tokens == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const float2* tab = reinterpret_cast<const float2*>(table);
+  if (act_dtype == kBF16) {
+    rope_kv_append_kernel<bf16_t><<<dim3(tokens), dim3(256), 0, s>>>(static_cast<bf16_t*>(qkv), hq, hkv, head_dim,
+                                                                    positions, tab, static_cast<bf16_t*>(kv), write_slot);
+  } else if (act_dtype == kF32) {
+    rope_kv_append_kernel<float><<<dim3(tokens), dim3(256), 0, s>>>(static_cast<float*>(qkv), hq, hkv, head_dim,
+                                                                   positions, tab, static_cast<float*>(kv), write_slot);
+  } else {
+    return fail("psamd_rope_kv_append: activation dtype must be float32 or bfloat16");
+  }
+  return check_launch("psamd_rope_kv_append");
+}
+
+}  // extern "C"

@@ -1,0 +1,235 @@
+"""Python face of the kernel library: checks shapes on the host, then launches the
+hand-written HIP kernels on torch's current stream with raw pointers.
+
+There is no other implementation behind these calls: without a GPU or without the
+compiled library, constructing ``HipOps`` raises. The only library routine on the path is
+the matrix product ``torch.matmul`` (hipBLASLt) for bfloat16 products with more than 64
+rows, where the reference's engine also calls a library (prefixserve/model/llama.py:113-126);
+every 32-bit product and every product with at most 64 rows is a kernel of this package.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Any
+
+import torch
+
+from prefixserve_amd.build import ensure_kernels
+
+_F32, _BF16 = 0, 1
+_vp, _i32, _i64, _f32 = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_float
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _code(dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return _F32
+    if dtype == torch.bfloat16:
+        return _BF16
+    raise KernelError(f"kernels take float32 or bfloat16, got {dtype}")
+
+
+def _ptr(t: torch.Tensor | None) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+_SIGNATURES = {
+    "psamd_embed": [_vp, _vp, _vp, _i32, _vp, _i64, _i32],
+    "psamd_add_rmsnorm": [_vp, _vp, _vp, _vp, _vp, _i32, _f32, _vp, _i32, _i64, _i32],
+    "psamd_swiglu": [_vp, _vp, _vp, _i32, _i64, _i32],
+    "psamd_rope_kv_append": [_vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp, _vp, _vp, _vp],
+    "psamd_linear": [_vp, _vp, _i32, _vp, _i32, _vp, _i32, _i64, _i32, _i32],
+    "psamd_linear_skinny": [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32],
+    "psamd_attention_generic": [_vp, _vp, _i32, _vp, _vp, _i32, _i64, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _f32, _i32],
+    "psamd_attention_mfma_supports": [_i32, _i32, _i32],
+    "psamd_attention_prefill": [_vp, _vp, _i32, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _f32, _i32],
+    "psamd_attention_decode": [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32,
+                               _i32, _f32, _i32],
+    "psamd_sample": [_vp, _vp, _vp, _vp, _vp, _i32, _i32],
+}
+
+
+class HipOps:
+    PREFILL_TILE_Q = 128   # queries per workgroup of the prefill attention kernel (4 waves x 32)
+    SKINNY_MAX_ROWS = 64
+    name = "hip"
+
+    def __init__(self, device: torch.device | str, workspace: Any = None) -> None:
+        self.device = torch.device(device)
+        if self.device.type != "cuda" or not torch.cuda.is_available():
+            raise KernelError("prefixserve_amd runs on a GPU only: no device kernels can run on "
+                              f"{self.device} and there is no CPU implementation to fall back to")
+        self.lib = ensure_kernels()
+        for name, argtypes in _SIGNATURES.items():
+            fn = getattr(self.lib, name)
+            fn.argtypes = argtypes
+            fn.restype = ctypes.c_int
+        self.lib.psamd_last_error.restype = ctypes.c_char_p
+        self.ws = workspace
+        self.decode_split_kv_len: int | None = None   # fixed key length to size splits by (graph capture)
+
+    # ---------------------------------------------------------------- helpers
+
+    def _stream(self) -> int:
+        return torch.cuda.current_stream(self.device).cuda_stream
+
+    def _ok(self, rc: int) -> None:
+        if rc != 0:
+            raise KernelError(self.lib.psamd_last_error().decode())
+
+    @staticmethod
+    def _need(cond: bool, msg: str) -> None:
+        if not cond:
+            raise KernelError(msg)
+
+    def prepare_matrix(self, w: torch.Tensor, rt: Any) -> torch.Tensor:
+        """A weight matrix on the device in the activation dtype (bfloat16 values widen to
+        float32 exactly on the 32-bit path)."""
+        return w.to(device=rt.device, dtype=rt.dtype).contiguous()
+
+    # ------------------------------------------------------------ elementwise
+
+    def embed(self, ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> None:
+        t, h = out.shape
+        self._need(ids.dtype == torch.int32 and ids.numel() == t, "embed: ids must be int32 [T]")
+        self._need(table.shape[1] == h and out.dtype == torch.float32 and out.is_contiguous(), "embed: bad output")
+        self._ok(self.lib.psamd_embed(self._stream(), ids.data_ptr(), table.data_ptr(), _code(table.dtype),
+                                      out.data_ptr(), t, h))
+
+    def add_rmsnorm(self, residual, delta, weight, eps: float, out) -> None:
+        t, h = residual.shape
+        self._need(residual.dtype == torch.float32 and residual.is_contiguous(), "add_rmsnorm: residual must be float32")
+        self._need(out.shape == (t, h) and out.is_contiguous(), "add_rmsnorm: bad output shape")
+        self._need(delta is None or (delta.shape == (t, h) and delta.dtype == out.dtype and delta.is_contiguous()),
+                   "add_rmsnorm: delta must match the output")
+        self._need(weight.numel() == h, "add_rmsnorm: weight size")
+        self._ok(self.lib.psamd_add_rmsnorm(self._stream(), residual.data_ptr(), _ptr(delta), None, weight.data_ptr(),
+                                            _code(weight.dtype), eps, out.data_ptr(), _code(out.dtype), t, h))
+
+    def add_rmsnorm_rows(self, residual, delta, rows, weight, eps: float, out) -> None:
+        t, h = residual.shape
+        s = rows.numel()
+        self._need(residual.dtype == torch.float32 and rows.dtype == torch.int32, "add_rmsnorm_rows: dtypes")
+        self._need(out.shape == (s, h) and out.is_contiguous(), "add_rmsnorm_rows: bad output shape")
+        self._need(delta is None or (delta.shape == (t, h) and delta.dtype == out.dtype), "add_rmsnorm_rows: delta")
+        self._ok(self.lib.psamd_add_rmsnorm(self._stream(), residual.data_ptr(), _ptr(delta), rows.data_ptr(),
+                                            weight.data_ptr(), _code(weight.dtype), eps, out.data_ptr(),
+                                            _code(out.dtype), s, h))
+
+    def swiglu(self, gate_up, out) -> None:
+        t, inter = out.shape
+        self._need(gate_up.shape == (t, 2 * inter) and gate_up.dtype == out.dtype, "swiglu: shapes")
+        self._ok(self.lib.psamd_swiglu(self._stream(), gate_up.data_ptr(), out.data_ptr(), _code(out.dtype), t, inter))
+
+    def rope_kv_append(self, qkv, hq: int, hkv: int, d: int, positions, table, kv, write_slot) -> None:
+        t = qkv.shape[0]
+        self._need(qkv.shape[1] == (hq + 2 * hkv) * d and qkv.is_contiguous(), "rope_kv_append: qkv shape")
+        self._need(positions.dtype == torch.int32 and positions.numel() == t, "rope_kv_append: positions")
+        if table is not None:
+            self._need(table.dtype == torch.float32 and table.shape[1:] == (d // 2, 2) and table.is_contiguous(),
+                       "rope_kv_append: table must be float32 [positions, D/2, 2]")
+        if kv is not None:
+            self._need(kv.dtype == qkv.dtype and kv.shape[1:] == (2, hkv, 16 * d) and kv.is_contiguous(),
+                       "rope_kv_append: cache must be [blocks, 2, kv_heads, 16*D] in the activation dtype")
+            self._need(write_slot.dtype == torch.int32 and write_slot.numel() == t, "rope_kv_append: write slots")
+        self._ok(self.lib.psamd_rope_kv_append(self._stream(), qkv.data_ptr(), _code(qkv.dtype), t, hq, hkv, d,
+                                               positions.data_ptr(), _ptr(table), _ptr(kv),
+                                               None if kv is None else write_slot.data_ptr()))
+
+    # ---------------------------------------------------------------- products
+
+    def linear(self, x, w, out) -> None:
+        m, k = x.shape
+        n = w.shape[0]
+        self._need(w.shape[1] == k and out.shape == (m, n), f"linear: shapes {tuple(x.shape)} x {tuple(w.shape)}")
+        self._need(x.is_contiguous() and w.is_contiguous() and out.is_contiguous(), "linear: contiguous operands")
+        self._need(x.dtype == w.dtype, "linear: x and w must have one dtype")
+        if m == 0:
+            return
+        if x.dtype == torch.bfloat16 and k % 8 == 0:
+            if m <= self.SKINNY_MAX_ROWS or out.dtype == torch.float32:
+                # Logits (float32 output) always come from this kernel, whatever the row
+                # count, so that a position's logits do not depend on how the step was cut.
+                for r0 in range(0, m, self.SKINNY_MAX_ROWS):
+                    r1 = min(m, r0 + self.SKINNY_MAX_ROWS)
+                    self._ok(self.lib.psamd_linear_skinny(self._stream(), x[r0:r1].data_ptr(), w.data_ptr(),
+                                                          out[r0:r1].data_ptr(), _code(out.dtype), r1 - r0, n, k, 0))
+                return
+            if out.dtype == torch.bfloat16:
+                torch.matmul(x, w.t(), out=out)   # library product, as in the reference
+                return
+        self._ok(self.lib.psamd_linear(self._stream(), x.data_ptr(), _code(x.dtype), w.data_ptr(), _code(w.dtype),
+                                       out.data_ptr(), _code(out.dtype), m, n, k))
+
+    def linear_swiglu(self, x, w_gate_up, out) -> None:
+        m, k = x.shape
+        inter = out.shape[1]
+        self._need(w_gate_up.shape == (2 * inter, k) and out.shape[0] == m, "linear_swiglu: shapes")
+        if m == 0:
+            return
+        if x.dtype == torch.bfloat16 and k % 8 == 0 and m <= self.SKINNY_MAX_ROWS:
+            self._ok(self.lib.psamd_linear_skinny(self._stream(), x.data_ptr(), w_gate_up.data_ptr(), out.data_ptr(),
+                                                  _BF16, m, inter, k, 1))
+            return
+        gu = self.ws.get("mlp.gate_up", (m, 2 * inter), x.dtype)
+        self.linear(x, w_gate_up, gu)
+        self.swiglu(gu, out)
+
+    # --------------------------------------------------------------- attention
+
+    def mfma_attention_supported(self, hq: int, hkv: int, d: int) -> bool:
+        return bool(self.lib.psamd_attention_mfma_supports(hq, hkv, d))
+
+    def paged_attention(self, qkv, out, kv, ctx, group: int, hq: int, hkv: int, d: int, scale: float,
+                        window: int | None) -> None:
+        t = qkv.shape[0]
+        g = ctx.groups[group]
+        self._need(out.shape == (t, hq * d) and out.is_contiguous() and out.dtype == qkv.dtype, "attention: output")
+        self._need(kv.dtype == qkv.dtype and kv.shape[1:] == (2, hkv, 16 * d) and kv.is_contiguous(),
+                   "attention: cache must be [blocks, 2, kv_heads, 16*D] in the activation dtype")
+        self._need(t == ctx.num_tokens, "attention: token count differs from the step batch")
+        win = int(window) if window is not None else 0
+        stride = qkv.shape[1]
+        s = self._stream()
+        if qkv.dtype == torch.bfloat16 and stride % 8 == 0 and self.mfma_attention_supported(hq, hkv, d):
+            if ctx.num_prefill_tiles:
+                self._ok(self.lib.psamd_attention_prefill(
+                    s, qkv.data_ptr(), stride, out.data_ptr(), kv.data_ptr(), ctx.pf_tiles.data_ptr(),
+                    ctx.num_prefill_tiles, ctx.item_start.data_ptr(), ctx.item_pos0.data_ptr(),
+                    g.table_off.data_ptr(), g.block_ids.data_ptr(), hq, hkv, d, scale, win))
+            if ctx.num_decode:
+                kv_len = self.decode_split_kv_len or ctx.max_kv_len
+                if win:
+                    kv_len = min(kv_len, win)
+                nsplit = max(1, min(64, 1024 // (ctx.num_decode * hkv), -(-kv_len // 128)))
+                part_o = self.ws.get("attn.part_o", (ctx.num_decode * hq * nsplit * d,), torch.float32)
+                part_ml = self.ws.get("attn.part_ml", (ctx.num_decode * hq * nsplit * 2,), torch.float32)
+                self._ok(self.lib.psamd_attention_decode(
+                    s, qkv.data_ptr(), stride, out.data_ptr(), kv.data_ptr(), part_o.data_ptr(), part_ml.data_ptr(),
+                    ctx.dec_items.data_ptr(), ctx.num_decode, ctx.item_start.data_ptr(), ctx.item_end.data_ptr(),
+                    g.table_off.data_ptr(), g.block_ids.data_ptr(), hq, hkv, d, nsplit, scale, win))
+            return
+        self._ok(self.lib.psamd_attention_generic(
+            s, qkv.data_ptr(), stride, out.data_ptr(), kv.data_ptr(), _code(qkv.dtype), t, ctx.positions.data_ptr(),
+            ctx.tok_item.data_ptr(), g.table_off.data_ptr(), g.block_ids.data_ptr(), hq, hkv, d, scale, win))
+
+    # ---------------------------------------------------------------- sampling
+
+    def sample(self, logits, temperatures, uniforms, out) -> None:
+        rows, vocab = logits.shape
+        self._need(logits.dtype == torch.float32 and logits.is_contiguous(), "sample: logits must be float32")
+        self._need(temperatures.dtype == torch.float32 and uniforms.dtype == torch.float32 and
+                   temperatures.numel() == rows and uniforms.numel() == rows, "sample: one temperature and uniform per row")
+        self._need(out.dtype == torch.int32 and out.numel() == rows, "sample: output must be int32 [rows]")
+        self._ok(self.lib.psamd_sample(self._stream(), logits.data_ptr(), temperatures.data_ptr(), uniforms.data_ptr(),
+                                       out.data_ptr(), rows, vocab))
+
+    def argmax(self, logits, out) -> None:
+        rows = logits.shape[0]
+        zeros = self.ws.get("sample.zeros", (rows,), torch.float32)
+        zeros.zero_()
+        self.sample(logits, zeros, zeros, out)
