@@ -1,0 +1,101 @@
+"""The engine a driver loop talks to: runs a scheduler batch on the GPU and returns the
+sampled tokens (prefixserve/llama_engine.py:39-150 and prefixserve/engine.py:10-29 of the
+reference define the same surface: ``EngineConfig``, ``step(batch)``, ``num_blocks``,
+``max_seq_len``, ``stop_token_ids``, ``capture_logits``/``last_logits``).
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from pathlib import Path
+from typing import Any
+
+import torch
+
+from prefixserve_amd.cache.manager import CacheManager
+from prefixserve_amd.engine.batch import EngineError, StepItem
+from prefixserve_amd.engine.runner import ModelRunner
+from prefixserve_amd.engine.scheduler import Batch, Scheduler
+from prefixserve_amd.sampling.sampler import Sampler, request_key, uniform_for
+
+
+@dataclass(frozen=True)
+class EngineConfig:
+    model_path: Path | str
+    dtype: str = "bfloat16"              # "bfloat16" (serving) or "float32" (exact)
+    device: str = "cuda:0"
+    # Must match the scheduler's limits: they size buffers and the slot pool.
+    max_num_seqs: int = 64
+    max_prefill_tokens: int = 512
+    max_seq_len: int = 8192
+    num_blocks: int | None = None        # None = sized from free GPU memory
+    reserve_bytes: int = 1 << 30
+    use_graphs: bool = True              # replay decode-only steps as captured HIP graphs
+    sample_seed: int = 0
+
+
+class Engine:
+    def __init__(self, cfg: EngineConfig, ops: Any = None) -> None:
+        self.cfg = cfg
+        self.runner = ModelRunner(
+            cfg.model_path, dtype=cfg.dtype, device=cfg.device, num_blocks=cfg.num_blocks,
+            max_seq_len=cfg.max_seq_len, max_num_seqs=cfg.max_num_seqs, max_prefill_tokens=cfg.max_prefill_tokens,
+            reserve_bytes=cfg.reserve_bytes, use_graphs=cfg.use_graphs, ops=ops)
+        self.sampler = Sampler(self.runner.ops, self.runner.device, max(cfg.max_num_seqs, 1))
+        self.capture_logits = False
+        self.last_logits: dict[str, torch.Tensor] = {}
+
+    @property
+    def num_blocks(self) -> int:
+        return self.runner.num_blocks
+
+    @property
+    def max_seq_len(self) -> int:
+        return self.cfg.max_seq_len
+
+    @property
+    def stop_token_ids(self) -> frozenset[int]:
+        return self.runner.stop_token_ids
+
+    def make_cache(self, enable_prefix_cache: bool = True) -> CacheManager:
+        """The host-side manager of exactly this engine's pools and slots."""
+        r = self.runner
+        return CacheManager(r.num_blocks_per_group, r.windows, r.max_num_seqs, r.state_bytes_per_slot,
+                            enable_prefix_cache=enable_prefix_cache)
+
+    def make_scheduler(self, *, max_waiting: int = 1024, chunk_size: int | None = None,
+                       enable_prefix_cache: bool = True) -> Scheduler:
+        return Scheduler(cache=self.make_cache(enable_prefix_cache), max_waiting=max_waiting,
+                         chunk_size=chunk_size if chunk_size is not None else self.cfg.max_prefill_tokens,
+                         stop_token_ids=self.stop_token_ids)
+
+    def step(self, batch: Batch) -> dict[str, int]:
+        """Runs one batch; returns req_id -> next token for the items that sample."""
+        if not batch.work:
+            return {}
+        if len(batch.work) > self.cfg.max_num_seqs:
+            raise EngineError(f"batch of {len(batch.work)} requests is over max_num_seqs {self.cfg.max_num_seqs}")
+        items, sampling = [], []
+        for w in batch.work:
+            req, n = w.req, w.end - w.start
+            if w.end > self.cfg.max_seq_len:
+                raise EngineError(f"{req.req_id}: position {w.end} > max_seq_len {self.cfg.max_seq_len}")
+            items.append(StepItem(key=req.req_id, tokens=req.tokens(w.start, w.end), start=w.start,
+                                  block_tables=req.block_tables, slot=max(req.slot, 0),
+                                  want=[n - 1] if w.samples else []))
+            if w.samples:
+                sampling.append(req)
+        logits = self.runner.step(items)
+        if not sampling:
+            return {}             # a portion in the middle of a prompt: nothing to wait for
+        assert logits is not None
+        if self.capture_logits:
+            self.last_logits = {r.req_id: logits[i].to("cpu", copy=True) for i, r in enumerate(sampling)}
+        temps = [r.temperature for r in sampling]
+        seeds = [uniform_for(self.cfg.sample_seed ^ r.seed, request_key(r.req_id), len(r.output)) if r.temperature > 0
+                 else 0.0 for r in sampling]
+        tokens = self.sampler.sample(logits, temps, seeds)
+        return {r.req_id: t for r, t in zip(sampling, tokens)}
+
+
+LlamaEngine = Engine   # the reference's name for its engine

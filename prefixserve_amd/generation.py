@@ -1,0 +1,60 @@
+"""Python entry point: run prompts to completion through the scheduler and the engine.
+
+The loop is the reference's driver loop (README.md:321-336, prefixserve/server.py:209-243):
+``add_request`` ... ``while has_work(): batch = schedule_step(); sampled = engine.step(batch);
+commit(batch, sampled)``.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Iterable, Sequence
+
+from prefixserve_amd.engine.engine import Engine
+from prefixserve_amd.engine.scheduler import AddResult, FinishReason, Scheduler, SchedulerStats
+
+
+@dataclass
+class Generation:
+    req_id: str
+    prompt: list[int]
+    tokens: list[int] = field(default_factory=list)
+    finish_reason: FinishReason | None = None
+    cached_tokens: int = 0
+    preemptions: int = 0
+
+
+def generate(engine: Engine, prompts: Sequence[Iterable[int]], max_tokens: int, *, temperature: float = 0.0,
+             seed: int = 0, ignore_eos: bool = False, scheduler: Scheduler | None = None,
+             max_prefill_tokens: int | None = None, max_running_requests: int | None = None,
+             enable_prefix_cache: bool = True) -> tuple[list[Generation], SchedulerStats]:
+    """Generates up to ``max_tokens`` tokens for every prompt (token ids in, token ids out)."""
+    budget = max_prefill_tokens if max_prefill_tokens is not None else engine.cfg.max_prefill_tokens
+    running = max_running_requests if max_running_requests is not None else engine.cfg.max_num_seqs
+    sched = scheduler if scheduler is not None else engine.make_scheduler(
+        chunk_size=budget, enable_prefix_cache=enable_prefix_cache)
+    results: dict[str, Generation] = {}
+    for i, p in enumerate(prompts):
+        rid = f"req-{i}"
+        ids = [int(t) for t in p]
+        if len(ids) + max_tokens > engine.max_seq_len:
+            raise ValueError(f"{rid}: {len(ids)} prompt + {max_tokens} new tokens exceed max_seq_len {engine.max_seq_len}")
+        res = sched.add_request(rid, ids, max_tokens, ignore_eos=ignore_eos, temperature=temperature, seed=seed)
+        if res is not AddResult.ACCEPTED:
+            raise ValueError(f"{rid} rejected: {res.value}")
+        results[rid] = Generation(rid, ids)
+    while sched.has_work():
+        batch = sched.schedule_step(budget, running)
+        if not batch.work:
+            raise RuntimeError("the scheduler has work but could schedule none of it (pool too small?)")
+        tracked = {w.req.req_id: w.req for w in batch.work}
+        sampled = engine.step(batch)
+        step = sched.commit(batch, sampled)
+        for rid, tok in step.new_tokens.items():
+            results[rid].tokens.append(tok)
+        for rid, why in step.finished.items():
+            g, r = results[rid], tracked.get(rid)
+            g.finish_reason = why
+            if r is not None:
+                g.cached_tokens, g.preemptions = r.cached_tokens, r.num_preemptions
+    return [results[f"req-{i}"] for i in range(len(prompts))], sched.stats()

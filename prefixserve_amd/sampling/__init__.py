@@ -1,0 +1,3 @@
+from .sampler import Sampler, request_key, uniform_for
+
+__all__ = ["Sampler", "request_key", "uniform_for"]

@@ -1,0 +1,69 @@
+"""Greedy and temperature sampling.
+
+The reference samples greedily only (prefixserve/llama_engine.py:146; its server refuses a
+temperature, prefixserve/server.py:427-428). Here a request may carry a temperature:
+p = softmax(logits / T) in float32 and a draw by inverse CDF in vocabulary order. The
+uniform number is a function of (seed, request, index of the output token) alone, never of
+the step or the batch slot, so a request that was preempted and recomputed, or batched
+differently, draws the same tokens. Temperature 0 is greedy with the lowest index winning
+ties. The draw itself runs in a device kernel over the step's logits.
+"""
+
+from __future__ import annotations
+
+import zlib
+from typing import Any, Sequence
+
+import torch
+
+_M64 = (1 << 64) - 1
+
+
+def _mix64(z: int) -> int:
+    z = (z + 0x9E3779B97F4A7C15) & _M64
+    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & _M64
+    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & _M64
+    return z ^ (z >> 31)
+
+
+def request_key(req_id: str) -> int:
+    """A stable 64-bit key of a request id (Python's own hash() differs between runs)."""
+    data = req_id.encode()
+    return (zlib.crc32(data) << 32) | zlib.adler32(data)
+
+
+def uniform_for(seed: int, key: int, output_index: int) -> float:
+    """u in [0, 1) with 24 random bits: a chain of splitmix64 finalizers over the three inputs."""
+    z = _mix64(seed & _M64)
+    z = _mix64(z ^ (key & _M64))
+    z = _mix64(z ^ (output_index & _M64))
+    return (z >> 40) / float(1 << 24)
+
+
+class Sampler:
+    """Draws one token per logits row on the device and brings the ids to the host in one copy."""
+
+    def __init__(self, ops: Any, device: torch.device, max_rows: int = 1024) -> None:
+        self.ops = ops
+        self.device = torch.device(device)
+        self._alloc(max_rows)
+
+    def _alloc(self, rows: int) -> None:
+        pin = self.device.type == "cuda"
+        self._host = torch.empty((2, rows), dtype=torch.float32, pin_memory=pin)
+        self._dev = torch.empty((2, rows), dtype=torch.float32, device=self.device)
+        self._out = torch.empty(rows, dtype=torch.int32, device=self.device)
+        self.max_rows = rows
+
+    def sample(self, logits: torch.Tensor, temperatures: Sequence[float], uniforms: Sequence[float]) -> list[int]:
+        rows = logits.shape[0]
+        if len(temperatures) != rows or len(uniforms) != rows:
+            raise ValueError("one temperature and one uniform number per logits row")
+        if rows > self.max_rows:
+            self._alloc(max(rows, 2 * self.max_rows))
+        self._host[0, :rows] = torch.tensor(temperatures, dtype=torch.float32)
+        self._host[1, :rows] = torch.tensor(uniforms, dtype=torch.float32)
+        self._dev[:, :rows].copy_(self._host[:, :rows], non_blocking=True)
+        out = self._out[:rows]
+        self.ops.sample(logits, self._dev[0, :rows], self._dev[1, :rows], out)
+        return out.tolist()   # the step's one device-to-host wait

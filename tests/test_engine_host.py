@@ -1,0 +1,158 @@
+"""Everything on the host side of a step, without a GPU: the kernel library is replaced by
+its torch stand-in (tests/emulated_ops.py), the rest is the product's own code. Compared
+with the plain implementation in every way of cutting the work."""
+
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+import traces
+from configs import TINY, TOL_F32
+from emulated_ops import EmulatedOps
+from prefixserve_amd.engine.batch import EngineError, GroupMeta, StepItem, StepPacker
+from prefixserve_amd.engine.engine import Engine, EngineConfig
+from prefixserve_amd.engine.replay import TraceReplayer
+from prefixserve_amd.engine.runner import ModelRunner
+from prefixserve_amd.generation import generate
+from prefixserve_amd.sampling import request_key, uniform_for
+
+
+def make_runner(model_dir, num_blocks=64, max_seq_len=512, **kw):
+    return ModelRunner(model_dir, dtype="float32", device="cpu", num_blocks=num_blocks, max_seq_len=max_seq_len,
+                       max_num_seqs=8, ops=EmulatedOps(), use_graphs=False, **kw)
+
+
+def requests_for(name, lengths, seed=0):
+    rng = np.random.default_rng(seed)
+    return [rng.integers(0, TINY[name]["vocab_size"], n).tolist() for n in lengths]
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_replay_in_every_cutting(name, model_dirs, plain_models):
+    reqs = requests_for(name, [70, 33, 5, 97, 64, 18])
+    truth = [plain_models[name].logits(t) for t in reqs]
+    runner = make_runner(model_dirs[name])
+    for build in (traces.whole, traces.decode_tail, traces.portions):
+        steps, expect = build(reqs)
+        traces.compare(TraceReplayer(runner).run_step, steps, expect, truth, TOL_F32)
+    reqs = requests_for(name, [70, 33, 120, 97, 64, 18, 130, 45, 101, 77, 128, 90], seed=1)
+    truth = [plain_models[name].logits(t) for t in reqs]
+    steps, expect, peak = traces.mixed(reqs, seed=3)
+    assert sum(len(r) for r in reqs) > 1.5 * peak                 # pages must be used again
+    small = make_runner(model_dirs[name], num_blocks=peak // 16)
+    small.pools.tensors[0].fill_(1e30)                            # stale pages hold junk, never zeros
+    rp = TraceReplayer(small)
+    traces.compare(rp.run_step, steps, expect, truth, TOL_F32)
+    assert rp.cache.num_free(0) == peak // 16 and not rp.live
+
+
+def test_replay_errors(model_dirs):
+    rp = TraceReplayer(make_runner(model_dirs["A"], num_blocks=2))
+    with pytest.raises(EngineError, match="out of pages"):
+        rp.run_step({"step": 0, "entries": [{"id": "a", "tokens": list(range(40)), "want": []}], "end": []})
+    with pytest.raises(EngineError, match="unknown request"):
+        rp.run_step({"step": 1, "entries": [], "end": ["zz"]})
+    with pytest.raises(EngineError, match="twice"):
+        rp.run_step({"step": 2, "entries": [{"id": "b", "tokens": [1], "want": []}, {"id": "b", "tokens": [2], "want": []}], "end": []})
+
+
+def test_packer_refuses_bad_batches():
+    pk = StepPacker(torch.device("cpu"), [GroupMeta(8)], vocab_size=100, max_position=64, num_slots=2, prefill_tile=128)
+    good = dict(key="a", tokens=[1, 2, 3], start=0, block_tables=[[0]], slot=0, want=[2])
+    pk.pack([StepItem(**good)])
+    for change, needle in [
+        (dict(block_tables=[[8]]), "outside the pool"), (dict(block_tables=[[-1]]), "outside the pool"),
+        (dict(block_tables=[[]]), "blocks in group"), (dict(block_tables=[[0], [0]]), "block tables"),
+        (dict(tokens=[100]), "token id"), (dict(tokens=[]), "no tokens"), (dict(start=62), "positions"),
+        (dict(want=[3]), "wanted place"), (dict(slot=2), "state slot"), (dict(start=-1), "positions"),
+    ]:
+        with pytest.raises(EngineError, match=needle):
+            pk.pack([StepItem(**{**good, **change})])
+    with pytest.raises(EngineError, match="empty"):
+        pk.pack([])
+
+
+def test_packer_layout():
+    pk = StepPacker(torch.device("cpu"), [GroupMeta(32)], vocab_size=200, max_position=256, num_slots=4, prefill_tile=128)
+    items = [StepItem("a", list(range(20)), 30, [[5, 6, 7, 8]], slot=1, want=[19]),
+             StepItem("b", [7], 16, [[9, 3]], slot=2, want=[0]),
+             StepItem("c", list(range(130)), 0, [list(range(10, 19))], slot=0, want=[])]
+    ctx = pk.pack(items)
+    assert (ctx.num_tokens, ctx.num_items, ctx.num_logit_rows, ctx.num_decode, ctx.num_prefill_tiles) == (151, 3, 2, 1, 3)
+    assert ctx.item_start.tolist() == [0, 20, 21, 151] and ctx.item_pos0.tolist() == [30, 16, 0]
+    assert ctx.item_end.tolist() == [50, 17, 130] and ctx.slots.tolist() == [1, 2, 0]
+    assert ctx.positions[:20].tolist() == list(range(30, 50)) and ctx.positions[20].item() == 16   # absolute
+    assert ctx.logit_rows.tolist() == [19, 20] and ctx.dec_items.tolist() == [1]
+    assert ctx.pf_tiles.tolist() == [[0, 0], [2, 0], [2, 128]]
+    g = ctx.groups[0]
+    assert g.table_off.tolist() == [0, 4, 6, 15] and g.block_ids[:6].tolist() == [5, 6, 7, 8, 9, 3]
+    assert g.write_slot[0].item() == 6 * 16 + 14 and g.write_slot[2].item() == 7 * 16 + 0   # pos 30 -> page 1 (id 6)
+    assert g.write_slot[20].item() == 3 * 16 + 0                                             # pos 16 -> second page
+    st = pk.pack(items[:2], static_pages=6)                        # fixed-width tables for captured graphs
+    assert st.groups[0].table_off.tolist() == [0, 6, 12] and st.groups[0].block_ids.numel() == 12
+
+
+def test_uniform_numbers_match_the_plain_ones():
+    from plain.llama_plain import uniform_for as plain_uniform
+
+    for seed, key, idx in [(0, 0, 0), (3, 99, 5), (2 ** 63 + 5, request_key("req-7"), 41)]:
+        assert uniform_for(seed, key, idx) == plain_uniform(seed, key, idx)
+    assert request_key("a") != request_key("b") and request_key("a") == request_key("a")
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_scheduler_driven_greedy_generation_equals_plain(name, model_dirs, plain_models):
+    """Chunked prefill, a shared prefix, eviction and preemption (the pool is small) must not
+    change a single token."""
+    vocab = TINY[name]["vocab_size"]
+    rng = np.random.default_rng(4)
+    shared = rng.integers(3, vocab, 37).tolist()
+    prompts = [shared + rng.integers(3, vocab, n).tolist() for n in (9, 21, 40)] + [rng.integers(3, vocab, 5).tolist()]
+    new = 10
+    eng = Engine(EngineConfig(model_path=model_dirs[name], dtype="float32", device="cpu", max_num_seqs=4,
+                              max_prefill_tokens=24, max_seq_len=256, num_blocks=11, use_graphs=False), ops=EmulatedOps())
+    eng.capture_logits = True
+    outs, stats = generate(eng, prompts, new, ignore_eos=True)
+    for p, o in zip(prompts, outs):
+        want, _ = plain_models[name].greedy(p, new)
+        assert o.tokens == want, f"prompt of {len(p)}: {o.tokens} != {want}"
+    assert stats.preemptions > 0 and stats.cached_prompt_tokens > 0
+    sched_cache = eng.make_cache()
+    assert sched_cache.num_free(0) == 11
+
+
+def test_temperature_sampling_is_reproducible_across_batching(model_dirs):
+    eng = Engine(EngineConfig(model_path=model_dirs["B"], dtype="float32", device="cpu", max_num_seqs=4,
+                              max_prefill_tokens=64, max_seq_len=256, num_blocks=64, use_graphs=False, sample_seed=5),
+                 ops=EmulatedOps())
+    rng = np.random.default_rng(8)
+    prompts = [rng.integers(3, 512, n).tolist() for n in (12, 30, 7)]
+    a, _ = generate(eng, prompts, 8, temperature=0.8, ignore_eos=True)
+    b, _ = generate(eng, prompts, 8, temperature=0.8, ignore_eos=True, max_running_requests=1, max_prefill_tokens=5)
+    assert [o.tokens for o in a] == [o.tokens for o in b]          # same draws whatever the batching
+    c, _ = generate(eng, prompts, 8, temperature=0.8, seed=1, ignore_eos=True)
+    assert [o.tokens for o in a] != [o.tokens for o in c]
+    g, _ = generate(eng, prompts, 8, temperature=0.0, ignore_eos=True)
+    assert [o.tokens for o in g] != [o.tokens for o in a]
+
+
+def test_stop_token_ends_generation(model_dirs, plain_models):
+    prompt = np.random.default_rng(2).integers(3, 256, 20).tolist()
+    want, _ = plain_models["A"].greedy(prompt, 6)
+    eng = Engine(EngineConfig(model_path=model_dirs["A"], dtype="float32", device="cpu", max_num_seqs=2,
+                              max_seq_len=128, num_blocks=16, use_graphs=False), ops=EmulatedOps())
+    sched = eng.make_scheduler()
+    sched._stop = frozenset({want[3]})
+    outs, _ = generate(eng, [prompt], 6, scheduler=sched)
+    stop_at = want.index(want[3])
+    assert outs[0].tokens == want[:stop_at + 1] and outs[0].finish_reason.value == "stop"
+    assert eng.stop_token_ids == {2}                               # from config.json's eos_token_id
+
+
+def test_engine_refuses_without_kernels_on_cpu(model_dirs):
+    from prefixserve_amd.kernels.ops import KernelError
+
+    with pytest.raises(KernelError, match="GPU only"):
+        ModelRunner(model_dirs["A"], dtype="float32", device="cpu", num_blocks=4, max_seq_len=64)

@@ -1,0 +1,320 @@
+"""Each kernel alone against a plain torch float32 reference of the same operation, at sizes
+other than the engine tests' (odd widths, tails that do not fill a tile, many heads)."""
+
+from __future__ import annotations
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from prefixserve_amd.engine.batch import GroupMeta, StepItem, StepPacker
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from prefixserve_amd.kernels.ops import HipOps
+    from prefixserve_amd.parts.base import Workspace
+
+    return HipOps(torch.device(DEV), Workspace(torch.device(DEV)))
+
+
+def rnd(*shape, dtype=torch.float32, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (scale * torch.randn(*shape, generator=g)).to(dtype).to(DEV)
+
+
+def rel(got, want):
+    return float((got.float() - want.float()).abs().max() / want.float().abs().max())
+
+
+# ------------------------------------------------------------------ elementwise
+
+@pytest.mark.parametrize("table_dtype", [torch.float32, torch.bfloat16])
+def test_embed(ops, table_dtype):
+    table = rnd(301, 72, dtype=table_dtype)
+    ids = torch.tensor([0, 300, 5, 5, 17], dtype=torch.int32, device=DEV)
+    out = torch.empty(5, 72, device=DEV)
+    ops.embed(ids, table, out)
+    assert torch.equal(out, table[ids.long()].float())
+
+
+@pytest.mark.parametrize("act", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("wdt", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("hidden", [72, 2048, 1000])
+def test_add_rmsnorm(ops, act, wdt, hidden):
+    t, eps = 7, 1e-5
+    res = rnd(t, hidden, seed=1)
+    delta = rnd(t, hidden, dtype=act, seed=2)
+    w = (1 + 0.1 * rnd(hidden, seed=3)).to(wdt)
+    want_res = res + delta.float()
+    want = w.float() * want_res * torch.rsqrt((want_res ** 2).mean(-1, keepdim=True) + eps)
+    out = torch.empty(t, hidden, dtype=act, device=DEV)
+    r = res.clone()
+    ops.add_rmsnorm(r, delta, w, eps, out)
+    assert torch.equal(r, want_res)                                 # the residual sum is 32-bit
+    assert rel(out, want) < (1e-6 if act == torch.float32 else 5e-3)
+    r2 = res.clone()
+    ops.add_rmsnorm(r2, None, w, eps, out)                          # first layer: nothing to add
+    assert torch.equal(r2, res)
+    rows = torch.tensor([6, 0, 3], dtype=torch.int32, device=DEV)
+    out3 = torch.empty(3, hidden, dtype=act, device=DEV)
+    r3 = res.clone()
+    ops.add_rmsnorm_rows(r3, delta, rows, w, eps, out3)
+    assert torch.equal(r3, res) and rel(out3, want[rows.long()]) < (1e-6 if act == torch.float32 else 5e-3)
+
+
+def test_rmsnorm_zero_row_and_eps(ops):
+    res = torch.zeros(2, 64, device=DEV)
+    res[1] = 1e-4
+    out = torch.empty(2, 64, device=DEV)
+    ops.add_rmsnorm(res, None, torch.ones(64, device=DEV), 1e-6, out)
+    assert torch.all(out[0] == 0) and torch.isfinite(out).all()
+    assert abs(float(out[1, 0]) - 1e-4 / math.sqrt(1e-8 + 1e-6)) < 1e-7
+
+
+@pytest.mark.parametrize("act", [torch.float32, torch.bfloat16])
+def test_swiglu(ops, act):
+    gu = rnd(9, 2 * 344, dtype=act, scale=2.0)
+    out = torch.empty(9, 344, dtype=act, device=DEV)
+    ops.swiglu(gu, out)
+    want = torch.nn.functional.silu(gu[:, :344].float()) * gu[:, 344:].float()
+    assert rel(out, want) < (1e-6 if act == torch.float32 else 5e-3)
+
+
+@pytest.mark.parametrize("act", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("hq,hkv,d", [(6, 3, 48), (5, 5, 16), (16, 2, 128)])
+def test_rope_kv_append(ops, act, hq, hkv, d):
+    from prefixserve_amd.parts.rope import rope_inv_freq
+
+    t, blocks = 11, 6
+    qkv = rnd(t, (hq + 2 * hkv) * d, dtype=act)
+    pos = torch.tensor([0, 1, 2, 15, 16, 17, 40, 41, 70, 5, 33], dtype=torch.int32, device=DEV)
+    inv = rope_inv_freq(d, 10000.0, None)
+    ang = torch.outer(torch.arange(96, dtype=torch.float32), inv).double()
+    table = torch.stack((ang.cos(), ang.sin()), -1).float().to(DEV).contiguous()
+    slots = torch.tensor([p % 16 + 16 * ((p // 16 * 5 + 1) % blocks) for p in pos.tolist()], dtype=torch.int32, device=DEV)
+    kv = torch.full((blocks, 2, hkv, 16 * d), 7.0, dtype=act, device=DEV)
+    src = qkv.clone().float()
+    ops.rope_kv_append(qkv, hq, hkv, d, pos, table, kv, slots)
+    x = src[:, : (hq + hkv) * d].view(t, hq + hkv, d)
+    cs = table[pos.long()]
+    cos, sin = cs[..., 0][:, None], cs[..., 1][:, None]
+    x1, x2 = x[..., : d // 2], x[..., d // 2:]
+    want = torch.cat((x1 * cos - x2 * sin, x2 * cos + x1 * sin), -1)
+    got = qkv[:, : (hq + hkv) * d].view(t, hq + hkv, d)
+    assert rel(got, want) < (1e-6 if act == torch.float32 else 5e-3)
+    assert torch.equal(qkv[:, (hq + hkv) * d:].float(), src[:, (hq + hkv) * d:])            # v untouched
+    kp = kv[:, 0].view(blocks, hkv, 16, d)
+    vp = kv[:, 1].view(blocks, hkv, d, 16)
+    page, off = (slots // 16).long(), (slots % 16).long()
+    assert torch.equal(kp[page, :, off, :], got[:, hq:])            # pages hold exactly what was rotated
+    assert torch.equal(vp[page, :, :, off].float(), src[:, (hq + hkv) * d:].view(t, hkv, d))
+    untouched = torch.ones(blocks, 16, dtype=torch.bool)
+    untouched[page.cpu(), off.cpu()] = False
+    assert torch.all(kp.permute(0, 2, 1, 3)[untouched.to(DEV)] == 7.0)                      # nothing else written
+    q2 = src.clone().to(act)
+    ops.rope_kv_append(q2, hq, hkv, d, pos, None, None, slots)     # no table, no cache: a no-op
+    assert torch.equal(q2.float(), src.to(act).float())
+
+
+# --------------------------------------------------------------------- products
+
+@pytest.mark.parametrize("m,n,k", [(1, 100, 72), (3, 64, 16), (17, 257, 96), (130, 70, 200), (64, 128, 64)])
+def test_linear_float32_is_exact_fp32(ops, m, n, k):
+    x, w = rnd(m, k, seed=1), rnd(n, k, seed=2)
+    out = torch.empty(m, n, device=DEV)
+    ops.linear(x, w, out)
+    want = (x.double() @ w.double().T)
+    assert rel(out, want) < 2e-6                                    # a reduced-precision mode would give ~1e-3
+
+
+@pytest.mark.parametrize("m", [1, 2, 7, 16, 17, 33, 64])
+@pytest.mark.parametrize("n,k", [(48, 64), (1000, 96), (129, 2048), (16, 8), (250, 72)])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+def test_linear_bf16_small_m(ops, m, n, k, out_dtype):
+    x, w = rnd(m, k, dtype=torch.bfloat16, seed=1), rnd(n, k, dtype=torch.bfloat16, seed=2, scale=0.1)
+    out = torch.empty(m, n, dtype=out_dtype, device=DEV)
+    ops.linear(x, w, out)
+    want = x.double() @ w.double().T
+    assert rel(out, want) < (1e-5 if out_dtype == torch.float32 else 5e-3)
+
+
+@pytest.mark.parametrize("m,n,k", [(65, 300, 96), (200, 64, 2048), (3, 50, 70)])
+def test_linear_bf16_other_paths(ops, m, n, k):
+    x, w = rnd(m, k, dtype=torch.bfloat16, seed=1), rnd(n, k, dtype=torch.bfloat16, seed=2, scale=0.1)
+    for out_dtype in (torch.bfloat16, torch.float32):
+        out = torch.empty(m, n, dtype=out_dtype, device=DEV)
+        ops.linear(x, w, out)
+        assert rel(out, x.double() @ w.double().T) < (2e-5 if out_dtype == torch.float32 else 5e-3)
+
+
+@pytest.mark.parametrize("m", [1, 5, 64, 100])
+@pytest.mark.parametrize("act", [torch.float32, torch.bfloat16])
+def test_linear_swiglu(ops, m, act):
+    k, inter = 96, 344
+    x, w = rnd(m, k, dtype=act, seed=1), rnd(2 * inter, k, dtype=act, seed=2, scale=0.2)
+    out = torch.empty(m, inter, dtype=act, device=DEV)
+    ops.linear_swiglu(x, w, out)
+    gu = x.double() @ w.double().T
+    want = torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:]
+    assert rel(out, want) < (2e-6 if act == torch.float32 else 1e-2)
+
+
+# -------------------------------------------------------------------- attention
+
+def paged_case(ops, act, hq, hkv, d, lens_new, lens_old, window=None, seed=0, num_blocks=64, poison=1e30):
+    """Random q/k/v for items with ``old`` cached and ``new`` fresh tokens each, pages from a
+    random permutation; returns (kernel output, reference output)."""
+    rng = np.random.default_rng(seed)
+    perm = rng.permutation(num_blocks).tolist()
+    pk = StepPacker(torch.device(DEV), [GroupMeta(num_blocks, window)], 10, 100000, 8, ops.PREFILL_TILE_Q)
+    kv = torch.full((num_blocks, 2, hkv, 16 * d), poison, dtype=act, device=DEV)
+    items, full = [], []
+    for i, (n, old) in enumerate(zip(lens_new, lens_old)):
+        pages = -(-(n + old) // 16)
+        table = [perm.pop() for _ in range(pages)]
+        k = rnd(n + old, hkv, d, dtype=act, seed=seed * 100 + 2 * i)
+        v = rnd(n + old, hkv, d, dtype=act, seed=seed * 100 + 2 * i + 1)
+        full.append((k, v))
+        kp = kv[:, 0].view(num_blocks, hkv, 16, d)
+        vp = kv[:, 1].view(num_blocks, hkv, d, 16)
+        pos = torch.arange(n + old)
+        pg = torch.tensor(table)[pos // 16].to(DEV)
+        kp[pg, :, (pos % 16).to(DEV), :] = k
+        vp[pg, :, :, (pos % 16).to(DEV)] = v
+        items.append(StepItem(i, [1] * n, old, [table], slot=i % 8))
+    ctx = pk.pack(items)
+    t = sum(lens_new)
+    qkv = rnd(t, (hq + 2 * hkv) * d, dtype=act, seed=seed + 999)
+    out = torch.empty(t, hq * d, dtype=act, device=DEV)
+    scale = 1.0 / math.sqrt(d)
+    ops.paged_attention(qkv, out, kv, ctx, 0, hq, hkv, d, scale, window)
+    want = torch.empty(t, hq, d, dtype=torch.float64, device=DEV)
+    t0 = 0
+    for (k, v), n, old in zip(full, lens_new, lens_old):
+        q = qkv[t0:t0 + n, : hq * d].view(n, hq, d).double()
+        kk = k.double().repeat_interleave(hq // hkv, 1)
+        vv = v.double().repeat_interleave(hq // hkv, 1)
+        s = torch.einsum("nhd,mhd->hnm", q, kk) * scale
+        qpos = torch.arange(old, old + n, device=DEV)[:, None]
+        kpos = torch.arange(old + n, device=DEV)[None, :]
+        hide = kpos > qpos
+        if window is not None:
+            hide = hide | (qpos - kpos >= window)
+        p = torch.softmax(s.masked_fill(hide, float("-inf")), -1)
+        want[t0:t0 + n] = torch.einsum("hnm,mhd->nhd", p, vv)
+        t0 += n
+    return out.view(t, hq, d), want
+
+
+SHAPES = [(4, 2, 16), (3, 1, 32), (8, 2, 64), (32, 8, 64), (6, 6, 96), (8, 1, 128), (40, 2, 64), (2, 2, 256), (6, 3, 48), (2, 1, 80)]
+
+
+@pytest.mark.parametrize("hq,hkv,d", SHAPES)
+@pytest.mark.parametrize("act", [torch.float32, torch.bfloat16])
+def test_paged_attention_mixed_batch(ops, act, hq, hkv, d):
+    """Fresh prompts, portions on top of a cached prefix, decodes with one slot left in the
+    last page and with a last page exactly full: one batch."""
+    new = [37, 1, 130, 1, 2, 16, 1, 1]
+    old = [0, 15, 50, 31, 94, 16, 0, 200]
+    got, want = paged_case(ops, act, hq, hkv, d, new, old, seed=hq + d)
+    assert rel(got, want) < (2e-5 if act == torch.float32 else 2e-2)
+
+
+@pytest.mark.parametrize("act", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window", [1, 16, 33, 100])
+def test_paged_attention_window(ops, act, window):
+    got, want = paged_case(ops, act, 8, 2, 64, [70, 1, 1, 9], [0, 40, 130, 64], window=window, seed=window)
+    assert rel(got, want) < (2e-5 if act == torch.float32 else 2e-2)
+
+
+@pytest.mark.parametrize("act", [torch.float32, torch.bfloat16])
+def test_attention_finds_one_far_key_among_hundreds(ops, act):
+    """One old key is made to match the query strongly; the output must be that key's value,
+    wherever its page lies. A kernel that skips or misplaces a page cannot pass."""
+    hq, hkv, d, n_old = 8, 2, 64, 700
+    for far in (0, 15, 16, 333, 511, 512, 699):
+        rng = np.random.default_rng(far)
+        num_blocks = 64
+        perm = rng.permutation(num_blocks).tolist()
+        table = [perm.pop() for _ in range(-(-(n_old + 1) // 16))]
+        kv = torch.zeros((num_blocks, 2, hkv, 16 * d), dtype=act, device=DEV)
+        k = rnd(n_old + 1, hkv, d, dtype=act, seed=1, scale=0.05)
+        v = rnd(n_old + 1, hkv, d, dtype=act, seed=2)
+        qkv = rnd(1, (hq + 2 * hkv) * d, dtype=act, seed=3, scale=0.05)
+        q = qkv[0, : hq * d].view(hq, d)
+        k[far] = 0
+        for h in range(hkv):
+            k[far, h] = 40.0 * q[h * (hq // hkv)] / q[h * (hq // hkv)].float().norm()     # aligned with the group's first head
+        pos = torch.arange(n_old + 1)
+        pg = torch.tensor(table)[pos // 16].to(DEV)
+        kv[:, 0].view(num_blocks, hkv, 16, d)[pg, :, (pos % 16).to(DEV), :] = k
+        kv[:, 1].view(num_blocks, hkv, d, 16)[pg, :, :, (pos % 16).to(DEV)] = v
+        pk = StepPacker(torch.device(DEV), [GroupMeta(num_blocks)], 10, 4096, 8, ops.PREFILL_TILE_Q)
+        ctx = pk.pack([StepItem("a", [1], n_old, [table])])
+        out = torch.empty(1, hq * d, dtype=act, device=DEV)
+        # a large scale makes the softmax one-hot on the planted key for the aligned heads
+        ops.paged_attention(qkv, out, kv, ctx, 0, hq, hkv, d, 50.0, None)
+        for h in range(hkv):
+            head = h * (hq // hkv)
+            assert rel(out.view(hq, d)[head], v[far, h]) < 2e-2, f"far key at {far}, head {head}"
+
+
+# --------------------------------------------------------------------- sampling
+
+def test_sampling_kernel(ops):
+    from plain.llama_plain import sample_plain
+
+    rows, vocab = 6, 1237
+    logits = rnd(rows, vocab, seed=4, scale=3.0)
+    logits[0, 77] = logits[0, 900] = 50.0                           # a tie: the lowest index wins
+    temps = torch.tensor([0.0, 0.0, 0.8, 0.8, 1.5, 0.3], device=DEV)
+    us = torch.tensor([0.0, 0.5, 0.1234, 0.9999, 0.5, 0.0], device=DEV)
+    out = torch.empty(rows, dtype=torch.int32, device=DEV)
+    ops.sample(logits, temps, us, out)
+    got = out.tolist()
+    assert got[0] == 77 and got[1] == int(torch.argmax(logits[1]))
+    lg = logits.cpu().numpy()
+    for r in range(2, rows):
+        want = sample_plain(lg[r], float(temps[r]), float(us[r]))
+        if got[r] != want:                                          # only a rounding of the CDF edge may differ
+            z = lg[r].astype(np.float64) / float(temps[r])
+            c = np.cumsum(np.exp(z - z.max()))
+            target = float(us[r]) * c[-1]
+            lo, hi = min(got[r], want), max(got[r], want)
+            assert hi - lo == 1 and abs(c[lo] - target) < 1e-5 * c[-1]
+    out2 = torch.empty(rows, dtype=torch.int32, device=DEV)
+    ops.argmax(logits, out2)
+    assert out2.tolist() == [77] + torch.argmax(logits[1:], -1).tolist()
+
+
+def test_sampling_frequencies(ops):
+    logits = torch.tensor([[0.0, 1.0, 2.0, -1.0, 0.5]], device=DEV).repeat(4000, 1).contiguous()
+    g = torch.Generator().manual_seed(0)
+    us = torch.rand(4000, generator=g).to(DEV)
+    temps = torch.full((4000,), 0.7, device=DEV)
+    out = torch.empty(4000, dtype=torch.int32, device=DEV)
+    ops.sample(logits, temps, us, out)
+    freq = torch.bincount(out.long().cpu(), minlength=5).double() / 4000
+    want = torch.softmax(logits[0].double().cpu() / 0.7, 0)
+    assert float((freq - want).abs().max()) < 0.03
+
+
+def test_kernels_refuse_what_they_do_not_take(ops):
+    from prefixserve_amd.kernels.ops import KernelError
+
+    with pytest.raises(KernelError):
+        ops.linear(rnd(2, 8), rnd(4, 9), torch.empty(2, 4, device=DEV))
+    with pytest.raises(KernelError):
+        ops.embed(torch.zeros(2, dtype=torch.int64, device=DEV), rnd(4, 8), torch.empty(2, 8, device=DEV))
+    with pytest.raises(KernelError):
+        ops.add_rmsnorm(rnd(2, 8).to(torch.bfloat16), None, rnd(8), 1e-5, torch.empty(2, 8, device=DEV))
+    x = rnd(2, 8).to(torch.float16)
+    with pytest.raises(KernelError):
+        ops.swiglu(x, torch.empty(2, 4, dtype=torch.float16, device=DEV))

@@ -1,0 +1,224 @@
+"""Each part of a layer alone against the plain implementation's function for it, and the
+openness of the part registries: a toy mixer with state of its own, defined here, is
+registered, built into a model and stepped without touching the package's files."""
+
+from __future__ import annotations
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from plain import llama_plain as P
+from prefixserve_amd.engine.batch import GroupMeta, StepItem, StepPacker
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+
+
+def runtime(dtype):
+    from prefixserve_amd.kernels.ops import HipOps
+    from prefixserve_amd.parts.base import Runtime, Workspace
+
+    ws = Workspace(DEV)
+    return Runtime(DEV, dtype, HipOps(DEV, ws), ws)
+
+
+def rel(got, want):
+    got = got.detach().float().cpu().numpy().astype(np.float64)
+    return float(np.abs(got - want).max() / np.abs(want).max())
+
+
+TOL = {torch.float32: 5e-6, torch.bfloat16: 2e-2}
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rmsnorm_part(dtype):
+    from prefixserve_amd.parts.norm import RMSNorm
+
+    rt = runtime(dtype)
+    part = RMSNorm(hidden_size=200, eps=1e-6, name="w")
+    assert part.weights()["w"].shape == (200,)
+    w = (1 + 0.1 * torch.randn(200)).to(torch.bfloat16)
+    part.bind({"w": w}, rt)
+    res = torch.randn(5, 200, device=DEV)
+    delta = torch.randn(5, 200, device=DEV).to(dtype)
+    want = P.rms_norm((res + delta.float()).cpu().double().numpy(), w.double().numpy(), 1e-6)
+    got = part.add_norm(res, delta, "x")
+    assert rel(got, want) < TOL[dtype]
+
+
+def test_rope_part_table():
+    from prefixserve_amd.parts.rope import RotaryEmbedding
+
+    scaling = dict(factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0, original_max_position_embeddings=64)
+    part = RotaryEmbedding(head_dim=32, theta=500000.0, scaling=scaling)
+    part.bind({}, runtime(torch.float32))
+    part.prepare(300)
+    inv = P.rope_inv_freq(32, 500000.0, scaling)
+    cos, sin = P.rope_cos_sin(np.arange(300), inv)
+    table = part.table.cpu().numpy()
+    assert table.shape == (300, 16, 2)
+    np.testing.assert_allclose(table[..., 0], cos[:, :16], atol=1e-7)
+    np.testing.assert_allclose(table[..., 1], sin[:, :16], atol=1e-7)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_swiglu_part(dtype):
+    from prefixserve_amd.parts.mlp import SwiGLU
+
+    rt = runtime(dtype)
+    part = SwiGLU(hidden_size=72, intermediate_size=200, names={"gate": "g", "up": "u", "down": "d"})
+    w = {"g": 0.2 * torch.randn(200, 72), "u": 0.2 * torch.randn(200, 72), "d": 0.2 * torch.randn(72, 200)}
+    w = {k: v.to(torch.bfloat16) for k, v in w.items()}
+    part.bind(w, rt)
+    for t in (3, 100):
+        x = torch.randn(t, 72, device=DEV).to(dtype)
+        want = P.swiglu_mlp(x.float().cpu().double().numpy(), *(w[k].double().numpy() for k in "gud"))
+        assert rel(part.forward(x, None), want) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("hq,hkv,d", [(6, 2, 32), (5, 5, 16), (8, 2, 64)])
+def test_attention_part_whole_and_in_portions(dtype, hq, hkv, d):
+    from prefixserve_amd.parts.attention import LayerCache, PagedAttention
+    from prefixserve_amd.parts.rope import RotaryEmbedding
+
+    rt = runtime(dtype)
+    hidden, n = 80, 75
+    rope = RotaryEmbedding(head_dim=d, theta=10000.0)
+    rope.bind({}, rt)
+    rope.prepare(128)
+    names = {"q": "q", "k": "k", "v": "v", "o": "o"}
+    part = PagedAttention(hidden_size=hidden, positions={"rope": rope}, num_heads=hq, num_kv_heads=hkv, head_dim=d,
+                          names=names, position="rope")
+    w = {"q": torch.randn(hq * d, hidden), "k": torch.randn(hkv * d, hidden), "v": torch.randn(hkv * d, hidden),
+         "o": torch.randn(hidden, hq * d)}
+    w = {k: (0.15 * v).to(torch.bfloat16) for k, v in w.items()}
+    part.bind(w, rt)
+    x = torch.randn(n, hidden, device=DEV).to(dtype)
+
+    xs = x.float().cpu().double().numpy()
+    wd = {k: v.double().numpy() for k, v in w.items()}
+    cos, sin = P.rope_cos_sin(np.arange(n), P.rope_inv_freq(d, 10000.0, None))
+    q = P.apply_rope((xs @ wd["q"].T).reshape(n, hq, d), cos, sin)
+    k = P.apply_rope((xs @ wd["k"].T).reshape(n, hkv, d), cos, sin)
+    v = (xs @ wd["v"].T).reshape(n, hkv, d)
+    want = P.causal_attention(q, k, v).reshape(n, hq * d) @ wd["o"].T
+
+    pk = StepPacker(DEV, [GroupMeta(8)], 10, 128, 4, rt.ops.PREFILL_TILE_Q)
+    table = [5, 2, 7, 0, 3]
+    for cuts in ([n], [30, 1, 1, 2, 41]):
+        cache = LayerCache(kv=torch.zeros(8, 2, hkv, 16 * d, dtype=dtype, device=DEV), group=0, window=None)
+        outs, p0 = [], 0
+        for c in cuts:
+            ctx = pk.pack([StepItem("a", [1] * c, p0, [table])])
+            outs.append(part.forward(x[p0:p0 + c].contiguous(), ctx, cache, None, True).clone())
+            p0 += c
+        assert rel(torch.cat(outs), want) < TOL[dtype] * 2
+
+
+def test_a_toy_mixer_with_state_of_its_own(tmp_path):
+    """A running mean over the request's tokens (fixed-size state per request, no pages),
+    alternating with attention layers; defined, registered and run from this test only."""
+    import json
+
+    from safetensors.torch import save_file
+
+    from prefixserve_amd.config import register_architecture, registered_architectures
+    from prefixserve_amd.engine.replay import TraceReplayer
+    from prefixserve_amd.engine.runner import ModelRunner
+    from prefixserve_amd.parts import (LayerRun, LayerSpec, Mixer, ModelSpec, PartSpec, StateNeed, WeightWant,
+                                       register_mixer)
+
+    class RunningMean(Mixer):
+        """out_t = W . mean(x_0..x_t); the state is (sum [hidden], count [1]) per request."""
+
+        def __init__(self, hidden_size, positions, name):
+            self.h, self.name = hidden_size, name
+
+        def weights(self):
+            return {self.name: WeightWant((self.h, self.h))}
+
+        def state_need(self):
+            return StateNeed((self.h + 1,), torch.float32)
+
+        def bind(self, tensors, rt):
+            super().bind(tensors, rt)
+            self.w = rt.ops.prepare_matrix(tensors[self.name], rt)
+
+        def forward(self, x, ctx, cache, state, writes_cache):
+            assert cache is None and state is not None
+            out = self.rt.workspace.get("toy.mean", tuple(x.shape), x.dtype)
+            starts = ctx.host["item_start"].tolist()
+            for i in range(ctx.num_items):
+                slot = int(ctx.host["slots"][i])
+                if int(ctx.host["item_pos0"][i]) == 0:
+                    state[slot].zero_()                               # a new request starts from nothing
+                seg = x[starts[i]:starts[i + 1]].float()
+                sums = state[slot, : self.h] + torch.cumsum(seg, 0)
+                counts = state[slot, self.h] + torch.arange(1, seg.shape[0] + 1, device=x.device)
+                out[starts[i]:starts[i + 1]] = (sums / counts[:, None]).to(x.dtype)
+                state[slot, : self.h] = sums[-1]
+                state[slot, self.h] = counts[-1]
+            delta = self.rt.workspace.get("toy.delta", tuple(x.shape), x.dtype)
+            self.rt.ops.linear(out, self.w, delta)
+            return delta
+
+    class ToyConfig:
+        def __init__(self, raw):
+            self.raw = raw
+
+        @classmethod
+        def from_dicts(cls, raw, gen=None):
+            return cls(dict(raw))
+
+    def build(cfg):
+        r = cfg.raw
+        h = r["hidden_size"]
+        attn = PartSpec("paged_attention", {"num_heads": 4, "num_kv_heads": 2, "head_dim": 16, "position": "rope",
+                                            "names": {"q": "q.weight", "k": "k.weight", "v": "v.weight", "o": "o.weight"}})
+        mean = PartSpec("test_running_mean", {"name": "mix.weight"})
+        ff = PartSpec("swiglu", {"intermediate_size": r["inner"], "names": {"gate": "g.weight", "up": "u.weight", "down": "d.weight"}})
+        norm = lambda n: PartSpec("rmsnorm", {"eps": 1e-5, "name": n})
+        layers = tuple(LayerSpec(prefix=f"l{i}.", mixer=mean if i % 2 else attn, feed_forward=ff,
+                                 mixer_norm=norm("n1.weight"), feed_forward_norm=norm("n2.weight")) for i in range(3))
+        # layer 1 (the toy mixer) runs twice; layer 2 reads the keys and values layer 0 wrote
+        order = (LayerRun(0, 0), LayerRun(1, 1), LayerRun(2, 0, writes_cache=False), LayerRun(1, 2))
+        return ModelSpec(vocab_size=r["vocab_size"], hidden_size=h, embedding="emb.weight", layers=layers, order=order,
+                         final_norm=norm("norm.weight"), final_norm_prefix="", head=None,
+                         positions={"rope": PartSpec("rope", {"head_dim": 16, "theta": 10000.0})}, max_position=512)
+
+    if "ToyMeanForCausalLM" not in registered_architectures():
+        register_mixer("test_running_mean", RunningMean)
+        register_architecture("ToyMeanForCausalLM", ToyConfig, build)
+
+    from prefixserve_amd.parts import DecoderModel
+    from prefixserve_amd.weights import random_tensors
+
+    raw = {"architectures": ["ToyMeanForCausalLM"], "hidden_size": 64, "inner": 96, "vocab_size": 100}
+    (tmp_path / "config.json").write_text(json.dumps(raw))
+    model = DecoderModel(build(ToyConfig(raw)))
+    save_file(random_tensors(model.weights(), seed=5, std=0.1), str(tmp_path / "model.safetensors"))
+
+    runner = ModelRunner(tmp_path, dtype="float32", device="cuda:0", num_blocks=16, max_seq_len=128, max_num_seqs=4,
+                         use_graphs=False)
+    assert runner.state_bytes_per_slot == 2 * 65 * 4 and len(runner.states) == 2
+    assert len(runner.layer_groups) == 1 and runner.layer_groups[0].entries == (0,)
+    toks = np.random.default_rng(0).integers(0, 100, 60).tolist()
+    other = np.random.default_rng(1).integers(0, 100, 33).tolist()
+    rp = TraceReplayer(runner)
+    whole = rp.run_step({"step": 0, "entries": [{"id": "a", "tokens": toks, "want": list(range(60))}], "end": ["a"]})
+    # the same request in portions, beside another request that keeps its own state
+    outs, p0 = [], 0
+    for k, c in enumerate([7, 2, 30, 1, 1, 19]):
+        entries = [{"id": "b", "tokens": toks[p0:p0 + c], "want": list(range(c))}]
+        if k < 3:
+            entries.insert(0, {"id": "c", "tokens": other[11 * k:11 * k + 11], "want": []})
+        got = rp.run_step({"step": k + 1, "entries": entries, "end": ["c"] if k == 2 else []})
+        outs.append(got)
+        p0 += c
+    cut = np.concatenate(outs)
+    assert np.abs(cut - whole).max() / np.abs(whole).max() < 1e-5
+    assert np.abs(whole).max() > 0.1 and np.isfinite(whole).all()

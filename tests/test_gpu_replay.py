@@ -1,0 +1,169 @@
+"""The engine against the plain implementation in every way of cutting the work, in 32-bit
+and in bfloat16: each request alone and whole; most of it in one step and the last 32 tokens
+one by one; portions of changing size down to two tokens; and mixed, up to four live
+requests with so few pages that they are used again. Once in-process, once through
+``bin/trace_run`` as a user would run it."""
+
+from __future__ import annotations
+
+import json
+import os
+import subprocess
+import sys
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+import traces
+from configs import TINY, TOL_BF16, TOL_F32
+from prefixserve_amd.engine.replay import TraceReplayer
+from prefixserve_amd.engine.runner import ModelRunner
+
+pytestmark = pytest.mark.gpu
+ROOT = Path(__file__).resolve().parent.parent
+TOL = {"float32": TOL_F32, "bfloat16": TOL_BF16}
+LENGTHS = [70, 33, 120, 97, 64, 18, 130, 45, 101, 77, 128, 90]
+
+
+def requests_for(name, lengths=LENGTHS, seed=1):
+    rng = np.random.default_rng(seed)
+    return [rng.integers(0, TINY[name]["vocab_size"], n).tolist() for n in lengths]
+
+
+def runner_for(model_dir, dtype, num_blocks, graphs=True, max_seq_len=256):
+    return ModelRunner(model_dir, dtype=dtype, device="cuda:0", num_blocks=num_blocks, max_seq_len=max_seq_len,
+                       max_num_seqs=8, use_graphs=graphs)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_every_cutting_matches_the_plain_model(name, dtype, model_dirs, plain_models):
+    reqs = requests_for(name)
+    truth = [plain_models[name].logits(t) for t in reqs]
+    runner = runner_for(model_dirs[name], dtype, 64)
+    worst = {}
+    for build in (traces.whole, traces.decode_tail, traces.portions):
+        steps, expect = build(reqs)
+        worst[build.__name__] = traces.compare(TraceReplayer(runner).run_step, steps, expect, truth, TOL[dtype])
+    steps, expect, peak = traces.mixed(reqs, seed=3)
+    assert sum(len(r) for r in reqs) > 1.5 * peak
+    small = runner_for(model_dirs[name], dtype, peak // 16)
+    small.pools.tensors[0].fill_(1e30)                              # a reused page never holds zeros
+    rp = TraceReplayer(small)
+    worst["mixed"] = traces.compare(rp.run_step, steps, expect, truth, TOL[dtype])
+    assert rp.cache.num_free(0) == peak // 16
+    print(name, dtype, {k: f"{v:.2e}" for k, v in worst.items()})
+    if dtype == "float32":
+        assert max(worst.values()) < 2e-5                           # well inside the bar
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_cuttings_agree_with_each_other(dtype, model_dirs):
+    """Whatever the distance to the plain model, the engine must agree with itself: the same
+    position's logits from a whole prompt, from a decode step and from a mixed batch differ
+    by rounding only."""
+    reqs = requests_for("C", [150, 99], seed=5)
+    runner = runner_for(model_dirs["C"], dtype, 64)
+    rows = {}
+    for build in (traces.whole, traces.decode_tail, traces.portions):
+        steps, expect = build(reqs)
+        rp = TraceReplayer(runner)
+        got = {}
+        for st, ex in zip(steps, expect):
+            out = rp.run_step(st)
+            for row, key in zip(out if out is not None else [], ex):
+                got[key] = row
+        rows[build.__name__] = got
+    tol = 1e-5 if dtype == "float32" else 3e-2
+    for key, ref in rows["whole"].items():
+        for other in ("decode_tail", "portions"):
+            if key in rows[other]:
+                err = np.abs(rows[other][key] - ref).max() / np.abs(ref).max()
+                assert err < tol, f"{other} vs whole at {key}: {err:.3e}"
+
+
+def test_graph_replay_equals_eager_decoding(model_dirs):
+    """Decode steps through a captured graph, replayed many times with other work in between,
+    against the same steps launched one by one."""
+    reqs = requests_for("C", [90, 61, 40], seed=9)
+    out = {}
+    for graphs in (False, True):
+        runner = runner_for(model_dirs["C"], "bfloat16", 32, graphs=graphs)
+        rp = TraceReplayer(runner)
+        rows = []
+        for i, t in enumerate(reqs):
+            rp.run_step({"step": 0, "entries": [{"id": f"r{i}", "tokens": t[:20], "want": []}], "end": []})
+        pos = [20, 20, 20]
+        for k in range(20):
+            entries = [{"id": f"r{i}", "tokens": [reqs[i][pos[i]]], "want": [0]} for i in range(3)]
+            rows.append(rp.run_step({"step": k, "entries": entries, "end": []}))
+            pos = [p + 1 for p in pos]
+            if k % 7 == 3:                                           # eager work between replays
+                rp.run_step({"step": 100 + k, "entries": [{"id": "x", "tokens": list(range(5, 40)), "want": [34]}], "end": ["x"]})
+        out[graphs] = np.stack(rows)
+        if graphs:
+            assert (3, 3) in runner._graphs
+    assert np.array_equal(out[False], out[True])
+
+
+def test_first_tokens_of_a_sequence(model_dirs, plain_models):
+    """Positions 0, 1, 2: a single key, no rotation at position 0."""
+    for dtype in ("float32", "bfloat16"):
+        runner = runner_for(model_dirs["B"], dtype, 8)
+        rp = TraceReplayer(runner)
+        toks = [7, 300, 12]
+        truth = plain_models["B"].logits(toks)
+        for p in range(3):
+            got = rp.run_step({"step": p, "entries": [{"id": "a", "tokens": [toks[p]], "want": [0]}], "end": []})
+            assert np.abs(got[0] - truth[p]).max() / np.abs(truth[p]).max() < TOL[dtype]
+
+
+def test_long_decoding(model_dirs, plain_models):
+    """Three hundred tokens one by one after a short prompt, crossing many pages, with the
+    graph path; compared at every position."""
+    toks = requests_for("A", [330], seed=12)[0]
+    truth = plain_models["A"].logits(toks)
+    for dtype in ("float32", "bfloat16"):
+        runner = runner_for(model_dirs["A"], dtype, 24, max_seq_len=384)
+        rp = TraceReplayer(runner)
+        rp.run_step({"step": 0, "entries": [{"id": "a", "tokens": toks[:10], "want": []}], "end": []})
+        worst = 0.0
+        for p in range(10, 330):
+            got = rp.run_step({"step": p, "entries": [{"id": "a", "tokens": [toks[p]], "want": [0]}], "end": []})
+            worst = max(worst, float(np.abs(got[0] - truth[p]).max() / np.abs(truth[p]).max()))
+        assert worst < TOL[dtype], f"{dtype}: {worst:.3e}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(dtype, model_dirs, plain_models, tmp_path):
+    """bin/trace_run as a user runs it: JSON lines in, <step>.f32 files and 'done <step>' out."""
+    name = "B"
+    reqs = requests_for(name, LENGTHS[:8])
+    truth = [plain_models[name].logits(t) for t in reqs]
+    steps, expect, peak = traces.mixed(reqs, seed=7)
+    out = tmp_path / "out"
+    proc = subprocess.Popen(
+        [sys.executable, str(ROOT / "bin" / "trace_run"), "--model", str(model_dirs[name]), "--dtype", dtype,
+         "--out", str(out), "--max-tokens", str(peak)],
+        stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True, env=dict(os.environ))
+    try:
+        for st, ex in zip(steps, expect):
+            proc.stdin.write(json.dumps(st) + "\n")
+            proc.stdin.flush()
+            line = proc.stdout.readline().strip()
+            assert line == f"done {st['step']}", line
+            path = out / f"{st['step']}.f32"
+            if ex:
+                got = np.fromfile(path, dtype="<f4").reshape(len(ex), -1)
+                for row, (i, p) in zip(got, ex):
+                    err = np.abs(row - truth[i][p]).max() / np.abs(truth[i][p]).max()
+                    assert err < TOL[dtype], f"step {st['step']} request {i} position {p}: {err:.3e}"
+            else:
+                assert not path.exists()
+        proc.stdin.close()
+        assert proc.wait(timeout=60) == 0
+    finally:
+        if proc.poll() is None:
+            proc.kill()
