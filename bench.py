@@ -1,0 +1,177 @@
+#!/usr/bin/env python3
+"""Headline benchmark: Llama 3.2 1B shape, random bfloat16 weights, 4,096-token context.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one decode step of the scheduler-driven engine (schedule, run, sample, commit)
+at batch 8 over 2,048-token prompts. Prints ONE JSON line: decoded tokens per second as
+``value``, the 2,048-token prefill under ``prefill``, the decode step's HBM roofline under
+``roofline`` and batch 1 / batch 64 decoding under ``points``. Synthetic data: seeded
+uniform-random token ids and seeded random weights; nothing is downloaded.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import tempfile
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+# MI355X published peaks.
+HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_TFLOPS = {"bfloat16": 2500.0, "float32": 157.3}
+
+LLAMA_1B = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama", "vocab_size": 128256, "hidden_size": 2048,
+    "intermediate_size": 8192, "num_hidden_layers": 16, "num_attention_heads": 32, "num_key_value_heads": 8,
+    "head_dim": 64, "rms_norm_eps": 1e-5, "rope_theta": 500000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 32.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 8192},
+    "max_position_embeddings": 131072, "tie_word_embeddings": True,
+}
+
+
+def prefill_flops(cfg: dict, layers: int, tokens: int) -> float:
+    h, i, v = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+    hq, hkv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    per_token_layer = 2 * h * (hq + 2 * hkv) * d + 2 * hq * d * h + 2 * h * 2 * i + 2 * i * h
+    attention = 2 * 2 * (tokens * (tokens + 1) / 2) * hq * d          # causal QK^T and PV
+    return layers * (tokens * per_token_layer + attention) + 2 * h * v  # one row through the output matrix
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
+    ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--prompt-len", type=int, default=2048)
+    ap.add_argument("--context", type=int, default=4096)
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / batch 64 points")
+    ap.add_argument("--no-graphs", action="store_true")
+    ap.add_argument("--model", default=None, help="use this model folder instead of writing random weights")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import numpy as np
+    import torch
+
+    from prefixserve_amd import Engine, EngineConfig
+    from prefixserve_amd.weights import write_random_model
+
+    cfg = dict(LLAMA_1B)
+    layers_full = cfg["num_hidden_layers"]
+    if args.layers is not None:
+        cfg["num_hidden_layers"] = args.layers
+    layers = cfg["num_hidden_layers"]
+    tmp = None
+    if args.model is None:
+        tmp = tempfile.TemporaryDirectory(prefix="psamd_bench_")
+        model_dir = write_random_model(tmp.name, cfg, seed=0)
+    else:
+        model_dir = Path(args.model)
+    max_batch = max(args.batch, 1 if args.no_points else 64)
+    blocks = max_batch * (args.context // 16) + 64
+    engine = Engine(EngineConfig(model_path=model_dir, dtype=args.dtype, max_num_seqs=max_batch,
+                                 max_prefill_tokens=args.prompt_len, max_seq_len=args.context, num_blocks=blocks,
+                                 use_graphs=not args.no_graphs))
+    runner = engine.runner
+    rng = np.random.default_rng(0)
+    vocab = cfg["vocab_size"]
+    weight_bytes = runner.model.step_weight_bytes()
+    kv_bytes_per_token = sum(runner.bytes_per_block) // 16
+
+    def sync() -> None:
+        torch.cuda.synchronize()
+
+    def decode_run(batch: int, steps: int, warmup: int) -> dict:
+        sched = engine.make_scheduler(chunk_size=args.prompt_len, enable_prefix_cache=False)
+        for b in range(batch):
+            sched.add_request(f"d{batch}-{b}", rng.integers(0, vocab, args.prompt_len), args.context - args.prompt_len - 1,
+                              ignore_eos=True)
+        # prompts, untimed: one request's prompt per step
+        while any(r.num_computed < len(r.prompt) for r in sched._requests.values()) or sched.stats().num_waiting:
+            bt = sched.schedule_step(args.prompt_len, batch)
+            sched.commit(bt, engine.step(bt))
+        for _ in range(warmup):
+            bt = sched.schedule_step(args.prompt_len, batch)
+            sched.commit(bt, engine.step(bt))
+        kv_start = sum(r.num_computed for r in sched._requests.values())
+        sync()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            bt = sched.schedule_step(args.prompt_len, batch)
+            assert len(bt.work) == batch and bt.num_tokens == batch
+            sched.commit(bt, engine.step(bt))
+        sync()
+        dt = time.perf_counter() - t0
+        kv_end = sum(r.num_computed for r in sched._requests.values())
+        for rid in list(sched._requests):
+            sched.free_request(rid)
+        mean_kv_tokens = 0.5 * (kv_start + kv_end) + 0.5 * batch       # keys read per step, summed over requests
+        bytes_per_step = weight_bytes + mean_kv_tokens * kv_bytes_per_token
+        return {"tok_s": batch * steps / dt, "ms_per_step": 1e3 * dt / steps,
+                "gbs": bytes_per_step * steps / dt / 1e9, "kv_len": mean_kv_tokens / batch}
+
+    def prefill_run(reps: int = 5, warm: int = 2) -> dict:
+        from prefixserve_amd.engine.batch import StepItem
+
+        n = args.prompt_len
+        table = [list(range(-(-n // 16)))]
+        toks = rng.integers(0, vocab, n)
+        item = [StepItem("p", toks, 0, table, 0, [n - 1])]
+        for _ in range(warm):
+            runner.step(item)
+        sync()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            runner.step(item)
+        sync()
+        ms = 1e3 * (time.perf_counter() - t0) / reps
+        flops = prefill_flops(cfg, layers, n)
+        return {"value": n / (ms / 1e3), "tokens": n, "ms": ms,
+                "frac": flops / (ms / 1e3) / (MFMA_PEAK_TFLOPS[args.dtype] * 1e12)}
+
+    prefill = prefill_run()
+    main_run = decode_run(args.batch, args.steps, args.warmup)
+    points = {}
+    if not args.no_points:
+        points["decode_b1"] = decode_run(1, max(16, args.steps // 2), max(4, args.warmup // 2))["tok_s"]
+        points["decode_b64"] = decode_run(64, max(16, args.steps // 4), max(4, args.warmup // 4))["tok_s"]
+
+    line = {
+        "metric": "decode_tokens_per_second", "value": main_run["tok_s"], "unit": "tok/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": main_run["ms_per_step"], "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic: seeded uniform-random token ids, seeded random weights",
+        "config": {
+            "model": "llama-3.2-1b-shape", "layers": layers_full, "layers_run": layers, "hidden": cfg["hidden_size"],
+            "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
+            "intermediate": cfg["intermediate_size"], "vocab": vocab, "rope_theta": cfg["rope_theta"],
+            "rope_factor": cfg["rope_scaling"]["factor"], "rms_norm_eps": cfg["rms_norm_eps"],
+            "tied": cfg["tie_word_embeddings"], "global_batch": args.batch, "seq_len": args.context,
+            "prompt_len": args.prompt_len, "page_tokens": 16, "parallelism": "none",
+        },
+        "prefill": prefill,
+        "roofline": {"bound": "hbm", "achieved": main_run["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": main_run["gbs"] / HBM_PEAK_GBS},
+        "points": points,
+    }
+    print(json.dumps(line), flush=True)
+    if tmp is not None:
+        tmp.cleanup()
+    return 0
+
+
+if __name__ == "__main__":
+    raise SystemExit(main())

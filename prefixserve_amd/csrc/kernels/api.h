@@ -17,10 +17,13 @@ const char* psamd_last_error(void);
 int psamd_embed(void* stream, const int32_t* ids, const void* table, int table_dtype, float* out, int64_t tokens,
                 int hidden);
 
-// rows == NULL: residual[r] += delta[r] (if delta), out[r] = weight * rmsnorm(residual[r]) for r < out_rows.
-// rows != NULL: out[i] = weight * rmsnorm(residual[rows[i]] + delta[rows[i]]); residual untouched.
-int psamd_add_rmsnorm(void* stream, float* residual, const void* delta, const int32_t* rows, const void* weight,
-                      int weight_dtype, float eps, void* out, int act_dtype, int64_t out_rows, int hidden);
+// x = residual + delta, where delta is [rows, hidden] (delta_dtype) or n_partials float32 slices of that
+// shape, partial_stride elements apart (the partial sums of a K-split product).
+// rows == NULL: residual[r] = x[r], out[r] = weight * rmsnorm(x[r]) for r < out_rows.
+// rows != NULL: out[i] = weight * rmsnorm(x[rows[i]]); residual untouched.
+int psamd_add_rmsnorm(void* stream, float* residual, const void* delta, int delta_dtype, int n_partials,
+                      int64_t partial_stride, const int32_t* rows, const void* weight, int weight_dtype, float eps,
+                      void* out, int act_dtype, int64_t out_rows, int hidden);
 
 // out[t, c] = silu(gate_up[t, c]) * gate_up[t, inter + c]
 int psamd_swiglu(void* stream, const void* gate_up, void* out, int act_dtype, int64_t tokens, int inter);
@@ -35,8 +38,15 @@ int psamd_linear(void* stream, const void* x, int x_dtype, const void* w, int w_
                  int64_t M, int N, int K);
 
 // bfloat16 product for M <= 64 on the matrix cores. epilogue 1: w = [gate; up], out = silu(gate) * up.
+// ksplit > 1: out receives ksplit float32 partial sums [ksplit][M, n_out] (plain epilogue only).
 int psamd_linear_skinny(void* stream, const void* x, const void* w, void* out, int out_dtype, int M, int n_out, int K,
-                        int epilogue);
+                        int epilogue, int ksplit);
+
+// The q/k/v projection of a step of at most 64 tokens fused with the rotation of q and k and the write of k
+// and v into their cache pages (see psamd_rope_kv_append for the meaning of table, kv and write_slot).
+int psamd_qkv_rope_append(void* stream, const void* x, const void* w, void* qkv_out, int M, int K, int hq, int hkv,
+                          int head_dim, const int32_t* positions, const float* table, void* kv,
+                          const int32_t* write_slot);
 
 int psamd_attention_generic(void* stream, const void* qkv, int q_stride, void* out, const void* kv, int act_dtype,
                             int64_t tokens, const int32_t* positions, const int32_t* tok_item,

@@ -11,7 +11,8 @@
 //  * decode: one workgroup per (request, kv head, split of the key range); the `group`
 //    query heads sharing the kv head are the columns of a 16x16x32 tile, so every key and
 //    value byte is read once for all of them; 4 waves interleave 32-key tiles and merge by
-//    log-sum-exp in LDS; a second small kernel merges the splits.
+//    log-sum-exp in LDS; a second small kernel merges the splits (a device-wide fence inside
+//    the kernel would be far dearer than a launch on this multi-die part).
 //
 // Softmax statistics, scaling and masks are float. Page layout per layer:
 // [num_blocks][2][kv_heads][16 * D], half 0 keys [16][D], half 1 values [D][16].
@@ -176,8 +177,9 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
 // part_o[dec][head][split][D], part_ml[dec][head][split][2] = (max, sum).
 template <int NS, int CT>
 __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
-    const bf16_t* __restrict__ qkv, int q_stride, const bf16_t* __restrict__ kv, float* __restrict__ part_o,
-    float* __restrict__ part_ml, const int32_t* __restrict__ dec_items, const int32_t* __restrict__ item_start,
+    const bf16_t* __restrict__ qkv, int q_stride, const bf16_t* __restrict__ kv, bf16_t* __restrict__ out,
+    float* __restrict__ part_o, float* __restrict__ part_ml, const int32_t* __restrict__ dec_items,
+    const int32_t* __restrict__ item_start,
     const int32_t* __restrict__ item_end, const int32_t* __restrict__ table_off,
     const int32_t* __restrict__ block_ids, int hq, int hkv, int nsplit, float scale, int window) {
   constexpr int D = 16 * NS;
@@ -320,6 +322,10 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
       acc += wgt * sm_o[(static_cast<int64_t>(w) * group + hh) * D + d];
       ll += wgt * sm_l[w * group + hh];
     }
+    if (nsplit == 1) {   // nothing to merge with: this is the result
+      out[t * (static_cast<int64_t>(hq) * D) + static_cast<int64_t>(kvh * group + hh) * D + d] = float_to_bf16(acc / ll);
+      continue;
+    }
     const int64_t slot = (static_cast<int64_t>(di) * hq + kvh * group + hh) * nsplit + split;
     part_o[slot * D + d] = acc;
     if (d == 0) {
@@ -361,25 +367,25 @@ static int launch_prefill(hipStream_t s, const void* qkv, int q_stride, void* ou
 }
 
 template <int NS, int CT>
-static int launch_decode(hipStream_t s, const void* qkv, int q_stride, const void* kv, float* part_o, float* part_ml,
-                         const int32_t* dec_items, int n_dec, const int32_t* item_start, const int32_t* item_end,
+static int launch_decode(hipStream_t s, const void* qkv, int q_stride, const void* kv, void* out, float* part_o,
+                         float* part_ml, const int32_t* dec_items, int n_dec, const int32_t* item_start, const int32_t* item_end,
                          const int32_t* table_off, const int32_t* block_ids, int hq, int hkv, int nsplit, float scale,
                          int window) {
   const int group = hq / hkv;
   const size_t smem = sizeof(float) * (8 * group + 4 * static_cast<size_t>(group) * 16 * NS);
   attn_decode_mfma_kernel<NS, CT><<<dim3(n_dec, hkv, nsplit), dim3(256), smem, s>>>(
-      static_cast<const bf16_t*>(qkv), q_stride, static_cast<const bf16_t*>(kv), part_o, part_ml, dec_items,
-      item_start, item_end, table_off, block_ids, hq, hkv, nsplit, scale, window);
+      static_cast<const bf16_t*>(qkv), q_stride, static_cast<const bf16_t*>(kv), static_cast<bf16_t*>(out), part_o,
+      part_ml, dec_items, item_start, item_end, table_off, block_ids, hq, hkv, nsplit, scale, window);
   return check_launch("psamd_attention_decode");
 }
 
 template <int NS>
-static int dispatch_decode_ct(int ct, hipStream_t s, const void* qkv, int q_stride, const void* kv, float* part_o,
-                              float* part_ml, const int32_t* dec_items, int n_dec, const int32_t* item_start,
+static int dispatch_decode_ct(int ct, hipStream_t s, const void* qkv, int q_stride, const void* kv, void* out,
+                              float* part_o, float* part_ml, const int32_t* dec_items, int n_dec, const int32_t* item_start,
                               const int32_t* item_end, const int32_t* table_off, const int32_t* block_ids, int hq,
                               int hkv, int nsplit, float scale, int window) {
 #define PSAMD_DEC(CT_)                                                                                             \
-  return launch_decode<NS, CT_>(s, qkv, q_stride, kv, part_o, part_ml, dec_items, n_dec, item_start, item_end, \
+  return launch_decode<NS, CT_>(s, qkv, q_stride, kv, out, part_o, part_ml, dec_items, n_dec, item_start, item_end, \
                                 table_off, block_ids, hq, hkv, nsplit, scale, window)
   switch (ct) {
     case 1: PSAMD_DEC(1);
@@ -441,8 +447,8 @@ int psamd_attention_decode(void* stream, const void* qkv, int q_stride, void* ou
   const int ct = group <= 16 ? 1 : (group <= 32 ? 2 : 4);
   int rc;
 #define PSAMD_DEC_NS(NS_)                                                                                          \
-  rc = dispatch_decode_ct<NS_>(ct, s, qkv, q_stride, kv, part_o, part_ml, dec_items, n_dec, item_start, item_end, \
-                               table_off, block_ids, hq, hkv, nsplit, scale, window);                            \
+  rc = dispatch_decode_ct<NS_>(ct, s, qkv, q_stride, kv, out, part_o, part_ml, dec_items, n_dec, item_start,    \
+                               item_end, table_off, block_ids, hq, hkv, nsplit, scale, window);                  \
   break
   switch (head_dim / 16) {
     case 1: PSAMD_DEC_NS(1);
@@ -453,7 +459,7 @@ int psamd_attention_decode(void* stream, const void* qkv, int q_stride, void* ou
     default: PSAMD_DEC_NS(16);
   }
 #undef PSAMD_DEC_NS
-  if (rc != 0) return rc;
+  if (rc != 0 || nsplit == 1) return rc;
   attn_decode_merge_kernel<<<dim3(n_dec, hq), dim3(64), 0, s>>>(part_o, part_ml, static_cast<bf16_t*>(out), dec_items,
                                                                item_start, hq, head_dim, nsplit);
   return check_launch("psamd_attention_decode(merge)");

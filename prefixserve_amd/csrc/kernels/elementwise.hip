@@ -24,31 +24,65 @@ __global__ void embed_kernel(const int32_t* __restrict__ ids, const W* __restric
 
 // ------------------------------------------------------------------ add + rmsnorm
 
-// One block per output row. residual (float) += delta; out = weight * x * rsqrt(mean(x^2)+eps).
-// With `rows` the block handles residual row rows[blockIdx.x] and leaves the residual as it is.
-template <typename A, int kThreads>
-__global__ void add_rmsnorm_kernel(float* __restrict__ residual, const A* __restrict__ delta,
-                                   const int32_t* __restrict__ rows, const void* __restrict__ weight,
-                                   int weight_dtype, float eps, A* __restrict__ out, int hidden) {
+// One block per output row. x = residual + sum of the delta slices; out = weight * x *
+// rsqrt(mean(x^2) + eps), everything in float. `delta` is either [rows, hidden] in the
+// activation type or n_partials float slices [n_partials][rows, hidden] (partial sums of a
+// K-split product). Without `rows` the block handles row blockIdx.x and stores x back as the
+// new residual; with `rows` it handles residual row rows[blockIdx.x] and leaves it as it is.
+// Rows up to kCache * kThreads wide stay in registers between the two passes.
+template <typename A, int kThreads, int kCache>
+__global__ __launch_bounds__(kThreads) void add_rmsnorm_kernel(
+    float* __restrict__ residual, const void* __restrict__ delta, int delta_dtype, int n_partials,
+    int64_t partial_stride, const int32_t* __restrict__ rows, const void* __restrict__ weight, int weight_dtype,
+    float eps, A* __restrict__ out, int hidden) {
   __shared__ float scratch[kThreads / kWave];
   const int64_t src = rows != nullptr ? rows[blockIdx.x] : blockIdx.x;
   float* r = residual + src * hidden;
-  const A* d = delta != nullptr ? delta + src * hidden : nullptr;
+  const int64_t doff = src * hidden;
   A* o = out + static_cast<int64_t>(blockIdx.x) * hidden;
-  const bool store = rows == nullptr && d != nullptr;
-  float ss = 0.f;
-  for (int i = threadIdx.x; i < hidden; i += kThreads) {
+  const bool store = rows == nullptr && delta != nullptr;
+  const bool cached = hidden <= kCache * kThreads;
+
+  auto value = [&](int i) {
     float x = r[i];
-    if (d != nullptr) x += to_float<A>(d[i]);
-    if (store) r[i] = x;
-    ss += x * x;
+    if (delta != nullptr) {
+      for (int p = 0; p < n_partials; ++p) x += load_as_float(delta, delta_dtype, p * partial_stride + doff + i);
+    }
+    return x;
+  };
+
+  float v[kCache];
+  float ss = 0.f;
+  if (cached) {
+#pragma unroll
+    for (int j = 0; j < kCache; ++j) {
+      const int i = threadIdx.x + j * kThreads;
+      v[j] = i < hidden ? value(i) : 0.f;
+      ss += v[j] * v[j];
+    }
+  } else {
+    for (int i = threadIdx.x; i < hidden; i += kThreads) {
+      const float x = value(i);
+      if (store) r[i] = x;
+      ss += x * x;
+    }
   }
   ss = block_sum(ss, scratch, kThreads / kWave);
   const float inv = rsqrtf(ss / static_cast<float>(hidden) + eps);
-  for (int i = threadIdx.x; i < hidden; i += kThreads) {
-    float x = r[i];
-    if (!store && d != nullptr) x += to_float<A>(d[i]);
-    o[i] = from_float<A>(load_as_float(weight, weight_dtype, i) * (x * inv));
+  if (cached) {
+#pragma unroll
+    for (int j = 0; j < kCache; ++j) {
+      const int i = threadIdx.x + j * kThreads;
+      if (i < hidden) {
+        if (store) r[i] = v[j];
+        o[i] = from_float<A>(load_as_float(weight, weight_dtype, i) * (v[j] * inv));
+      }
+    }
+  } else {
+    for (int i = threadIdx.x; i < hidden; i += kThreads) {
+      const float x = store ? r[i] : value(i);
+      o[i] = from_float<A>(load_as_float(weight, weight_dtype, i) * (x * inv));
+    }
   }
 }
 
@@ -143,19 +177,25 @@ int psamd_embed(void* stream, const int32_t* ids, const void* table, int table_d
   return check_launch("psamd_embed");
 }
 
-int psamd_add_rmsnorm(void* stream, float* residual, const void* delta, const int32_t* rows, const void* weight,
-                      int weight_dtype, float eps, void* out, int act_dtype, int64_t out_rows, int hidden) {
+int psamd_add_rmsnorm(void* stream, float* residual, const void* delta, int delta_dtype, int n_partials,
+                      int64_t partial_stride, const int32_t* rows, const void* weight, int weight_dtype, float eps,
+                      void* out, int act_dtype, int64_t out_rows, int hidden) {
   PSAMD_REQUIRE(out_rows >= 0 && hidden > 0, "bad sizes");
   PSAMD_REQUIRE(weight_dtype == kF32 || weight_dtype == kBF16, "weight dtype must be float32 or bfloat16");
+  PSAMD_REQUIRE(delta == nullptr || delta_dtype == kF32 || delta_dtype == kBF16, "delta dtype");
+  PSAMD_REQUIRE(delta == nullptr || (n_partials >= 1 && (n_partials == 1 || delta_dtype == kF32)),
+                "partial sums must be float32");
   if (out_rows == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  constexpr int kThreads = 256;
+  constexpr int kThreads = 256, kCache = 16;
   if (act_dtype == kBF16) {
-    add_rmsnorm_kernel<bf16_t, kThreads><<<dim3(out_rows), dim3(kThreads), 0, s>>>(
-        residual, static_cast<const bf16_t*>(delta), rows, weight, weight_dtype, eps, static_cast<bf16_t*>(out), hidden);
+    add_rmsnorm_kernel<bf16_t, kThreads, kCache><<<dim3(out_rows), dim3(kThreads), 0, s>>>(
+        residual, delta, delta_dtype, n_partials, partial_stride, rows, weight, weight_dtype, eps,
+        static_cast<bf16_t*>(out), hidden);
   } else if (act_dtype == kF32) {
-    add_rmsnorm_kernel<float, kThreads><<<dim3(out_rows), dim3(kThreads), 0, s>>>(
-        residual, static_cast<const float*>(delta), rows, weight, weight_dtype, eps, static_cast<float*>(out), hidden);
+    add_rmsnorm_kernel<float, kThreads, kCache><<<dim3(out_rows), dim3(kThreads), 0, s>>>(
+        residual, delta, delta_dtype, n_partials, partial_stride, rows, weight, weight_dtype, eps,
+        static_cast<float*>(out), hidden);
   } else {
     return fail("psamd_add_rmsnorm: activation dtype must be float32 or bfloat16");
   }

@@ -87,36 +87,44 @@ __device__ __forceinline__ bf16x8 zero8() {
 
 __device__ __forceinline__ float silu_f(float g) { return g / (1.f + __expf(-g)); }
 
-// Each wave owns 16 output columns (rows of w) and walks all of K. Operand layout of
-// v_mfma_f32_16x16x32_bf16: lane l supplies row (l % 16), k = 8 * (l / 16) + [0, 8) of both
-// operands, and receives C[4 * (l / 16) + v][l % 16], v = 0..3, where C rows are rows of w
-// and C columns are tokens.
-// MT = number of 16-token column tiles. SWIGLU: w is [gate; up] with `n_out` rows each and
-// the wave computes silu(gate) * up for its 16 columns.
+// One workgroup (4 waves) owns 16 output columns (rows of w) and a range of K; its waves
+// take the 32-wide k-steps of that range in turn, so together they stream 256 contiguous
+// bytes of each row per round, and their partial tiles are summed through LDS. With
+// gridDim.y > 1 the K range is also split over workgroups and the float partial sums go to
+// out[blockIdx.y][M][n_out] for the consumer (the fused add+norm) to add up: that is how a
+// product with few output columns still fills the chip.
+//
+// Operand layout of v_mfma_f32_16x16x32_bf16: lane l supplies row (l % 16), k = 8 * (l / 16)
+// + [0, 8) of both operands and receives C[4 * (l / 16) + v][l % 16], v = 0..3; C rows are
+// rows of w, C columns are tokens. MT = number of 16-token column tiles. SWIGLU: w is
+// [gate; up] with n_out rows each and the result is silu(gate) * up.
 template <int MT, bool SWIGLU, typename TO>
 __global__ __launch_bounds__(256) void skinny_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                           TO* __restrict__ out, int M, int n_out, int K) {
+  constexpr int NACC = SWIGLU ? 2 * MT : MT;
+  __shared__ f32x4 red[4][NACC][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int n0 = (blockIdx.x * 4 + wave) * 16;
-  if (n0 >= n_out) return;
+  const int n0 = blockIdx.x * 16;
   const int r = lane & 15, g = lane >> 4;
   const int row = min(n0 + r, n_out - 1);
-  const bf16_t* wrow = w + static_cast<int64_t>(row) * K;
-  const bf16_t* wrow_up = SWIGLU ? w + static_cast<int64_t>(n_out + row) * K : nullptr;
+  const bf16_t* wrow = w + static_cast<int64_t>(row) * K + 8 * g;
+  const bf16_t* wrow_up = SWIGLU ? w + static_cast<int64_t>(n_out + row) * K + 8 * g : nullptr;
   const bf16_t* xrow[MT];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) xrow[mt] = x + static_cast<int64_t>(min(mt * 16 + r, M - 1)) * K;
+  for (int mt = 0; mt < MT; ++mt) xrow[mt] = x + static_cast<int64_t>(min(mt * 16 + r, M - 1)) * K + 8 * g;
 
-  f32x4 acc[MT], acc_up[MT];
+  f32x4 acc[NACC];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-    acc_up[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  }
-  const int kfull = K & ~31;
+  for (int i = 0; i < NACC; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const int steps = (K + 31) >> 5;
+  const int per_wg = (steps + gridDim.y - 1) / gridDim.y;
+  const int s_begin = blockIdx.y * per_wg;
+  const int s_end = min(s_begin + per_wg, steps);
+  const int s_full = min(s_end, K >> 5);          // steps that lie wholly inside K
 #pragma unroll 4
-  for (int k0 = 0; k0 < kfull; k0 += 32) {
-    const int k = k0 + 8 * g;
+  for (int s = s_begin + wave; s < s_full; s += 4) {
+    const int k = s << 5;
     const bf16x8 a = load8(wrow + k);
     bf16x8 a_up;
     if (SWIGLU) a_up = load8(wrow_up + k);
@@ -124,12 +132,13 @@ __global__ __launch_bounds__(256) void skinny_mfma_kernel(const bf16_t* __restri
     for (int mt = 0; mt < MT; ++mt) {
       const bf16x8 b = load8(xrow[mt] + k);
       acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mt], 0, 0, 0);
-      if (SWIGLU) acc_up[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_up, b, acc_up[mt], 0, 0, 0);
+      if (SWIGLU) acc[MT + mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_up, b, acc[MT + mt], 0, 0, 0);
     }
   }
-  if (kfull < K) {  // K % 32 in {8, 16, 24}: lane groups past the end contribute zeros
-    const int k = kfull + 8 * g;
-    const bool in = k < K;
+  // K % 32 in {8, 16, 24}: the last step is partial; lane groups past the end contribute zeros.
+  if (s_full < s_end && ((s_full - s_begin) & 3) == wave) {
+    const int k = s_full << 5;
+    const bool in = k + 8 * g < K;
     const bf16x8 a = in ? load8(wrow + k) : zero8();
     bf16x8 a_up = zero8();
     if (SWIGLU && in) a_up = load8(wrow_up + k);
@@ -137,32 +146,38 @@ __global__ __launch_bounds__(256) void skinny_mfma_kernel(const bf16_t* __restri
     for (int mt = 0; mt < MT; ++mt) {
       const bf16x8 b = in ? load8(xrow[mt] + k) : zero8();
       acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mt], 0, 0, 0);
-      if (SWIGLU) acc_up[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_up, b, acc_up[mt], 0, 0, 0);
+      if (SWIGLU) acc[MT + mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_up, b, acc[MT + mt], 0, 0, 0);
     }
   }
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    const int m = mt * 16 + r;
-    if (m >= M) continue;
+  for (int i = 0; i < NACC; ++i) red[wave][i][lane] = acc[i];
+  __syncthreads();
+  // Wave `wave` finishes column tiles wave, wave + 4, ... (MT <= 4: at most one each).
+  if (wave >= MT) return;
+  const int mt = wave;
+  f32x4 sum = red[0][mt][lane] + red[1][mt][lane] + red[2][mt][lane] + red[3][mt][lane];
+  if (SWIGLU) {
+    const f32x4 up = red[0][MT + mt][lane] + red[1][MT + mt][lane] + red[2][MT + mt][lane] + red[3][MT + mt][lane];
 #pragma unroll
-    for (int v = 0; v < 4; ++v) {
-      const int n = n0 + 4 * g + v;
-      if (n >= n_out) continue;
-      float val = acc[mt][v];
-      if (SWIGLU) val = silu_f(val) * acc_up[mt][v];
-      out[static_cast<int64_t>(m) * n_out + n] = from_float<TO>(val);
-    }
+    for (int v = 0; v < 4; ++v) sum[v] = silu_f(sum[v]) * up[v];
+  }
+  const int m = mt * 16 + r;
+  if (m >= M) return;
+  TO* dst = out + (static_cast<int64_t>(blockIdx.y) * M + m) * n_out;
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    const int n = n0 + 4 * g + v;
+    if (n < n_out) dst[n] = from_float<TO>(sum[v]);
   }
 }
 
 template <int MT>
 static int launch_skinny(hipStream_t s, const void* x, const void* w, void* out, int out_dtype, int M, int n_out,
-                         int K, int epilogue) {
-  const dim3 grid(static_cast<unsigned>(ceil_div(ceil_div(n_out, 16), 4))), block(256);
+                         int K, int epilogue, int ksplit) {
+  const dim3 grid(static_cast<unsigned>(ceil_div(n_out, 16)), static_cast<unsigned>(ksplit)), block(256);
   const bf16_t* xp = static_cast<const bf16_t*>(x);
   const bf16_t* wp = static_cast<const bf16_t*>(w);
   if (epilogue == 1) {
-    if (out_dtype != kBF16) return fail("psamd_linear_skinny: the SwiGLU epilogue writes bfloat16");
     skinny_mfma_kernel<MT, true, bf16_t><<<grid, block, 0, s>>>(xp, wp, static_cast<bf16_t*>(out), M, n_out, K);
   } else if (out_dtype == kBF16) {
     skinny_mfma_kernel<MT, false, bf16_t><<<grid, block, 0, s>>>(xp, wp, static_cast<bf16_t*>(out), M, n_out, K);
@@ -170,6 +185,99 @@ static int launch_skinny(hipStream_t s, const void* x, const void* w, void* out,
     skinny_mfma_kernel<MT, false, float><<<grid, block, 0, s>>>(xp, wp, static_cast<float*>(out), M, n_out, K);
   }
   return check_launch("psamd_linear_skinny");
+}
+
+// The q/k/v projection of a small step fused with what follows it: rotary encoding of q and
+// k, and the write of k and v into their cache pages. Same streaming scheme as skinny_mfma
+// (one workgroup = 16 rows of w over all of K, 4 waves taking k-steps in turn), but the 16
+// rows are chosen so that a rotation pair lies in one tile: 8 columns of a head's first half
+// and their 8 partners in the second half. After the product, lane groups 0-1 hold
+// first-half elements and groups 2-3 their partners, one shuffle apart.
+// qkv_out[m] receives the rotated q and k and v (the layout the attention kernels read q
+// from); k and v also go to page slot write_slot[m] when a cache is given.
+template <int MT>
+__global__ __launch_bounds__(256) void qkv_rope_append_kernel(
+    const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, bf16_t* __restrict__ qkv_out, int M, int K, int hq,
+    int hkv, int d, const int32_t* __restrict__ positions, const float2* __restrict__ table,
+    bf16_t* __restrict__ kv, const int32_t* __restrict__ write_slot) {
+  __shared__ f32x4 red[4][MT][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int half = d >> 1;
+  const int tiles_per_head = d >> 4;
+  const int head = blockIdx.x / tiles_per_head;
+  const int p = (blockIdx.x - head * tiles_per_head) << 3;          // first of 8 pair indices
+  const int row = head * d + (r < 8 ? p + r : half + p + r - 8);
+  const bf16_t* wrow = w + static_cast<int64_t>(row) * K + 8 * g;
+  const bf16_t* xrow[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) xrow[mt] = x + static_cast<int64_t>(min(mt * 16 + r, M - 1)) * K + 8 * g;
+  f32x4 acc[MT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int s_full = K >> 5;
+#pragma unroll 4
+  for (int s = wave; s < s_full; s += 4) {
+    const int k = s << 5;
+    const bf16x8 a = load8(wrow + k);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+      acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, load8(xrow[mt] + k), acc[mt], 0, 0, 0);
+  }
+  if ((K & 31) != 0 && (s_full & 3) == wave) {
+    const int k = s_full << 5;
+    const bool in = k + 8 * g < K;
+    const bf16x8 a = in ? load8(wrow + k) : zero8();
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const bf16x8 b = in ? load8(xrow[mt] + k) : zero8();
+      acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mt], 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < MT; ++i) red[wave][i][lane] = acc[i];
+  __syncthreads();
+  if (wave >= MT) return;
+  const int mt = wave;
+  const f32x4 own = red[0][mt][lane] + red[1][mt][lane] + red[2][mt][lane] + red[3][mt][lane];
+  const int m = mt * 16 + r;
+  const int mc = min(m, M - 1);
+  const bool second = g >= 2;
+  const bool rotate = table != nullptr && head < hq + hkv;
+  const int pos = positions[mc];
+  f32x4 res;
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    const float other = __shfl_xor(own[v], 32, kWave);              // the pair's other half
+    float val = own[v];
+    if (rotate) {
+      const float2 cs = table[static_cast<int64_t>(pos) * half + p + 4 * (g & 1) + v];
+      val = second ? own[v] * cs.x + other * cs.y : own[v] * cs.x - other * cs.y;
+    }
+    res[v] = val;
+  }
+  if (m >= M) return;
+  const int e0 = (second ? half : 0) + p + 4 * (g & 1);              // element of the head, 4 consecutive
+  ushort4 pk;
+  pk.x = float_to_bf16(res[0]);
+  pk.y = float_to_bf16(res[1]);
+  pk.z = float_to_bf16(res[2]);
+  pk.w = float_to_bf16(res[3]);
+  *reinterpret_cast<ushort4*>(qkv_out + static_cast<int64_t>(m) * ((hq + 2 * hkv) * d) + head * d + e0) = pk;
+  if (kv == nullptr || head < hq) return;
+  const int slot = write_slot[m];
+  const int64_t page_elems = 2LL * hkv * kPage * d;
+  bf16_t* page = kv + static_cast<int64_t>(slot / kPage) * page_elems;
+  const int off = slot % kPage;
+  if (head < hq + hkv) {                                             // key row [16][D]
+    *reinterpret_cast<ushort4*>(page + (static_cast<int64_t>(head - hq) * kPage + off) * d + e0) = pk;
+  } else {                                                           // value, transposed [D][16]
+    bf16_t* vp = page + static_cast<int64_t>(hkv) * kPage * d + (static_cast<int64_t>(head - hq - hkv) * d + e0) * kPage + off;
+    vp[0] = pk.x;
+    vp[kPage] = pk.y;
+    vp[2 * kPage] = pk.z;
+    vp[3 * kPage] = pk.w;
+  }
 }
 
 }  // namespace psamd
@@ -190,21 +298,53 @@ int psamd_linear(void* stream, const void* x, int x_dtype, const void* w, int w_
   return fail("psamd_linear: supported types are (f32,f32)->f32, (bf16,bf16)->bf16 and (bf16,bf16)->f32");
 }
 
-// out[M, n_out]; epilogue 0: n_out = rows of w; epilogue 1 (SwiGLU): w has 2 * n_out rows.
+// out[ksplit][M, n_out]; epilogue 0: n_out = rows of w; epilogue 1 (SwiGLU): w has 2 * n_out rows.
+// ksplit > 1 splits K over workgroups: out then holds ksplit float32 partial sums to be added.
 int psamd_linear_skinny(void* stream, const void* x, const void* w, void* out, int out_dtype, int M, int n_out, int K,
-                        int epilogue) {
+                        int epilogue, int ksplit) {
   PSAMD_REQUIRE(M >= 1 && M <= 64, "M must be in [1, 64]");
   PSAMD_REQUIRE(n_out > 0 && K > 0 && K % 8 == 0, "K must be a positive multiple of 8");
   PSAMD_REQUIRE(epilogue == 0 || epilogue == 1, "unknown epilogue");
   PSAMD_REQUIRE(out_dtype == kBF16 || out_dtype == kF32, "output must be bfloat16 or float32");
+  PSAMD_REQUIRE(epilogue == 0 || out_dtype == kBF16, "the SwiGLU epilogue writes bfloat16");
+  PSAMD_REQUIRE(ksplit >= 1 && ksplit <= 64, "ksplit must be in [1, 64]");
+  PSAMD_REQUIRE(ksplit == 1 || (epilogue == 0 && out_dtype == kF32), "partial sums are float32 and linear");
+  PSAMD_REQUIRE(ceil_div(n_out, 16) <= 2147483647LL, "too many columns");
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int mt = static_cast<int>(ceil_div(M, 16));
   switch (mt) {
-    case 1: return launch_skinny<1>(s, x, w, out, out_dtype, M, n_out, K, epilogue);
-    case 2: return launch_skinny<2>(s, x, w, out, out_dtype, M, n_out, K, epilogue);
-    case 3: return launch_skinny<3>(s, x, w, out, out_dtype, M, n_out, K, epilogue);
-    default: return launch_skinny<4>(s, x, w, out, out_dtype, M, n_out, K, epilogue);
+    case 1: return launch_skinny<1>(s, x, w, out, out_dtype, M, n_out, K, epilogue, ksplit);
+    case 2: return launch_skinny<2>(s, x, w, out, out_dtype, M, n_out, K, epilogue, ksplit);
+    case 3: return launch_skinny<3>(s, x, w, out, out_dtype, M, n_out, K, epilogue, ksplit);
+    default: return launch_skinny<4>(s, x, w, out, out_dtype, M, n_out, K, epilogue, ksplit);
   }
+}
+
+
+// qkv_out[M, (hq + 2 hkv) * d] = x[M, K] * w^T with q and k rotated by table[positions[m]] (NULL: no rotation);
+// k and v are also written to page slot write_slot[m] of kv (NULL: no cache write).
+int psamd_qkv_rope_append(void* stream, const void* x, const void* w, void* qkv_out, int M, int K, int hq, int hkv,
+                          int head_dim, const int32_t* positions, const float* table, void* kv,
+                          const int32_t* write_slot) {
+  PSAMD_REQUIRE(M >= 1 && M <= 64, "M must be in [1, 64]");
+  PSAMD_REQUIRE(K > 0 && K % 8 == 0, "K must be a positive multiple of 8");
+  PSAMD_REQUIRE(hq > 0 && hkv > 0 && head_dim >= 16 && head_dim % 16 == 0, "head_dim must be a multiple of 16");
+  PSAMD_REQUIRE(positions != nullptr, "positions are needed");
+  PSAMD_REQUIRE(kv == nullptr || write_slot != nullptr, "a cache needs write slots");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid(static_cast<unsigned>((hq + 2 * hkv) * (head_dim / 16))), block(256);
+  const bf16_t* xp = static_cast<const bf16_t*>(x);
+  const bf16_t* wp = static_cast<const bf16_t*>(w);
+  bf16_t* op = static_cast<bf16_t*>(qkv_out);
+  const float2* tab = reinterpret_cast<const float2*>(table);
+  bf16_t* kvp = static_cast<bf16_t*>(kv);
+  switch (static_cast<int>(ceil_div(M, 16))) {
+    case 1: qkv_rope_append_kernel<1><<<grid, block, 0, s>>>(xp, wp, op, M, K, hq, hkv, head_dim, positions, tab, kvp, write_slot); break;
+    case 2: qkv_rope_append_kernel<2><<<grid, block, 0, s>>>(xp, wp, op, M, K, hq, hkv, head_dim, positions, tab, kvp, write_slot); break;
+    case 3: qkv_rope_append_kernel<3><<<grid, block, 0, s>>>(xp, wp, op, M, K, hq, hkv, head_dim, positions, tab, kvp, write_slot); break;
+    default: qkv_rope_append_kernel<4><<<grid, block, 0, s>>>(xp, wp, op, M, K, hq, hkv, head_dim, positions, tab, kvp, write_slot); break;
+  }
+  return check_launch("psamd_qkv_rope_append");
 }
 
 }  // extern "C"

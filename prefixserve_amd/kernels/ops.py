@@ -39,11 +39,12 @@ def _ptr(t: torch.Tensor | None) -> int | None:
 
 _SIGNATURES = {
     "psamd_embed": [_vp, _vp, _vp, _i32, _vp, _i64, _i32],
-    "psamd_add_rmsnorm": [_vp, _vp, _vp, _vp, _vp, _i32, _f32, _vp, _i32, _i64, _i32],
+    "psamd_add_rmsnorm": [_vp, _vp, _vp, _i32, _i32, _i64, _vp, _vp, _i32, _f32, _vp, _i32, _i64, _i32],
     "psamd_swiglu": [_vp, _vp, _vp, _i32, _i64, _i32],
     "psamd_rope_kv_append": [_vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp, _vp, _vp, _vp],
     "psamd_linear": [_vp, _vp, _i32, _vp, _i32, _vp, _i32, _i64, _i32, _i32],
-    "psamd_linear_skinny": [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32],
+    "psamd_linear_skinny": [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32],
+    "psamd_qkv_rope_append": [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp],
     "psamd_attention_generic": [_vp, _vp, _i32, _vp, _vp, _i32, _i64, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _f32, _i32],
     "psamd_attention_mfma_supports": [_i32, _i32, _i32],
     "psamd_attention_prefill": [_vp, _vp, _i32, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _f32, _i32],
@@ -100,25 +101,37 @@ class HipOps:
         self._ok(self.lib.psamd_embed(self._stream(), ids.data_ptr(), table.data_ptr(), _code(table.dtype),
                                       out.data_ptr(), t, h))
 
+    def _delta_args(self, delta, t: int, h: int, out_dtype: torch.dtype) -> tuple:
+        """(pointer, dtype code, slices, stride) of a delta: [T, H] in the activation dtype, or
+        [S, T, H] float32 partial sums of a K-split product."""
+        if delta is None:
+            return None, _F32, 0, 0
+        self._need(delta.is_contiguous(), "delta must be contiguous")
+        if delta.dim() == 3:
+            self._need(delta.dtype == torch.float32 and delta.shape[1:] == (t, h), "partial sums must be float32 [S, T, H]")
+            return delta.data_ptr(), _F32, delta.shape[0], t * h
+        self._need(delta.shape == (t, h) and delta.dtype == out_dtype, "delta must match the output")
+        return delta.data_ptr(), _code(delta.dtype), 1, 0
+
     def add_rmsnorm(self, residual, delta, weight, eps: float, out) -> None:
         t, h = residual.shape
         self._need(residual.dtype == torch.float32 and residual.is_contiguous(), "add_rmsnorm: residual must be float32")
         self._need(out.shape == (t, h) and out.is_contiguous(), "add_rmsnorm: bad output shape")
-        self._need(delta is None or (delta.shape == (t, h) and delta.dtype == out.dtype and delta.is_contiguous()),
-                   "add_rmsnorm: delta must match the output")
         self._need(weight.numel() == h, "add_rmsnorm: weight size")
-        self._ok(self.lib.psamd_add_rmsnorm(self._stream(), residual.data_ptr(), _ptr(delta), None, weight.data_ptr(),
-                                            _code(weight.dtype), eps, out.data_ptr(), _code(out.dtype), t, h))
+        dptr, dcode, slices, stride = self._delta_args(delta, t, h, out.dtype)
+        self._ok(self.lib.psamd_add_rmsnorm(self._stream(), residual.data_ptr(), dptr, dcode, slices, stride, None,
+                                            weight.data_ptr(), _code(weight.dtype), eps, out.data_ptr(),
+                                            _code(out.dtype), t, h))
 
     def add_rmsnorm_rows(self, residual, delta, rows, weight, eps: float, out) -> None:
         t, h = residual.shape
         s = rows.numel()
         self._need(residual.dtype == torch.float32 and rows.dtype == torch.int32, "add_rmsnorm_rows: dtypes")
         self._need(out.shape == (s, h) and out.is_contiguous(), "add_rmsnorm_rows: bad output shape")
-        self._need(delta is None or (delta.shape == (t, h) and delta.dtype == out.dtype), "add_rmsnorm_rows: delta")
-        self._ok(self.lib.psamd_add_rmsnorm(self._stream(), residual.data_ptr(), _ptr(delta), rows.data_ptr(),
-                                            weight.data_ptr(), _code(weight.dtype), eps, out.data_ptr(),
-                                            _code(out.dtype), s, h))
+        dptr, dcode, slices, stride = self._delta_args(delta, t, h, out.dtype)
+        self._ok(self.lib.psamd_add_rmsnorm(self._stream(), residual.data_ptr(), dptr, dcode, slices, stride,
+                                            rows.data_ptr(), weight.data_ptr(), _code(weight.dtype), eps,
+                                            out.data_ptr(), _code(out.dtype), s, h))
 
     def swiglu(self, gate_up, out) -> None:
         t, inter = out.shape
@@ -140,6 +153,28 @@ class HipOps:
                                                positions.data_ptr(), _ptr(table), _ptr(kv),
                                                None if kv is None else write_slot.data_ptr()))
 
+    def qkv_rope_append(self, x, w_qkv, qkv, hq: int, hkv: int, d: int, positions, table, kv, write_slot) -> None:
+        """qkv = x @ w_qkv^T, q and k rotated, k and v written to their pages. One kernel for a
+        bfloat16 step of at most 64 tokens; otherwise the product followed by ``rope_kv_append``."""
+        m, k = x.shape
+        if (x.dtype == torch.bfloat16 and 0 < m <= self.SKINNY_MAX_ROWS and k % 8 == 0 and d % 16 == 0):
+            self._need(w_qkv.shape == ((hq + 2 * hkv) * d, k) and qkv.shape == (m, (hq + 2 * hkv) * d), "qkv: shapes")
+            self._need(x.is_contiguous() and w_qkv.is_contiguous() and qkv.is_contiguous(), "qkv: contiguous operands")
+            self._need(positions.dtype == torch.int32 and positions.numel() == m, "qkv: positions")
+            if table is not None:
+                self._need(table.dtype == torch.float32 and table.shape[1:] == (d // 2, 2) and table.is_contiguous(),
+                           "qkv: table must be float32 [positions, D/2, 2]")
+            if kv is not None:
+                self._need(kv.dtype == qkv.dtype and kv.shape[1:] == (2, hkv, 16 * d) and kv.is_contiguous(),
+                           "qkv: cache must be [blocks, 2, kv_heads, 16*D] in the activation dtype")
+                self._need(write_slot.dtype == torch.int32 and write_slot.numel() == m, "qkv: write slots")
+            self._ok(self.lib.psamd_qkv_rope_append(self._stream(), x.data_ptr(), w_qkv.data_ptr(), qkv.data_ptr(), m, k,
+                                                    hq, hkv, d, positions.data_ptr(), _ptr(table), _ptr(kv),
+                                                    None if kv is None else write_slot.data_ptr()))
+            return
+        self.linear(x, w_qkv, qkv)
+        self.rope_kv_append(qkv, hq, hkv, d, positions, table, kv, write_slot)
+
     # ---------------------------------------------------------------- products
 
     def linear(self, x, w, out) -> None:
@@ -157,13 +192,33 @@ class HipOps:
                 for r0 in range(0, m, self.SKINNY_MAX_ROWS):
                     r1 = min(m, r0 + self.SKINNY_MAX_ROWS)
                     self._ok(self.lib.psamd_linear_skinny(self._stream(), x[r0:r1].data_ptr(), w.data_ptr(),
-                                                          out[r0:r1].data_ptr(), _code(out.dtype), r1 - r0, n, k, 0))
+                                                          out[r0:r1].data_ptr(), _code(out.dtype), r1 - r0, n, k, 0, 1))
                 return
             if out.dtype == torch.bfloat16:
                 torch.matmul(x, w.t(), out=out)   # library product, as in the reference
                 return
         self._ok(self.lib.psamd_linear(self._stream(), x.data_ptr(), _code(x.dtype), w.data_ptr(), _code(w.dtype),
                                        out.data_ptr(), _code(out.dtype), m, n, k))
+
+    def linear_to_residual(self, x, w, name: str) -> torch.Tensor:
+        """x @ w^T for a consumer that adds it to the residual stream (the fused add+norm).
+        Returns [T, N] in the activation dtype or, for a small bfloat16 step whose product has
+        few output columns, [S, T, N] float32 partial sums of a K-split, which the consumer adds
+        up: splitting K over workgroups is what lets such a product use the whole chip."""
+        m, k = x.shape
+        n = w.shape[0]
+        if x.dtype == torch.bfloat16 and k % 8 == 0 and 0 < m <= self.SKINNY_MAX_ROWS:
+            tiles, steps = -(-n // 16), -(-k // 32)
+            ksplit = max(1, min(8, 512 // tiles, steps // 8))
+            if ksplit > 1:
+                self._need(w.shape[1] == k and x.is_contiguous() and w.is_contiguous(), "linear_to_residual: operands")
+                out = self.ws.get(name, (ksplit, m, n), torch.float32)
+                self._ok(self.lib.psamd_linear_skinny(self._stream(), x.data_ptr(), w.data_ptr(), out.data_ptr(),
+                                                      _F32, m, n, k, 0, ksplit))
+                return out
+        out = self.ws.get(name, (m, n), x.dtype)
+        self.linear(x, w, out)
+        return out
 
     def linear_swiglu(self, x, w_gate_up, out) -> None:
         m, k = x.shape
@@ -173,7 +228,7 @@ class HipOps:
             return
         if x.dtype == torch.bfloat16 and k % 8 == 0 and m <= self.SKINNY_MAX_ROWS:
             self._ok(self.lib.psamd_linear_skinny(self._stream(), x.data_ptr(), w_gate_up.data_ptr(), out.data_ptr(),
-                                                  _BF16, m, inter, k, 1))
+                                                  _BF16, m, inter, k, 1, 1))
             return
         gu = self.ws.get("mlp.gate_up", (m, 2 * inter), x.dtype)
         self.linear(x, w_gate_up, gu)
@@ -210,8 +265,9 @@ class HipOps:
                 part_ml = self.ws.get("attn.part_ml", (ctx.num_decode * hq * nsplit * 2,), torch.float32)
                 self._ok(self.lib.psamd_attention_decode(
                     s, qkv.data_ptr(), stride, out.data_ptr(), kv.data_ptr(), part_o.data_ptr(), part_ml.data_ptr(),
-                    ctx.dec_items.data_ptr(), ctx.num_decode, ctx.item_start.data_ptr(), ctx.item_end.data_ptr(),
-                    g.table_off.data_ptr(), g.block_ids.data_ptr(), hq, hkv, d, nsplit, scale, win))
+                    ctx.dec_items.data_ptr(), ctx.num_decode, ctx.item_start.data_ptr(),
+                    ctx.item_end.data_ptr(), g.table_off.data_ptr(), g.block_ids.data_ptr(), hq, hkv, d, nsplit, scale,
+                    win))
             return
         self._ok(self.lib.psamd_attention_generic(
             s, qkv.data_ptr(), stride, out.data_ptr(), kv.data_ptr(), _code(qkv.dtype), t, ctx.positions.data_ptr(),

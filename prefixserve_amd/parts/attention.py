@@ -85,16 +85,13 @@ class PagedAttention(Mixer):
         rt, ops, ws = self.rt, self.rt.ops, self.rt.workspace
         t = x.shape[0]
         qkv = ws.get("attn.qkv", (t, self.q_size + 2 * self.kv_size), rt.dtype)
-        ops.linear(x, self.w_qkv, qkv)
         table = self.pos.table if self.pos is not None else None
-        ops.rope_kv_append(qkv, self.num_heads, self.num_kv_heads, self.head_dim, ctx.positions, table,
-                           cache.kv if writes_cache else None, ctx.groups[cache.group].write_slot)
+        ops.qkv_rope_append(x, self.w_qkv, qkv, self.num_heads, self.num_kv_heads, self.head_dim, ctx.positions, table,
+                            cache.kv if writes_cache else None, ctx.groups[cache.group].write_slot)
         out = ws.get("attn.out", (t, self.q_size), rt.dtype)
         ops.paged_attention(qkv, out, cache.kv, ctx, cache.group, self.num_heads, self.num_kv_heads,
                             self.head_dim, self.scale, cache.window)
-        delta = ws.get("attn.delta", (t, self.hidden_size), rt.dtype)
-        ops.linear(out, self.w_o, delta)
-        return delta
+        return ops.linear_to_residual(out, self.w_o, "attn.delta")
 
 
 register_mixer("paged_attention", PagedAttention)

@@ -70,6 +70,15 @@ class Workspace:
             self.version += 1
         return buf[:n].view(*shape)
 
+    def get_zeroed(self, name: str, shape: tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
+        """Like ``get``, but the buffer is zero when first handed out or after it grew. Users
+        that need zeros on every call must leave the buffer zero themselves."""
+        before = self.version
+        out = self.get(name, shape, dtype)
+        if self.version != before:
+            self._bufs[name].zero_()
+        return out
+
     def nbytes(self) -> int:
         return sum(b.numel() * b.element_size() for b in self._bufs.values())
 
@@ -107,7 +116,8 @@ class Norm(Part):
 
     def add_norm(self, residual: torch.Tensor, delta: torch.Tensor | None, out_name: str) -> torch.Tensor:
         """residual (float32 [T,H], updated in place) += delta; returns norm(residual) in the
-        activation dtype. The sum and the statistics are 32-bit."""
+        activation dtype. ``delta`` is [T,H] or [S,T,H] float32 slices to be summed. The sum and
+        the statistics are 32-bit."""
         raise NotImplementedError
 
     def add_norm_rows(self, residual: torch.Tensor, delta: torch.Tensor | None, rows: torch.Tensor,
@@ -134,8 +144,9 @@ class Mixer(Part):
 
     def forward(self, x: torch.Tensor, ctx: "StepContext", cache: Any, state: torch.Tensor | None,
                 writes_cache: bool) -> torch.Tensor:
-        """x [T, hidden] (activation dtype) -> [T, hidden] to be added to the residual.
-        ``cache`` is this run's ``LayerCache`` (pages of its group) or None; ``state`` is
+        """x [T, hidden] (activation dtype) -> what is to be added to the residual: [T, hidden]
+        in the activation dtype, or [S, T, hidden] float32 slices whose sum it is (what
+        ``ops.linear_to_residual`` returns). ``cache`` is this run's ``LayerCache`` (pages of its group) or None; ``state`` is
         ``[num_slots, *shape]`` or None, indexed by ``ctx.slots``."""
         raise NotImplementedError
 

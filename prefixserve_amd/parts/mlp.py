@@ -40,9 +40,7 @@ class SwiGLU(FeedForward):
         t = x.shape[0]
         act = ws.get("mlp.act", (t, self.intermediate_size), rt.dtype)
         ops.linear_swiglu(x, self.w_gate_up, act)
-        delta = ws.get("mlp.delta", (t, self.hidden_size), rt.dtype)
-        ops.linear(act, self.w_down, delta)
-        return delta
+        return ops.linear_to_residual(act, self.w_down, "mlp.delta")
 
 
 register_feed_forward("swiglu", SwiGLU)

@@ -48,3 +48,23 @@ def plain_models(model_dirs: dict[str, Path]) -> dict:
     from plain.llama_plain import PlainLlama
 
     return {name: PlainLlama(d) for name, d in model_dirs.items()}
+
+
+@pytest.fixture(scope="session")
+def plain_bf16_error(model_dirs: dict[str, Path], plain_models: dict) -> dict[str, float]:
+    """The yardstick for bfloat16: the mean error (per row, relative to the row's largest
+    logit) of the plain model when every operation's result is rounded to bfloat16, against
+    the plain model in float64. The reference accepts its bfloat16 engine when it is no worse
+    than 1.5x a plain bfloat16 run (tests/gpu/test_engine_flashinfer.py:104-108)."""
+    import numpy as np
+
+    from configs import TINY
+    from plain.llama_plain import PlainLlama
+
+    out = {}
+    for name, d in model_dirs.items():
+        toks = np.random.default_rng(77).integers(0, TINY[name]["vocab_size"], 130).tolist()
+        truth = plain_models[name].logits(toks)
+        rough = PlainLlama(d, bf16=True).logits(toks)
+        out[name] = float(np.mean(np.abs(rough - truth).max(-1) / np.abs(truth).max(-1)))
+    return out

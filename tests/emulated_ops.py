@@ -43,10 +43,19 @@ class EmulatedOps:
     def linear(self, x, w, out) -> None:
         out.copy_((x.float() @ w.float().T).to(out.dtype))
 
+    def linear_to_residual(self, x, w, name):
+        out = self.ws.get(name, (x.shape[0], w.shape[0]), x.dtype)
+        self.linear(x, w, out)
+        return out
+
     def linear_swiglu(self, x, w_gate_up, out) -> None:
         gu = x.float() @ w_gate_up.float().T
         inter = gu.shape[1] // 2
         out.copy_((torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:]).to(out.dtype))
+
+    def qkv_rope_append(self, x, w_qkv, qkv, hq, hkv, d, positions, table, kv, write_slot) -> None:
+        self.linear(x, w_qkv, qkv)
+        self.rope_kv_append(qkv, hq, hkv, d, positions, table, kv, write_slot)
 
     def rope_kv_append(self, qkv, hq, hkv, d, positions, table, kv, write_slot) -> None:
         t = qkv.shape[0]

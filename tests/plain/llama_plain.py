@@ -166,21 +166,77 @@ def swiglu_mlp(x: np.ndarray, w_gate: np.ndarray, w_up: np.ndarray, w_down: np.n
     return (silu(x @ w_gate.T) * (x @ w_up.T)) @ w_down.T
 
 
+def round_bf16(x: np.ndarray) -> np.ndarray:
+    """Rounds to the nearest bfloat16 (ties to even) and returns the values widened again."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    r = ((u >> 16) & 1) + np.uint32(0x7FFF)
+    return ((u + r) & np.uint32(0xFFFF0000)).view(np.float32)
+
+
 # ---------------------------------------------------------------------- model
 
 
 class PlainLlama:
     """Whole-sequence forward from a model folder (config.json + model.safetensors)."""
 
-    def __init__(self, model_dir: str | Path, dtype: Any = np.float64) -> None:
+    def __init__(self, model_dir: str | Path, dtype: Any = np.float64, bf16: bool = False) -> None:
+        """``bf16``: round the result of every operation to bfloat16, as a library that runs
+        the reference's model code in bfloat16 does (prefixserve/model/llama.py:105-126 with
+        dtype=bfloat16; softmax and the norm's statistics stay float32, llama.py:63-69 and
+        prefixserve/model/attention.py:119). It is the yardstick for the engine's bfloat16 error."""
         model_dir = Path(model_dir)
         self.cfg = PlainConfig(json.loads((model_dir / "config.json").read_text()))
+        self.bf16 = bf16
+        if bf16:
+            dtype = np.float32
         self.dtype = dtype
         self.w = {k: v.astype(dtype) for k, v in read_safetensors(model_dir / "model.safetensors").items()}
         self.inv_freq = rope_inv_freq(self.cfg.head_dim, self.cfg.theta, self.cfg.scaling)
 
+    def _r(self, x: np.ndarray) -> np.ndarray:
+        return round_bf16(x) if self.bf16 else x
+
+    def _layer_bf16(self, i: int, h: np.ndarray, cos: np.ndarray, sin: np.ndarray) -> np.ndarray:
+        """The same layer with every operation's result rounded to bfloat16."""
+        c, w, r = self.cfg, self.w, round_bf16
+        p = f"model.layers.{i}."
+        n = h.shape[0]
+
+        def norm(x: np.ndarray, weight: np.ndarray) -> np.ndarray:
+            xf = x / np.sqrt(np.mean(x * x, axis=-1, keepdims=True) + np.float32(c.eps))
+            return r(weight * r(xf))
+
+        def rope(x: np.ndarray) -> np.ndarray:
+            half = x.shape[-1] // 2
+            rot = np.concatenate([-x[..., half:], x[..., :half]], axis=-1)
+            return r(r(x * cos[:, None, :]) + r(rot * sin[:, None, :]))
+
+        x = norm(h, w[p + "input_layernorm.weight"])
+        q = rope(r(x @ w[p + "self_attn.q_proj.weight"].T).reshape(n, c.heads, c.head_dim))
+        k = rope(r(x @ w[p + "self_attn.k_proj.weight"].T).reshape(n, c.kv_heads, c.head_dim))
+        v = r(x @ w[p + "self_attn.v_proj.weight"].T).reshape(n, c.kv_heads, c.head_dim)
+        group = c.heads // c.kv_heads
+        scale = np.float32(1.0 / math.sqrt(c.head_dim))
+        pos = np.arange(n)
+        masked = pos[None, :] > pos[:, None]
+        o = np.empty_like(q)
+        for hd in range(c.heads):
+            s = r(r(q[:, hd, :] @ k[:, hd // group, :].T) * scale)
+            s = np.where(masked, -np.inf, s)
+            e = np.exp(s - s.max(axis=-1, keepdims=True))
+            pr = r(e / e.sum(axis=-1, keepdims=True))
+            o[:, hd, :] = r(pr @ v[:, hd // group, :])
+        h = r(h + r(o.reshape(n, -1) @ w[p + "self_attn.o_proj.weight"].T))
+        x = norm(h, w[p + "post_attention_layernorm.weight"])
+        g = r(x @ w[p + "mlp.gate_proj.weight"].T)
+        u = r(x @ w[p + "mlp.up_proj.weight"].T)
+        act = r(r(g / (1.0 + np.exp(-g))) * u)
+        return r(h + r(act @ w[p + "mlp.down_proj.weight"].T))
+
     def layer(self, i: int, h: np.ndarray, cos: np.ndarray, sin: np.ndarray, window: int | None = None) -> np.ndarray:
         """One decoder layer in the reference's order (prefixserve/model/llama.py:111-121)."""
+        if self.bf16:
+            return self._layer_bf16(i, h, self._r(cos), self._r(sin))
         c, w = self.cfg, self.w
         p = f"model.layers.{i}."
         n = h.shape[0]
@@ -207,9 +263,12 @@ class PlainLlama:
     def logits(self, tokens: Any, first_position: int = 0) -> np.ndarray:
         """Logits at every position, [n, vocab] (prefixserve/model/llama.py:123-126);
         the head is the embedding table when tied (prefixserve/model/weights.py:133-136)."""
-        h = rms_norm(self.hidden(tokens, first_position), self.w["model.norm.weight"], self.cfg.eps)
+        h = self.hidden(tokens, first_position)
         head = self.w["model.embed_tokens.weight"] if self.cfg.tied else self.w["lm_head.weight"]
-        return h @ head.T
+        if self.bf16:
+            xf = h / np.sqrt(np.mean(h * h, axis=-1, keepdims=True) + np.float32(self.cfg.eps))
+            return round_bf16(round_bf16(self.w["model.norm.weight"] * round_bf16(xf)) @ head.T)
+        return rms_norm(h, self.w["model.norm.weight"], self.cfg.eps) @ head.T
 
     def greedy(self, prompt: Any, steps: int) -> tuple[list[int], list[np.ndarray]]:
         """Greedy generation by recomputing the whole sequence each step, as the

@@ -69,6 +69,25 @@ def test_add_rmsnorm(ops, act, wdt, hidden):
     assert torch.equal(r3, res) and rel(out3, want[rows.long()]) < (1e-6 if act == torch.float32 else 5e-3)
 
 
+@pytest.mark.parametrize("hidden", [96, 2048, 5000])
+def test_add_rmsnorm_sums_partial_slices(ops, hidden):
+    t, eps = 5, 1e-6
+    res = rnd(t, hidden, seed=1)
+    parts = rnd(3, t, hidden, seed=2)
+    w = (1 + 0.1 * rnd(hidden, seed=3)).to(torch.bfloat16)
+    want_res = res + parts[0] + parts[1] + parts[2]
+    want = w.float() * want_res * torch.rsqrt((want_res ** 2).mean(-1, keepdim=True) + eps)
+    out = torch.empty(t, hidden, dtype=torch.bfloat16, device=DEV)
+    r = res.clone()
+    ops.add_rmsnorm(r, parts, w, eps, out)
+    assert torch.equal(r, want_res) and rel(out, want) < 5e-3
+    rows = torch.tensor([4, 1], dtype=torch.int32, device=DEV)
+    out2 = torch.empty(2, hidden, dtype=torch.bfloat16, device=DEV)
+    r2 = res.clone()
+    ops.add_rmsnorm_rows(r2, parts, rows, w, eps, out2)
+    assert torch.equal(r2, res) and rel(out2, want[rows.long()]) < 5e-3
+
+
 def test_rmsnorm_zero_row_and_eps(ops):
     res = torch.zeros(2, 64, device=DEV)
     res[1] = 1e-4
@@ -123,6 +142,47 @@ def test_rope_kv_append(ops, act, hq, hkv, d):
     assert torch.equal(q2.float(), src.to(act).float())
 
 
+@pytest.mark.parametrize("m", [1, 8, 17, 64])
+@pytest.mark.parametrize("hq,hkv,d,k", [(6, 3, 48, 72), (4, 2, 16, 64), (32, 8, 64, 2048), (3, 1, 32, 96), (2, 2, 128, 200)])
+def test_fused_qkv_rope_append_equals_the_separate_kernels(ops, m, hq, hkv, d, k):
+    """One kernel for projection + rotation + cache write (small steps) against the product
+    followed by rope_kv_append, and against float64."""
+    from prefixserve_amd.parts.rope import rope_inv_freq
+
+    blocks = 12
+    x = rnd(m, k, dtype=torch.bfloat16, seed=1)
+    w = rnd((hq + 2 * hkv) * d, k, dtype=torch.bfloat16, seed=2, scale=0.1)
+    pos = torch.tensor([(7 * i + 3) % 150 for i in range(m)], dtype=torch.int32, device=DEV)
+    slots = torch.tensor(np.random.default_rng(m).permutation(blocks * 16)[:m].tolist(), dtype=torch.int32, device=DEV)
+    ang = torch.outer(torch.arange(150, dtype=torch.float32), rope_inv_freq(d, 10000.0, None)).double()
+    table = torch.stack((ang.cos(), ang.sin()), -1).float().to(DEV).contiguous()
+    n = (hq + 2 * hkv) * d
+    kv_a = torch.full((blocks, 2, hkv, 16 * d), 3.0, dtype=torch.bfloat16, device=DEV)
+    kv_b = kv_a.clone()
+    fused = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+    ops.qkv_rope_append(x, w, fused, hq, hkv, d, pos, table, kv_a, slots)
+    plain = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+    ops.linear(x, w, plain)
+    ops.rope_kv_append(plain, hq, hkv, d, pos, table, kv_b, slots)
+    # float64 truth
+    y = (x.double() @ w.double().T)
+    z = y[:, : (hq + hkv) * d].view(m, hq + hkv, d)
+    cs = table[pos.long()].double()
+    cos, sin = cs[..., 0][:, None], cs[..., 1][:, None]
+    z1, z2 = z[..., : d // 2], z[..., d // 2:]
+    want = torch.cat((torch.cat((z1 * cos - z2 * sin, z2 * cos + z1 * sin), -1).reshape(m, -1), y[:, (hq + hkv) * d:]), 1)
+    assert rel(fused, want) < 5e-3 and rel(plain, want) < 1e-2
+    page, off = (slots // 16).long(), (slots % 16).long()
+    kp = kv_a[:, 0].view(blocks, hkv, 16, d)
+    vp = kv_a[:, 1].view(blocks, hkv, d, 16)
+    assert torch.equal(kp[page, :, off, :].reshape(m, -1), fused[:, hq * d:(hq + hkv) * d])      # pages hold what q/k/v hold
+    assert torch.equal(vp[page, :, :, off].reshape(m, -1), fused[:, (hq + hkv) * d:])
+    assert rel(kv_a.float(), kv_b.float()) < 1e-2
+    touched = torch.zeros(blocks, 16, dtype=torch.bool, device=DEV)
+    touched[page, off] = True
+    assert torch.all(kp.permute(0, 2, 1, 3)[~touched] == 3.0) and torch.all(vp.permute(0, 3, 1, 2)[~touched] == 3.0)
+
+
 # --------------------------------------------------------------------- products
 
 @pytest.mark.parametrize("m,n,k", [(1, 100, 72), (3, 64, 16), (17, 257, 96), (130, 70, 200), (64, 128, 64)])
@@ -143,6 +203,17 @@ def test_linear_bf16_small_m(ops, m, n, k, out_dtype):
     ops.linear(x, w, out)
     want = x.double() @ w.double().T
     assert rel(out, want) < (1e-5 if out_dtype == torch.float32 else 5e-3)
+
+
+@pytest.mark.parametrize("m", [1, 8, 33, 64])
+@pytest.mark.parametrize("n,k", [(2048, 2048), (200, 8192), (72, 520), (256, 688)])
+def test_linear_to_residual_splits_k(ops, m, n, k):
+    x, w = rnd(m, k, dtype=torch.bfloat16, seed=1), rnd(n, k, dtype=torch.bfloat16, seed=2, scale=0.05)
+    out = ops.linear_to_residual(x, w, "test.delta")
+    assert out.dim() == 3 and out.dtype == torch.float32 and out.shape[0] > 1      # these shapes do split
+    assert rel(out.sum(0), x.double() @ w.double().T) < 1e-5
+    small = ops.linear_to_residual(x[:, :64].contiguous(), w[:, :64].contiguous(), "test.delta2")
+    assert small.dim() == 2 and small.dtype == torch.bfloat16                      # too little K to split
 
 
 @pytest.mark.parametrize("m,n,k", [(65, 300, 96), (200, 64, 2048), (3, 50, 70)])

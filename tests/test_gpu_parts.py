@@ -76,7 +76,8 @@ def test_swiglu_part(dtype):
     for t in (3, 100):
         x = torch.randn(t, 72, device=DEV).to(dtype)
         want = P.swiglu_mlp(x.float().cpu().double().numpy(), *(w[k].double().numpy() for k in "gud"))
-        assert rel(part.forward(x, None), want) < TOL[dtype]
+        o = part.forward(x, None)
+        assert rel(o.sum(0) if o.dim() == 3 else o, want) < TOL[dtype]
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -114,7 +115,8 @@ def test_attention_part_whole_and_in_portions(dtype, hq, hkv, d):
         outs, p0 = [], 0
         for c in cuts:
             ctx = pk.pack([StepItem("a", [1] * c, p0, [table])])
-            outs.append(part.forward(x[p0:p0 + c].contiguous(), ctx, cache, None, True).clone())
+            o = part.forward(x[p0:p0 + c].contiguous(), ctx, cache, None, True)
+            outs.append(o.sum(0) if o.dim() == 3 else o.float().clone())   # float32 slices of a K-split
             p0 += c
         assert rel(torch.cat(outs), want) < TOL[dtype] * 2
 

@@ -39,28 +39,31 @@ def runner_for(model_dir, dtype, num_blocks, graphs=True, max_seq_len=256):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B", "C"])
-def test_every_cutting_matches_the_plain_model(name, dtype, model_dirs, plain_models):
+def test_every_cutting_matches_the_plain_model(name, dtype, model_dirs, plain_models, plain_bf16_error):
     reqs = requests_for(name)
     truth = [plain_models[name].logits(t) for t in reqs]
     runner = runner_for(model_dirs[name], dtype, 64)
-    worst = {}
+    worst, errors = {}, []
     for build in (traces.whole, traces.decode_tail, traces.portions):
         steps, expect = build(reqs)
-        worst[build.__name__] = traces.compare(TraceReplayer(runner).run_step, steps, expect, truth, TOL[dtype])
+        worst[build.__name__] = traces.compare(TraceReplayer(runner).run_step, steps, expect, truth, TOL[dtype], errors)
     steps, expect, peak = traces.mixed(reqs, seed=3)
     assert sum(len(r) for r in reqs) > 1.5 * peak
     small = runner_for(model_dirs[name], dtype, peak // 16)
     small.pools.tensors[0].fill_(1e30)                              # a reused page never holds zeros
     rp = TraceReplayer(small)
-    worst["mixed"] = traces.compare(rp.run_step, steps, expect, truth, TOL[dtype])
+    worst["mixed"] = traces.compare(rp.run_step, steps, expect, truth, TOL[dtype], errors)
     assert rp.cache.num_free(0) == peak // 16
-    print(name, dtype, {k: f"{v:.2e}" for k, v in worst.items()})
+    print(name, dtype, {k: f"{v:.2e}" for k, v in worst.items()}, f"mean {np.mean(errors):.2e}")
     if dtype == "float32":
         assert max(worst.values()) < 2e-5                           # well inside the bar
+    else:
+        # no worse than a plain bfloat16 run of the same model (the reference allows 1.5x)
+        assert np.mean(errors) <= plain_bf16_error[name], f"{np.mean(errors):.3e} > {plain_bf16_error[name]:.3e}"
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_cuttings_agree_with_each_other(dtype, model_dirs):
+def test_cuttings_agree_with_each_other(dtype, model_dirs, plain_bf16_error):
     """Whatever the distance to the plain model, the engine must agree with itself: the same
     position's logits from a whole prompt, from a decode step and from a mixed batch differ
     by rounding only."""
@@ -76,12 +79,20 @@ def test_cuttings_agree_with_each_other(dtype, model_dirs):
             for row, key in zip(out if out is not None else [], ex):
                 got[key] = row
         rows[build.__name__] = got
-    tol = 1e-5 if dtype == "float32" else 3e-2
+    # Each cutting is within TOL of the plain model, so two cuttings are within 2 * TOL of each
+    # other: the only bound that follows for the worst row. The typical row must agree at
+    # least as well as a plain bfloat16 run agrees with the truth.
+    worst_tol = 1e-5 if dtype == "float32" else 2 * TOL_BF16
+    median_tol = 2e-6 if dtype == "float32" else plain_bf16_error["C"]
+    errs = []
     for key, ref in rows["whole"].items():
         for other in ("decode_tail", "portions"):
             if key in rows[other]:
-                err = np.abs(rows[other][key] - ref).max() / np.abs(ref).max()
-                assert err < tol, f"{other} vs whole at {key}: {err:.3e}"
+                err = float(np.abs(rows[other][key] - ref).max() / np.abs(ref).max())
+                assert err < worst_tol, f"{other} vs whole at {key}: {err:.3e}"
+                errs.append(err)
+    assert len(errs) > 250 and float(np.median(errs)) < median_tol, f"median {np.median(errs):.3e}"
+    print(dtype, f"cuttings against each other: worst {max(errs):.2e}, median {np.median(errs):.2e}")
 
 
 def test_graph_replay_equals_eager_decoding(model_dirs):

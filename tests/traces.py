@@ -94,9 +94,9 @@ def mixed(reqs: Sequence[Sequence[int]], max_live: int = 4, seed: int = 0, promp
     return steps, expect, peak
 
 
-def compare(run_step, steps: Steps, expect: Expect, truth: Sequence, tol: float) -> float:
+def compare(run_step, steps: Steps, expect: Expect, truth: Sequence, tol: float, errors: list | None = None) -> float:
     """Runs the steps and checks every row against ``truth[req][pos]``. Returns the worst
-    relative error; fails naming the first wrong place."""
+    relative error (and appends every row's to ``errors``); fails naming the first wrong place."""
     import numpy as np
 
     worst = 0.0
@@ -113,4 +113,6 @@ def compare(run_step, steps: Steps, expect: Expect, truth: Sequence, tol: float)
                 f"step {step['step']}: request {i} position {p}: relative error {err:.3e} > {tol:.1e} "
                 f"(entries {[(e['id'], len(e['tokens'])) for e in step['entries']]})")
             worst = max(worst, err)
+            if errors is not None:
+                errors.append(err)
     return worst
