@@ -87,24 +87,31 @@ __device__ __forceinline__ bf16x8 zero8() {
 
 __device__ __forceinline__ float silu_f(float g) { return g / (1.f + __expf(-g)); }
 
-// One workgroup (4 waves) owns 16 output columns (rows of w) and a range of K; its waves
-// take the 32-wide k-steps of that range in turn, so together they stream 256 contiguous
-// bytes of each row per round, and their partial tiles are summed through LDS. With
-// gridDim.y > 1 the K range is also split over workgroups and the float partial sums go to
-// out[blockIdx.y][M][n_out] for the consumer (the fused add+norm) to add up: that is how a
-// product with few output columns still fills the chip.
+// Streams rows of w through v_mfma_f32_16x16x32_bf16 with the M tokens as the other operand.
+// Two ways to lay the work over a workgroup's 4 waves:
+//  * SPLIT (few output columns): the workgroup owns 16 rows of w and a range of K; its waves
+//    take the 32-wide k-steps of that range in turn and their partial tiles are summed
+//    through LDS. With gridDim.y > 1 the K range is also split over workgroups and float
+//    partial sums go to out[blockIdx.y][M][n_out] for the consumer (the fused add+norm) to add
+//    up: that is how a product with few output columns still fills the chip.
+//  * !SPLIT (many output columns): every wave owns 16 rows of its own over all of K; the 4
+//    waves read the same tokens at the same time, so x comes from L1 rather than L2.
+// Loads are issued U steps ahead of the matrix instructions that use them: the kernel is
+// bound by memory latency unless many loads are in flight.
 //
-// Operand layout of v_mfma_f32_16x16x32_bf16: lane l supplies row (l % 16), k = 8 * (l / 16)
-// + [0, 8) of both operands and receives C[4 * (l / 16) + v][l % 16], v = 0..3; C rows are
-// rows of w, C columns are tokens. MT = number of 16-token column tiles. SWIGLU: w is
-// [gate; up] with n_out rows each and the result is silu(gate) * up.
-template <int MT, bool SWIGLU, typename TO>
+// Operand layout: lane l supplies row (l % 16), k = 8 * (l / 16) + [0, 8) of both operands
+// and receives C[4 * (l / 16) + v][l % 16], v = 0..3; C rows are rows of w, C columns are
+// tokens. MT = number of 16-token column tiles. SWIGLU: w is [gate; up] with n_out rows each
+// and the result is silu(gate) * up.
+template <int MT, bool SWIGLU, bool SPLIT, typename TO>
 __global__ __launch_bounds__(256) void skinny_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                           TO* __restrict__ out, int M, int n_out, int K) {
   constexpr int NACC = SWIGLU ? 2 * MT : MT;
-  __shared__ f32x4 red[4][NACC][64];
+  constexpr int U = MT == 1 ? 8 : (MT == 2 ? 4 : 2);
+  __shared__ f32x4 red[SPLIT ? 4 : 1][NACC][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int n0 = blockIdx.x * 16;
+  const int n0 = SPLIT ? blockIdx.x * 16 : (blockIdx.x * 4 + wave) * 16;
+  if (!SPLIT && n0 >= n_out) return;
   const int r = lane & 15, g = lane >> 4;
   const int row = min(n0 + r, n_out - 1);
   const bf16_t* wrow = w + static_cast<int64_t>(row) * K + 8 * g;
@@ -122,21 +129,36 @@ __global__ __launch_bounds__(256) void skinny_mfma_kernel(const bf16_t* __restri
   const int s_begin = blockIdx.y * per_wg;
   const int s_end = min(s_begin + per_wg, steps);
   const int s_full = min(s_end, K >> 5);          // steps that lie wholly inside K
-#pragma unroll 4
-  for (int s = s_begin + wave; s < s_full; s += 4) {
-    const int k = s << 5;
-    const bf16x8 a = load8(wrow + k);
-    bf16x8 a_up;
-    if (SWIGLU) a_up = load8(wrow_up + k);
+  const int stride = SPLIT ? 4 : 1;
+  for (int base = s_begin + (SPLIT ? wave : 0); base < s_full; base += stride * U) {
+    bf16x8 a[U], a_up[U], b[MT][U];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const bf16x8 b = load8(xrow[mt] + k);
-      acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mt], 0, 0, 0);
-      if (SWIGLU) acc[MT + mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_up, b, acc[MT + mt], 0, 0, 0);
+    for (int u = 0; u < U; ++u) {
+      const int s = base + stride * u;
+      if (s < s_full) {
+        const int k = s << 5;
+        a[u] = load8(wrow + k);
+        if (SWIGLU) a_up[u] = load8(wrow_up + k);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) b[mt][u] = load8(xrow[mt] + k);
+      } else {
+        a[u] = zero8();
+        if (SWIGLU) a_up[u] = zero8();
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) b[mt][u] = zero8();
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b[mt][u], acc[mt], 0, 0, 0);
+        if (SWIGLU) acc[MT + mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_up[u], b[mt][u], acc[MT + mt], 0, 0, 0);
+      }
     }
   }
   // K % 32 in {8, 16, 24}: the last step is partial; lane groups past the end contribute zeros.
-  if (s_full < s_end && ((s_full - s_begin) & 3) == wave) {
+  if (s_full < s_end && (!SPLIT || ((s_full - s_begin) & 3) == wave)) {
     const int k = s_full << 5;
     const bool in = k + 8 * g < K;
     const bf16x8 a = in ? load8(wrow + k) : zero8();
@@ -149,42 +171,62 @@ __global__ __launch_bounds__(256) void skinny_mfma_kernel(const bf16_t* __restri
       if (SWIGLU) acc[MT + mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_up, b, acc[MT + mt], 0, 0, 0);
     }
   }
+
+  auto finish = [&](int mt, f32x4 sum, f32x4 up) {
+    if (SWIGLU) {
+#pragma unroll
+      for (int v = 0; v < 4; ++v) sum[v] = silu_f(sum[v]) * up[v];
+    }
+    const int m = mt * 16 + r;
+    if (m >= M) return;
+    TO* dst = out + (static_cast<int64_t>(blockIdx.y) * M + m) * n_out;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int n = n0 + 4 * g + v;
+      if (n < n_out) dst[n] = from_float<TO>(sum[v]);
+    }
+  };
+
+  if (!SPLIT) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) finish(mt, acc[mt], SWIGLU ? acc[MT + mt] : acc[mt]);
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < NACC; ++i) red[wave][i][lane] = acc[i];
   __syncthreads();
-  // Wave `wave` finishes column tiles wave, wave + 4, ... (MT <= 4: at most one each).
+  // Wave `wave` finishes column tile `wave` (MT <= 4: at most one each).
   if (wave >= MT) return;
   const int mt = wave;
-  f32x4 sum = red[0][mt][lane] + red[1][mt][lane] + red[2][mt][lane] + red[3][mt][lane];
-  if (SWIGLU) {
-    const f32x4 up = red[0][MT + mt][lane] + red[1][MT + mt][lane] + red[2][MT + mt][lane] + red[3][MT + mt][lane];
-#pragma unroll
-    for (int v = 0; v < 4; ++v) sum[v] = silu_f(sum[v]) * up[v];
+  const f32x4 sum = red[0][mt][lane] + red[1][mt][lane] + red[2][mt][lane] + red[3][mt][lane];
+  f32x4 up = sum;
+  if (SWIGLU) up = red[0][MT + mt][lane] + red[1][MT + mt][lane] + red[2][MT + mt][lane] + red[3][MT + mt][lane];
+  finish(mt, sum, up);
+}
+
+template <int MT, bool SPLIT>
+static int launch_skinny2(hipStream_t s, const void* x, const void* w, void* out, int out_dtype, int M, int n_out,
+                          int K, int epilogue, int ksplit) {
+  const int64_t tiles = ceil_div(n_out, 16);
+  const dim3 grid(static_cast<unsigned>(SPLIT ? tiles : ceil_div(tiles, 4)), static_cast<unsigned>(ksplit)), block(256);
+  const bf16_t* xp = static_cast<const bf16_t*>(x);
+  const bf16_t* wp = static_cast<const bf16_t*>(w);
+  if (epilogue == 1) {
+    skinny_mfma_kernel<MT, true, SPLIT, bf16_t><<<grid, block, 0, s>>>(xp, wp, static_cast<bf16_t*>(out), M, n_out, K);
+  } else if (out_dtype == kBF16) {
+    skinny_mfma_kernel<MT, false, SPLIT, bf16_t><<<grid, block, 0, s>>>(xp, wp, static_cast<bf16_t*>(out), M, n_out, K);
+  } else {
+    skinny_mfma_kernel<MT, false, SPLIT, float><<<grid, block, 0, s>>>(xp, wp, static_cast<float*>(out), M, n_out, K);
   }
-  const int m = mt * 16 + r;
-  if (m >= M) return;
-  TO* dst = out + (static_cast<int64_t>(blockIdx.y) * M + m) * n_out;
-#pragma unroll
-  for (int v = 0; v < 4; ++v) {
-    const int n = n0 + 4 * g + v;
-    if (n < n_out) dst[n] = from_float<TO>(sum[v]);
-  }
+  return check_launch("psamd_linear_skinny");
 }
 
 template <int MT>
 static int launch_skinny(hipStream_t s, const void* x, const void* w, void* out, int out_dtype, int M, int n_out,
                          int K, int epilogue, int ksplit) {
-  const dim3 grid(static_cast<unsigned>(ceil_div(n_out, 16)), static_cast<unsigned>(ksplit)), block(256);
-  const bf16_t* xp = static_cast<const bf16_t*>(x);
-  const bf16_t* wp = static_cast<const bf16_t*>(w);
-  if (epilogue == 1) {
-    skinny_mfma_kernel<MT, true, bf16_t><<<grid, block, 0, s>>>(xp, wp, static_cast<bf16_t*>(out), M, n_out, K);
-  } else if (out_dtype == kBF16) {
-    skinny_mfma_kernel<MT, false, bf16_t><<<grid, block, 0, s>>>(xp, wp, static_cast<bf16_t*>(out), M, n_out, K);
-  } else {
-    skinny_mfma_kernel<MT, false, float><<<grid, block, 0, s>>>(xp, wp, static_cast<float*>(out), M, n_out, K);
-  }
-  return check_launch("psamd_linear_skinny");
+  // Enough 16-row tiles to fill the chip with one wave each: no need to split K inside a workgroup.
+  if (ceil_div(n_out, 16) >= 2048) return launch_skinny2<MT, false>(s, x, w, out, out_dtype, M, n_out, K, epilogue, ksplit);
+  return launch_skinny2<MT, true>(s, x, w, out, out_dtype, M, n_out, K, epilogue, ksplit);
 }
 
 // The q/k/v projection of a small step fused with what follows it: rotary encoding of q and
@@ -216,13 +258,27 @@ __global__ __launch_bounds__(256) void qkv_rope_append_kernel(
 #pragma unroll
   for (int i = 0; i < MT; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int s_full = K >> 5;
-#pragma unroll 4
-  for (int s = wave; s < s_full; s += 4) {
-    const int k = s << 5;
-    const bf16x8 a = load8(wrow + k);
+  constexpr int U = MT == 1 ? 8 : (MT == 2 ? 4 : 2);   // steps whose loads are in flight together
+  for (int base = wave; base < s_full; base += 4 * U) {
+    bf16x8 a[U], b[MT][U];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-      acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, load8(xrow[mt] + k), acc[mt], 0, 0, 0);
+    for (int u = 0; u < U; ++u) {
+      const int s = base + 4 * u;
+      if (s < s_full) {
+        a[u] = load8(wrow + (s << 5));
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) b[mt][u] = load8(xrow[mt] + (s << 5));
+      } else {
+        a[u] = zero8();
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) b[mt][u] = zero8();
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b[mt][u], acc[mt], 0, 0, 0);
   }
   if ((K & 31) != 0 && (s_full & 3) == wave) {
     const int k = s_full << 5;
