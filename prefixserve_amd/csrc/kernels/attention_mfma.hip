@@ -335,24 +335,30 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
   }
 }
 
-// One block per (decode item, head): merges the splits and writes bfloat16.
-__global__ void attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                         bf16_t* __restrict__ out, const int32_t* __restrict__ dec_items,
-                                         const int32_t* __restrict__ item_start, int hq, int d, int nsplit) {
-  const int di = blockIdx.x, h = blockIdx.y;
+// One block (64 threads) per (decode item, head): merges the splits and writes bfloat16.
+// Lane s first loads the statistics of split s, so the weights of all splits come from one
+// round of loads; then every lane sums its dimensions over the splits with loads that do
+// not depend on each other.
+__global__ __launch_bounds__(64) void attn_decode_merge_kernel(
+    const float* __restrict__ part_o, const float* __restrict__ part_ml, bf16_t* __restrict__ out,
+    const int32_t* __restrict__ dec_items, const int32_t* __restrict__ item_start, int hq, int d, int nsplit) {
+  __shared__ float wgt_s[64];
+  const int di = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int64_t t = item_start[dec_items[di]];
   const int64_t base = (static_cast<int64_t>(di) * hq + h) * nsplit;
-  float mm = -INFINITY;
-  for (int s = 0; s < nsplit; ++s) mm = fmaxf(mm, part_ml[(base + s) * 2]);
-  for (int i = threadIdx.x; i < d; i += blockDim.x) {
-    float acc = 0.f, ll = 0.f;
-    for (int s = 0; s < nsplit; ++s) {
-      const float ms = part_ml[(base + s) * 2];
-      const float wgt = ms == -INFINITY ? 0.f : __expf(ms - mm);
-      acc += wgt * part_o[(base + s) * d + i];
-      ll += wgt * part_ml[(base + s) * 2 + 1];
-    }
-    out[t * (static_cast<int64_t>(hq) * d) + h * d + i] = float_to_bf16(acc / ll);
+  const bool has = lane < nsplit;                       // nsplit <= 64
+  const float ms = has ? part_ml[(base + lane) * 2] : -INFINITY;
+  const float ls = has ? part_ml[(base + lane) * 2 + 1] : 0.f;
+  const float mm = wave_max(ms);
+  const float w = ms == -INFINITY ? 0.f : __expf(ms - mm);
+  const float ll = wave_sum(w * ls);
+  wgt_s[lane] = w / ll;
+  __syncthreads();
+  for (int i = lane; i < d; i += kWave) {
+    float acc = 0.f;
+#pragma unroll 8
+    for (int s = 0; s < nsplit; ++s) acc += wgt_s[s] * part_o[(base + s) * d + i];
+    out[t * (static_cast<int64_t>(hq) * d) + h * d + i] = float_to_bf16(acc);
   }
 }
 
@@ -440,7 +446,7 @@ int psamd_attention_decode(void* stream, const void* qkv, int q_stride, void* ou
                            int hkv, int head_dim, int nsplit, float scale, int window) {
   PSAMD_REQUIRE(psamd_attention_mfma_supports(hq, hkv, head_dim), "shape not supported by the matrix-core kernels");
   PSAMD_REQUIRE(q_stride % 8 == 0, "query row stride must be a multiple of 8 elements");
-  PSAMD_REQUIRE(nsplit >= 1 && nsplit <= 65535, "nsplit out of range");
+  PSAMD_REQUIRE(nsplit >= 1 && nsplit <= 64, "nsplit must be in [1, 64]");
   if (n_dec == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int group = hq / hkv;

@@ -29,60 +29,73 @@ __global__ void embed_kernel(const int32_t* __restrict__ ids, const W* __restric
 // activation type or n_partials float slices [n_partials][rows, hidden] (partial sums of a
 // K-split product). Without `rows` the block handles row blockIdx.x and stores x back as the
 // new residual; with `rows` it handles residual row rows[blockIdx.x] and leaves it as it is.
-// Rows up to kCache * kThreads wide stay in registers between the two passes.
-template <typename A, int kThreads, int kCache>
+// Rows up to kCache * kThreads wide stay in registers between the two passes, and all loads
+// of a pass are independent of each other (clamped addresses, no branches around them), so
+// they are in flight together: with one row per block the kernel is pure latency.
+template <typename A, typename DT, int kThreads, int kCache>
 __global__ __launch_bounds__(kThreads) void add_rmsnorm_kernel(
-    float* __restrict__ residual, const void* __restrict__ delta, int delta_dtype, int n_partials,
-    int64_t partial_stride, const int32_t* __restrict__ rows, const void* __restrict__ weight, int weight_dtype,
-    float eps, A* __restrict__ out, int hidden) {
+    float* __restrict__ residual, const DT* __restrict__ delta, int n_partials, int64_t partial_stride,
+    const int32_t* __restrict__ rows, const void* __restrict__ weight, int weight_dtype, float eps,
+    A* __restrict__ out, int hidden) {
   __shared__ float scratch[kThreads / kWave];
   const int64_t src = rows != nullptr ? rows[blockIdx.x] : blockIdx.x;
   float* r = residual + src * hidden;
-  const int64_t doff = src * hidden;
+  const DT* d0 = delta != nullptr ? delta + src * hidden : nullptr;
   A* o = out + static_cast<int64_t>(blockIdx.x) * hidden;
   const bool store = rows == nullptr && delta != nullptr;
-  const bool cached = hidden <= kCache * kThreads;
+  const int np = delta != nullptr ? n_partials : 0;
+
+  if (hidden <= kCache * kThreads) {
+    float v[kCache], wv[kCache];
+    int idx[kCache];
+#pragma unroll
+    for (int j = 0; j < kCache; ++j) {
+      idx[j] = min(static_cast<int>(threadIdx.x) + j * kThreads, hidden - 1);
+      v[j] = r[idx[j]];
+      wv[j] = load_as_float(weight, weight_dtype, idx[j]);
+    }
+    for (int p = 0; p < np; ++p) {
+      const DT* dp = d0 + p * partial_stride;
+      float t[kCache];
+#pragma unroll
+      for (int j = 0; j < kCache; ++j) t[j] = to_float<DT>(dp[idx[j]]);
+#pragma unroll
+      for (int j = 0; j < kCache; ++j) v[j] += t[j];
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < kCache; ++j) {
+      const bool in = static_cast<int>(threadIdx.x) + j * kThreads < hidden;
+      ss += in ? v[j] * v[j] : 0.f;
+    }
+    ss = block_sum(ss, scratch, kThreads / kWave);
+    const float inv = rsqrtf(ss / static_cast<float>(hidden) + eps);
+#pragma unroll
+    for (int j = 0; j < kCache; ++j) {
+      if (static_cast<int>(threadIdx.x) + j * kThreads < hidden) {
+        if (store) r[idx[j]] = v[j];
+        o[idx[j]] = from_float<A>(wv[j] * (v[j] * inv));
+      }
+    }
+    return;
+  }
 
   auto value = [&](int i) {
     float x = r[i];
-    if (delta != nullptr) {
-      for (int p = 0; p < n_partials; ++p) x += load_as_float(delta, delta_dtype, p * partial_stride + doff + i);
-    }
+    for (int p = 0; p < np; ++p) x += to_float<DT>(d0[p * partial_stride + i]);
     return x;
   };
-
-  float v[kCache];
   float ss = 0.f;
-  if (cached) {
-#pragma unroll
-    for (int j = 0; j < kCache; ++j) {
-      const int i = threadIdx.x + j * kThreads;
-      v[j] = i < hidden ? value(i) : 0.f;
-      ss += v[j] * v[j];
-    }
-  } else {
-    for (int i = threadIdx.x; i < hidden; i += kThreads) {
-      const float x = value(i);
-      if (store) r[i] = x;
-      ss += x * x;
-    }
+  for (int i = threadIdx.x; i < hidden; i += kThreads) {
+    const float x = value(i);
+    if (store) r[i] = x;
+    ss += x * x;
   }
   ss = block_sum(ss, scratch, kThreads / kWave);
   const float inv = rsqrtf(ss / static_cast<float>(hidden) + eps);
-  if (cached) {
-#pragma unroll
-    for (int j = 0; j < kCache; ++j) {
-      const int i = threadIdx.x + j * kThreads;
-      if (i < hidden) {
-        if (store) r[i] = v[j];
-        o[i] = from_float<A>(load_as_float(weight, weight_dtype, i) * (v[j] * inv));
-      }
-    }
-  } else {
-    for (int i = threadIdx.x; i < hidden; i += kThreads) {
-      const float x = store ? r[i] : value(i);
-      o[i] = from_float<A>(load_as_float(weight, weight_dtype, i) * (x * inv));
-    }
+  for (int i = threadIdx.x; i < hidden; i += kThreads) {
+    const float x = store ? r[i] : value(i);
+    o[i] = from_float<A>(load_as_float(weight, weight_dtype, i) * (x * inv));
   }
 }
 
@@ -188,17 +201,20 @@ int psamd_add_rmsnorm(void* stream, float* residual, const void* delta, int delt
   if (out_rows == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   constexpr int kThreads = 256, kCache = 16;
+  const dim3 grid(static_cast<unsigned>(out_rows)), block(kThreads);
+#define PSAMD_NORM(A_, D_)                                                                                      \
+  add_rmsnorm_kernel<A_, D_, kThreads, kCache><<<grid, block, 0, s>>>(                                          \
+      residual, static_cast<const D_*>(delta), n_partials, partial_stride, rows, weight, weight_dtype, eps, \
+      static_cast<A_*>(out), hidden)
+  const bool delta_f32 = delta == nullptr || delta_dtype == kF32;
   if (act_dtype == kBF16) {
-    add_rmsnorm_kernel<bf16_t, kThreads, kCache><<<dim3(out_rows), dim3(kThreads), 0, s>>>(
-        residual, delta, delta_dtype, n_partials, partial_stride, rows, weight, weight_dtype, eps,
-        static_cast<bf16_t*>(out), hidden);
+    if (delta_f32) PSAMD_NORM(bf16_t, float); else PSAMD_NORM(bf16_t, bf16_t);
   } else if (act_dtype == kF32) {
-    add_rmsnorm_kernel<float, kThreads, kCache><<<dim3(out_rows), dim3(kThreads), 0, s>>>(
-        residual, delta, delta_dtype, n_partials, partial_stride, rows, weight, weight_dtype, eps,
-        static_cast<float*>(out), hidden);
+    if (delta_f32) PSAMD_NORM(float, float); else PSAMD_NORM(float, bf16_t);
   } else {
     return fail("psamd_add_rmsnorm: activation dtype must be float32 or bfloat16");
   }
+#undef PSAMD_NORM
   return check_launch("psamd_add_rmsnorm");
 }
 
