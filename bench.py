@@ -57,6 +57,7 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / batch 64 points")
     ap.add_argument("--no-graphs", action="store_true")
+    ap.add_argument("--prefill-reps", type=int, default=5, help="timed repetitions of the 2,048-token prefill")
     ap.add_argument("--model", default=None, help="use this model folder instead of writing random weights")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -142,7 +143,7 @@ def main() -> int:
         return {"value": n / (ms / 1e3), "tokens": n, "ms": ms,
                 "frac": flops / (ms / 1e3) / (MFMA_PEAK_TFLOPS[args.dtype] * 1e12)}
 
-    prefill = prefill_run()
+    prefill = prefill_run(reps=args.prefill_reps)
     main_run = decode_run(args.batch, args.steps, args.warmup)
     points = {}
     if not args.no_points:
