@@ -42,6 +42,10 @@ HIPCC_FLAGS = [
     # Packed fp32 instructions are kept out of every kernel of this library.
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-result",
+    # Matrix-core results stay in ordinary vector registers: the softmax and epilogues read
+    # them at once, and copies to and from the accumulator file were a fifth of all vector
+    # instructions in the attention kernels.
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",
 ]
 
 
@@ -80,14 +84,16 @@ def lib_dir() -> Path:
 
 
 def _existing(name: str) -> Path | None:
-    """A built library, looked for in-tree first and then in the fallback folder."""
+    """A built library: in the folder ``PREFIXSERVE_AMD_LIB_DIR`` names if it is set, else
+    in-tree, else in the per-user fallback folder."""
+    override = os.environ.get("PREFIXSERVE_AMD_LIB_DIR")
+    if override:
+        p = Path(override) / name
+        return p if p.exists() else None
     for d in (PKG_DIR / "_lib", Path(tempfile.gettempdir()) / f"prefixserve_amd-lib-{os.getuid()}"):
         p = d / name
         if p.exists():
             return p
-    override = os.environ.get("PREFIXSERVE_AMD_LIB_DIR")
-    if override and (Path(override) / name).exists():
-        return Path(override) / name
     return None
 
 
@@ -144,9 +150,12 @@ def build_kernels() -> Path:
         raise BuildError(f"no kernel sources under {CSRC / 'kernels'}")
     _say(f"compiling {len(srcs)} HIP sources for {GPU_ARCH} ...")
 
+    extra = os.environ.get("PREFIXSERVE_AMD_HIPCC_FLAGS", "").split()
+
     def one(src: Path) -> Path:
         obj = obj_dir / (src.stem + ".o")
-        _run([hipcc, *HIPCC_FLAGS, f"-I{CSRC / 'kernels'}", "-c", str(src), "-o", str(obj)], f"hipcc {src.name}")
+        _run([hipcc, *HIPCC_FLAGS, *extra, f"-I{CSRC / 'kernels'}", "-c", str(src), "-o", str(obj)],
+             f"hipcc {src.name}")
         return obj
 
     workers = max(1, min(len(srcs), (os.cpu_count() or 2), 8))

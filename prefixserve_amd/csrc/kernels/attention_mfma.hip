@@ -6,8 +6,9 @@
 // second without passing through LDS. The cache stores values transposed per page
 // ([D][16], see elementwise.hip) so that V^T rows are contiguous 8-byte runs.
 //
-//  * prefill: one wave per (32 new tokens, query head); v_mfma_f32_32x32x16_bf16; online
-//    softmax per query column held redundantly in lanes l and l^32.
+//  * prefill: one workgroup per (32 new tokens, query head), its 4 waves splitting the keys;
+//    v_mfma_f32_32x32x16_bf16; online softmax per query column held redundantly in lanes l
+//    and l^32; log-sum-exp merge of the waves in LDS.
 //  * decode: one workgroup per (request, kv head, split of the key range); the `group`
 //    query heads sharing the kv head are the columns of a 16x16x32 tile, so every key and
 //    value byte is read once for all of them; 4 waves interleave 32-key tiles and merge by
@@ -49,7 +50,16 @@ __device__ __forceinline__ bf16x8 join(bf16x4 a, bf16x4 b) {
 
 // ------------------------------------------------------------------ prefill
 
-// NS = D / 16. Block = 4 waves = 128 consecutive queries of one item, one query head.
+// NS = D / 16. A workgroup owns 32 consecutive queries of one item and one query head; its
+// 4 waves take the 32-key tiles in turn and merge by log-sum-exp through LDS. Splitting the
+// keys (not the queries) over the waves keeps the longest dependent chain of tiles four
+// times shorter, which is what bounds a causal prompt's last rows.
+// Per wave the loop is unrolled by two with two register sets: the keys and values of the
+// wave's next tile are loaded before the current one is computed. The block table is staged
+// in LDS once (a page id fetched from global memory inside the loop would put a second,
+// unhidden latency in front of every tile's loads). Only tiles that touch the diagonal (or a
+// window's edge) pay for masking; the softmax uses exp2 with the scale folded into one
+// multiply-add per score.
 template <int NS>
 __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
     const bf16_t* __restrict__ qkv, int q_stride, bf16_t* __restrict__ out, const bf16_t* __restrict__ kv,
@@ -58,16 +68,19 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
     const int32_t* __restrict__ block_ids, int hq, int hkv, float scale, int window) {
   constexpr int D = 16 * NS;
   constexpr int DT = (D + 31) / 32;
-  const int tile = blockIdx.x, h = blockIdx.y;
+  constexpr int DTC = DT < 2 ? DT : 2;      // d-tiles merged per pass (bounds the LDS buffer)
+  __shared__ float sm_m[4][32], sm_l[4][32];
+  __shared__ float sm_o[3 * DTC * 16 * 64];
+  extern __shared__ int32_t table[];
+  // Late tiles of a prompt see the most keys: start them first.
+  const int tile = gridDim.x - 1 - blockIdx.x, h = blockIdx.y;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int item = pf_tiles[2 * tile];
-  const int q_off = pf_tiles[2 * tile + 1] + wave * 32;
+  const int q_off = pf_tiles[2 * tile + 1];
   const int t0 = item_start[item];
   const int n = item_start[item + 1] - t0;
-  if (q_off >= n) return;
   const int pos0 = item_pos0[item];
   const int kvh = h / (hq / hkv);
-  const int32_t* table = block_ids + table_off[item];
   const int col = lane & 31, hi = lane >> 5;
 
   const int qi = min(q_off + col, n - 1);          // lanes past the end repeat the last query
@@ -78,6 +91,12 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
   const int max_key = pos0 + n - 1;
   const int k_lo_q = window > 0 ? max(0, q_pos - window + 1) : 0;
   const int k_begin = window > 0 ? (max(0, first_pos - window + 1) & ~31) : 0;
+  const float c = scale * 1.44269504088896340736f;  // scores are exponentiated in base 2
+  {
+    const int32_t* gtable = block_ids + table_off[item];
+    for (int i = threadIdx.x; i <= (last_pos >> 4); i += blockDim.x) table[i] = gtable[i];
+  }
+  __syncthreads();
 
   bf16x8 qf[NS];
   {
@@ -91,83 +110,156 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
     for (int v = 0; v < 16; ++v) o[dt][v] = 0.f;
-  float m = -INFINITY, l = 0.f;
+  float m = -INFINITY, l = 0.f;       // m in base-2 units (score * c)
 
   const int64_t page_elems = 2LL * hkv * kPage * D;
   const int64_t khead = static_cast<int64_t>(kvh) * kPage * D;
   const int64_t vhead = static_cast<int64_t>(hkv) * kPage * D + static_cast<int64_t>(kvh) * D * kPage;
 
-  for (int k0 = k_begin; k0 <= last_pos; k0 += 32) {
-    // ---- S^T[key][query] = K . Q^T : lane supplies key row (k0 + col) of K
-    const int key_a = min(k0 + col, max_key);
+  struct Tile {
+    bf16x8 k[NS];        // A operand of S^T = K.Q^T: key row (k0 + col), 8 dims per 16-wide step
+    bf16x8 v[2][DT];     // A operand of O^T += V^T.P^T: page c of the tile, V^T row d
+  };
+  auto load_tile = [&](Tile& t, int k0) {
+    const int key_a = min(k0 + col, last_pos);
     const bf16_t* kp = kv + static_cast<int64_t>(table[key_a >> 4]) * page_elems + khead + (key_a & 15) * D + 8 * hi;
-    f32x16 s;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) s[v] = 0.f;
+    for (int i = 0; i < NS; ++i) t.k[i] = ld8(kp + 16 * i);
 #pragma unroll
-    for (int i = 0; i < NS; ++i) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ld8(kp + 16 * i), qf[i], s, 0, 0, 0);
-
-    // ---- mask, scale, online softmax for query column `col`
-    float sv[16];
-    float mx = -INFINITY;
+    for (int cpage = 0; cpage < 2; ++cpage) {
+      const int key_p = min(k0 + 16 * cpage, last_pos);
+      const bf16_t* vp = kv + static_cast<int64_t>(table[key_p >> 4]) * page_elems + vhead + 4 * hi;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int key = k0 + 8 * (v >> 2) + 4 * hi + (v & 3);
-      const bool ok = key <= q_pos && key >= k_lo_q;
-      sv[v] = ok ? s[v] * scale : -INFINITY;
-      mx = fmaxf(mx, sv[v]);
+      for (int dt = 0; dt < DT; ++dt) {
+        const bf16_t* vr = vp + min(32 * dt + col, D - 1) * kPage;
+        t.v[cpage][dt] = join(ld4(vr), ld4(vr + 8));
+      }
     }
-    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
-    const float m_new = fmaxf(m, mx);
-    const float m_use = m_new == -INFINITY ? 0.f : m_new;
-    const float alpha = __expf(m - m_use);
+  };
+  auto compute = [&](const Tile& t, int k0) {
+    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    f32x16 s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(t.k[0], qf[0], zero, 0, 0, 0);
+#pragma unroll
+    for (int i = 1; i < NS; ++i) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(t.k[i], qf[i], s, 0, 0, 0);
+    // A tile whose last key is not after the first query, with no window, needs no mask.
+    if (window > 0 || k0 + 31 > first_pos) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int key = k0 + 8 * (v >> 2) + 4 * hi + (v & 3);
+        s[v] = (key <= q_pos && key >= k_lo_q) ? s[v] : -INFINITY;
+      }
+    }
+    float mx = s[0];
+#pragma unroll
+    for (int v = 1; v < 16; ++v) mx = fmaxf(mx, s[v]);
+    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave)) * c;
+    // The running maximum is only raised (and the accumulators rescaled) when some query's
+    // scores outgrow it by more than 2^8: probabilities stay below 256, nothing overflows,
+    // the final division by the sum is exact either way, and most tiles skip the rescale of
+    // the whole accumulator.
+    if (__any(mx > m + 8.f)) {
+      const float m_new = fmaxf(m, mx);
+      const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m - m_new);
+      l *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o[dt][v] *= alpha;
+      m = m_new;
+    }
+    const float m_use = m == -INFINITY ? 0.f : m;
     float rowsum = 0.f;
     bf16x8 pb[2];
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
-      const float p = __expf(sv[v] - m_use);
+      const float p = __builtin_amdgcn_exp2f(fmaf(s[v], c, -m_use));
       rowsum += p;
       pb[v >> 3][v & 7] = static_cast<__bf16>(p);
     }
-    rowsum += __shfl_xor(rowsum, 32, kWave);
-    l = l * alpha + rowsum;
-    m = m_new;
+    l += rowsum + __shfl_xor(rowsum, 32, kWave);
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
+    for (int cpage = 0; cpage < 2; ++cpage)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) o[dt][v] *= alpha;
+      for (int dt = 0; dt < DT; ++dt)
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(t.v[cpage][dt], pb[cpage], o[dt], 0, 0, 0);
+  };
 
-    // ---- O^T[d][query] += V^T . P^T : half c of the tile is page c; lane supplies V^T row d
-#pragma unroll
-    for (int c = 0; c < 2; ++c) {
-      const int key_p = min(k0 + 16 * c, max_key);
-      const bf16_t* vp = kv + static_cast<int64_t>(table[key_p >> 4]) * page_elems + vhead + 4 * hi;
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        const int drow = min(32 * dt + col, D - 1);
-        const bf16_t* vr = vp + drow * kPage;
-        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(join(ld4(vr), ld4(vr + 8)), pb[c], o[dt], 0, 0, 0);
+  {
+    Tile ta, tb;
+    int k0 = k_begin + 32 * wave;
+    if (k0 <= last_pos) {
+      load_tile(ta, k0);
+      while (true) {
+        // The next tile is loaded whether or not it exists (addresses are clamped to the last
+        // key): with no branch around the loads, the wait in front of the matrix instructions
+        // counts exactly the loads of the current tile and leaves the next tile's in flight.
+        load_tile(tb, k0 + 128);
+        compute(ta, k0);
+        k0 += 128;
+        if (k0 > last_pos) break;
+        load_tile(ta, k0 + 128);
+        compute(tb, k0);
+        k0 += 128;
+        if (k0 > last_pos) break;
       }
     }
   }
 
-  if (!q_valid) return;
-  const float inv = 1.f / l;
+  // ---- merge the 4 waves' partial results for the 32 queries
+  if (hi == 0) {
+    sm_m[wave][col] = m;
+    sm_l[wave][col] = l;
+  }
+  __syncthreads();
+  float mm = sm_m[0][col];
+#pragma unroll
+  for (int w = 1; w < 4; ++w) mm = fmaxf(mm, sm_m[w][col]);
+  float ll = 0.f, mine = 0.f;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    const float mw = sm_m[w][col];
+    const float f = mw == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw - mm);
+    ll += f * sm_l[w][col];
+    if (w == wave) mine = f;
+  }
+  const float inv = 1.f / ll;
   bf16_t* op = out + static_cast<int64_t>(t0 + qi) * (static_cast<int64_t>(hq) * D) + h * D;
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt) {
+  for (int d0 = 0; d0 < DT; d0 += DTC) {
+    if (wave > 0) {
 #pragma unroll
-    for (int v4 = 0; v4 < 4; ++v4) {
-      const int d = 32 * dt + 8 * v4 + 4 * hi;
-      if (d < D) {
-        ushort4 pk;
-        pk.x = float_to_bf16(o[dt][4 * v4 + 0] * inv);
-        pk.y = float_to_bf16(o[dt][4 * v4 + 1] * inv);
-        pk.z = float_to_bf16(o[dt][4 * v4 + 2] * inv);
-        pk.w = float_to_bf16(o[dt][4 * v4 + 3] * inv);
-        *reinterpret_cast<ushort4*>(op + d) = pk;
+      for (int dt = 0; dt < DTC; ++dt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          if (d0 + dt < DT) sm_o[(((wave - 1) * DTC + dt) * 16 + v) * 64 + lane] = o[d0 + dt][v] * mine;
+    }
+    __syncthreads();
+    if (wave == 0 && q_valid) {
+#pragma unroll
+      for (int dt = 0; dt < DTC; ++dt) {
+        if (d0 + dt >= DT) continue;
+        float r[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          r[v] = o[d0 + dt][v] * mine;
+#pragma unroll
+          for (int w = 0; w < 3; ++w) r[v] += sm_o[((w * DTC + dt) * 16 + v) * 64 + lane];
+        }
+#pragma unroll
+        for (int v4 = 0; v4 < 4; ++v4) {
+          const int d = 32 * (d0 + dt) + 8 * v4 + 4 * hi;
+          if (d < D) {
+            ushort4 pk;
+            pk.x = float_to_bf16(r[4 * v4 + 0] * inv);
+            pk.y = float_to_bf16(r[4 * v4 + 1] * inv);
+            pk.z = float_to_bf16(r[4 * v4 + 2] * inv);
+            pk.w = float_to_bf16(r[4 * v4 + 3] * inv);
+            *reinterpret_cast<ushort4*>(op + d) = pk;
+          }
+        }
       }
     }
+    if (d0 + DTC < DT) __syncthreads();
   }
 }
 
@@ -364,9 +456,9 @@ __global__ __launch_bounds__(64) void attn_decode_merge_kernel(
 
 template <int NS>
 static int launch_prefill(hipStream_t s, const void* qkv, int q_stride, void* out, const void* kv,
-                          const int32_t* pf_tiles, int n_tiles, const int32_t* item_start, const int32_t* item_pos0,
+                          const int32_t* pf_tiles, int n_tiles, int table_pages, const int32_t* item_start, const int32_t* item_pos0,
                           const int32_t* table_off, const int32_t* block_ids, int hq, int hkv, float scale, int window) {
-  attn_prefill_mfma_kernel<NS><<<dim3(n_tiles, hq), dim3(256), 0, s>>>(
+  attn_prefill_mfma_kernel<NS><<<dim3(n_tiles, hq), dim3(256), sizeof(int32_t) * static_cast<size_t>(table_pages), s>>>(
       static_cast<const bf16_t*>(qkv), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(kv), pf_tiles,
       item_start, item_pos0, table_off, block_ids, hq, hkv, scale, window);
   return check_launch("psamd_attention_prefill");
@@ -417,17 +509,20 @@ int psamd_attention_mfma_supports(int hq, int hkv, int head_dim) {
   return dim_ok && group <= 64 && smem <= 64 * 1024 && hq <= 65535 && hkv <= 65535;
 }
 
+// max_kv_len: the longest request of the step after it (sizes the block table staged in LDS).
 int psamd_attention_prefill(void* stream, const void* qkv, int q_stride, void* out, const void* kv,
-                            const int32_t* pf_tiles, int n_tiles, const int32_t* item_start,
+                            const int32_t* pf_tiles, int n_tiles, int max_kv_len, const int32_t* item_start,
                             const int32_t* item_pos0, const int32_t* table_off, const int32_t* block_ids, int hq,
                             int hkv, int head_dim, float scale, int window) {
   PSAMD_REQUIRE(psamd_attention_mfma_supports(hq, hkv, head_dim), "shape not supported by the matrix-core kernels");
   PSAMD_REQUIRE(q_stride % 8 == 0, "query row stride must be a multiple of 8 elements");
+  PSAMD_REQUIRE(max_kv_len >= 1 && max_kv_len <= 8192 * kPage, "context too long for the block table staged in LDS");
   if (n_tiles == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  const int table_pages = static_cast<int>(ceil_div(max_kv_len, kPage));
 #define PSAMD_PF(NS_)                                                                                           \
-  return launch_prefill<NS_>(s, qkv, q_stride, out, kv, pf_tiles, n_tiles, item_start, item_pos0, table_off, \
-                             block_ids, hq, hkv, scale, window)
+  return launch_prefill<NS_>(s, qkv, q_stride, out, kv, pf_tiles, n_tiles, table_pages, item_start, item_pos0, \
+                             table_off, block_ids, hq, hkv, scale, window)
   switch (head_dim / 16) {
     case 1: PSAMD_PF(1);
     case 2: PSAMD_PF(2);

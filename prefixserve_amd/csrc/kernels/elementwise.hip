@@ -99,6 +99,89 @@ __global__ __launch_bounds__(kThreads) void add_rmsnorm_kernel(
   }
 }
 
+// The same operation for bfloat16 activations and rows that are a multiple of 8 wide: every
+// thread owns runs of 8 consecutive elements, moved as 16- and 32-byte accesses. kIter runs
+// per thread stay in registers (hidden <= 8 * kThreads * kIter).
+template <typename DT, int kThreads, int kIter>
+__global__ __launch_bounds__(kThreads) void add_rmsnorm_vec8_kernel(
+    float* __restrict__ residual, const DT* __restrict__ delta, int n_partials, int64_t partial_stride,
+    const int32_t* __restrict__ rows, const void* __restrict__ weight, int weight_dtype, float eps,
+    bf16_t* __restrict__ out, int hidden) {
+  __shared__ float scratch[kThreads / kWave];
+  const int64_t src = rows != nullptr ? rows[blockIdx.x] : blockIdx.x;
+  float* r = residual + src * hidden;
+  const DT* d0 = delta != nullptr ? delta + src * hidden : nullptr;
+  bf16_t* o = out + static_cast<int64_t>(blockIdx.x) * hidden;
+  const bool store = rows == nullptr && delta != nullptr;
+  const int np = delta != nullptr ? n_partials : 0;
+  const int chunks = hidden >> 3;
+
+  float v[kIter][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < kIter; ++j) {
+    const int cidx = threadIdx.x + j * kThreads;
+    const int e = min(cidx, chunks - 1) << 3;
+    const float4 a = *reinterpret_cast<const float4*>(r + e);
+    const float4 b = *reinterpret_cast<const float4*>(r + e + 4);
+    v[j][0] = a.x; v[j][1] = a.y; v[j][2] = a.z; v[j][3] = a.w;
+    v[j][4] = b.x; v[j][5] = b.y; v[j][6] = b.z; v[j][7] = b.w;
+    for (int p = 0; p < np; ++p) {
+      const DT* dp = d0 + p * partial_stride + e;
+      if (sizeof(DT) == 2) {
+        const uint4 q = *reinterpret_cast<const uint4*>(dp);
+        const uint32_t w4[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          v[j][2 * i] += __uint_as_float(w4[i] << 16);
+          v[j][2 * i + 1] += __uint_as_float(w4[i] & 0xffff0000u);
+        }
+      } else {
+        const float4 x0 = *reinterpret_cast<const float4*>(dp);
+        const float4 x1 = *reinterpret_cast<const float4*>(dp + 4);
+        v[j][0] += x0.x; v[j][1] += x0.y; v[j][2] += x0.z; v[j][3] += x0.w;
+        v[j][4] += x1.x; v[j][5] += x1.y; v[j][6] += x1.z; v[j][7] += x1.w;
+      }
+    }
+    if (cidx < chunks) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) ss += v[j][i] * v[j][i];
+    }
+  }
+  ss = block_sum(ss, scratch, kThreads / kWave);
+  const float inv = rsqrtf(ss / static_cast<float>(hidden) + eps);
+#pragma unroll
+  for (int j = 0; j < kIter; ++j) {
+    const int cidx = threadIdx.x + j * kThreads;
+    if (cidx >= chunks) continue;
+    const int e = cidx << 3;
+    if (store) {
+      *reinterpret_cast<float4*>(r + e) = make_float4(v[j][0], v[j][1], v[j][2], v[j][3]);
+      *reinterpret_cast<float4*>(r + e + 4) = make_float4(v[j][4], v[j][5], v[j][6], v[j][7]);
+    }
+    float w[8];
+    if (weight_dtype == kBF16) {
+      const uint4 q = *reinterpret_cast<const uint4*>(static_cast<const bf16_t*>(weight) + e);
+      const uint32_t w4[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        w[2 * i] = __uint_as_float(w4[i] << 16);
+        w[2 * i + 1] = __uint_as_float(w4[i] & 0xffff0000u);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) w[i] = static_cast<const float*>(weight)[e + i];
+    }
+    uint32_t pk[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      pk[i] = static_cast<uint32_t>(float_to_bf16(w[2 * i] * (v[j][2 * i] * inv))) |
+              (static_cast<uint32_t>(float_to_bf16(w[2 * i + 1] * (v[j][2 * i + 1] * inv))) << 16);
+    }
+    *reinterpret_cast<uint4*>(o + e) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+  }
+}
+
 // ------------------------------------------------------------------ swiglu
 
 template <typename A>
@@ -110,6 +193,30 @@ __global__ void swiglu_kernel(const A* __restrict__ gate_up, A* __restrict__ out
     const float g = to_float<A>(gate_up[t * 2 * inter + c]);
     const float u = to_float<A>(gate_up[t * 2 * inter + inter + c]);
     out[i] = from_float<A>(g / (1.f + __expf(-g)) * u);
+  }
+}
+
+// bfloat16, intermediate size a multiple of 8: 16-byte accesses, 8 elements per thread.
+__global__ void swiglu_vec8_kernel(const bf16_t* __restrict__ gate_up, bf16_t* __restrict__ out, int64_t tokens,
+                                   int inter) {
+  const int chunks = inter >> 3;
+  const int64_t n = tokens * chunks;
+  for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < n;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const int64_t t = i / chunks;
+    const int e = static_cast<int>(i - t * chunks) << 3;
+    const uint4 g = *reinterpret_cast<const uint4*>(gate_up + t * 2 * inter + e);
+    const uint4 u = *reinterpret_cast<const uint4*>(gate_up + t * 2 * inter + inter + e);
+    const uint32_t g4[4] = {g.x, g.y, g.z, g.w}, u4[4] = {u.x, u.y, u.z, u.w};
+    uint32_t pk[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float g0 = __uint_as_float(g4[k] << 16), g1 = __uint_as_float(g4[k] & 0xffff0000u);
+      const float u0 = __uint_as_float(u4[k] << 16), u1 = __uint_as_float(u4[k] & 0xffff0000u);
+      pk[k] = static_cast<uint32_t>(float_to_bf16(g0 / (1.f + __expf(-g0)) * u0)) |
+              (static_cast<uint32_t>(float_to_bf16(g1 / (1.f + __expf(-g1)) * u1)) << 16);
+    }
+    *reinterpret_cast<uint4*>(out + t * inter + e) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
   }
 }
 
@@ -207,6 +314,21 @@ int psamd_add_rmsnorm(void* stream, float* residual, const void* delta, int delt
       residual, static_cast<const D_*>(delta), n_partials, partial_stride, rows, weight, weight_dtype, eps, \
       static_cast<A_*>(out), hidden)
   const bool delta_f32 = delta == nullptr || delta_dtype == kF32;
+  if (act_dtype == kBF16 && hidden % 8 == 0 && hidden <= 8 * kThreads * 4) {
+    bf16_t* o16 = static_cast<bf16_t*>(out);
+#define PSAMD_NORM8(D_, IT_)                                                                                 \
+  add_rmsnorm_vec8_kernel<D_, kThreads, IT_><<<grid, block, 0, s>>>(                                         \
+      residual, static_cast<const D_*>(delta), n_partials, partial_stride, rows, weight, weight_dtype, eps, \
+      o16, hidden)
+    const int iters = static_cast<int>(ceil_div(hidden / 8, kThreads));
+    if (delta_f32) {
+      if (iters <= 1) PSAMD_NORM8(float, 1); else if (iters <= 2) PSAMD_NORM8(float, 2); else PSAMD_NORM8(float, 4);
+    } else {
+      if (iters <= 1) PSAMD_NORM8(bf16_t, 1); else if (iters <= 2) PSAMD_NORM8(bf16_t, 2); else PSAMD_NORM8(bf16_t, 4);
+    }
+#undef PSAMD_NORM8
+    return check_launch("psamd_add_rmsnorm");
+  }
   if (act_dtype == kBF16) {
     if (delta_f32) PSAMD_NORM(bf16_t, float); else PSAMD_NORM(bf16_t, bf16_t);
   } else if (act_dtype == kF32) {
@@ -224,7 +346,11 @@ int psamd_swiglu(void* stream, const void* gate_up, void* out, int act_dtype, in
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int64_t n = tokens * inter;
   const int blocks = static_cast<int>(std::min<int64_t>(ceil_div(n, 256), 65536));
-  if (act_dtype == kBF16) {
+  if (act_dtype == kBF16 && inter % 8 == 0) {
+    const int vblocks = static_cast<int>(std::min<int64_t>(ceil_div(n / 8, 256), 65536));
+    swiglu_vec8_kernel<<<dim3(vblocks), dim3(256), 0, s>>>(static_cast<const bf16_t*>(gate_up),
+                                                           static_cast<bf16_t*>(out), tokens, inter);
+  } else if (act_dtype == kBF16) {
     swiglu_kernel<bf16_t><<<dim3(blocks), dim3(256), 0, s>>>(static_cast<const bf16_t*>(gate_up),
                                                             static_cast<bf16_t*>(out), tokens, inter);
   } else if (act_dtype == kF32) {
