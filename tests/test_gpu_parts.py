@@ -224,3 +224,125 @@ def test_a_toy_mixer_with_state_of_its_own(tmp_path):
     cut = np.concatenate(outs)
     assert np.abs(cut - whole).max() / np.abs(whole).max() < 1e-5
     assert np.abs(whole).max() > 0.1 and np.isfinite(whole).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_prenorm_block_is_one_plain_layer(dtype, model_dirs, plain_models):
+    """The block arrangement alone: norm -> mixer -> add, norm -> feed-forward -> add, with the
+    sums handed on as pending deltas, against the plain model's layer function."""
+    from configs import TINY
+    from prefixserve_amd.config import architecture_of
+    from prefixserve_amd.parts import DecoderModel
+    from prefixserve_amd.parts.attention import LayerCache
+    from prefixserve_amd.weights import load_weights
+
+    name = "B"
+    raw = TINY[name]
+    arch = architecture_of(raw)
+    spec = arch.build_spec(arch.config_cls.from_dicts(raw, {}))
+    model = DecoderModel(spec)
+    rt = runtime(dtype)
+    model.bind(load_weights(model_dirs[name], model.weights(), spec.ignored_weights), rt, 128)
+    plain = plain_models[name]
+    n, hidden = 50, raw["hidden_size"]
+    h0 = (0.5 * torch.randn(n, hidden)).to(torch.bfloat16).float()
+    cos, sin = P.rope_cos_sin(np.arange(n), plain.inv_freq)
+    want = plain.layer(1, h0.double().numpy(), cos, sin)
+
+    pk = StepPacker(DEV, [GroupMeta(8)], 10, 128, 4, rt.ops.PREFILL_TILE_Q)
+    hkv, d = raw["num_key_value_heads"], raw["head_dim"]
+    cache = LayerCache(kv=torch.zeros(8, 2, hkv, 16 * d, dtype=dtype, device=DEV), group=0, window=None)
+    block = model.blocks[1]
+    got, p0 = [], 0
+    for c in (33, 1, 16):                                         # a portion, a decode token, a portion
+        ctx = pk.pack([StepItem("a", [1] * c, p0, [[3, 1, 4, 6]])])
+        residual = h0[p0:p0 + c].to(DEV).contiguous()
+        pending = block.forward(residual, None, ctx, cache, None, True)
+        pend = pending.sum(0) if pending.dim() == 3 else pending.float()
+        got.append((residual + pend).clone())                     # the last add is the next block's
+        p0 += c
+    assert rel(torch.cat(got), want) < TOL[dtype] * 2
+
+
+def test_windowed_attention_through_the_engine(tmp_path):
+    """A toy architecture whose layers keep different things: one layer attends over a window
+    of 24 positions (its pages are given back as the window passes), one over everything.
+    Replayed whole, in portions and token by token, with a window-group pool too small for a
+    whole request; compared with the plain functions in both dtypes."""
+    import json
+
+    from safetensors.torch import save_file
+
+    from prefixserve_amd.config import register_architecture, registered_architectures
+    from prefixserve_amd.engine.replay import TraceReplayer
+    from prefixserve_amd.engine.runner import ModelRunner
+    from prefixserve_amd.parts import DecoderModel, LayerRun, LayerSpec, ModelSpec, PartSpec
+    from prefixserve_amd.weights import random_tensors
+
+    WINDOW, H, HQ, HKV, D, INNER, V = 24, 64, 4, 2, 16, 96, 120
+
+    class Cfg:
+        def __init__(self, raw):
+            self.raw = raw
+
+        @classmethod
+        def from_dicts(cls, raw, gen=None):
+            return cls(dict(raw))
+
+    def build(cfg):
+        def attn(window):
+            return PartSpec("paged_attention", {"num_heads": HQ, "num_kv_heads": HKV, "head_dim": D, "position": "rope",
+                                                "window": window,
+                                                "names": {"q": "q.weight", "k": "k.weight", "v": "v.weight", "o": "o.weight"}})
+        ff = PartSpec("swiglu", {"intermediate_size": INNER, "names": {"gate": "g.weight", "up": "u.weight", "down": "d.weight"}})
+        norm = lambda nm: PartSpec("rmsnorm", {"eps": 1e-5, "name": nm})
+        layers = tuple(LayerSpec(prefix=f"l{i}.", mixer=attn(WINDOW if i == 0 else None), feed_forward=ff,
+                                 mixer_norm=norm("n1.weight"), feed_forward_norm=norm("n2.weight")) for i in range(2))
+        return ModelSpec(vocab_size=V, hidden_size=H, embedding="emb.weight", layers=layers,
+                         order=(LayerRun(0, 0), LayerRun(1, 1)), final_norm=norm("norm.weight"), final_norm_prefix="",
+                         head=None, positions={"rope": PartSpec("rope", {"head_dim": D, "theta": 10000.0})}, max_position=512)
+
+    if "ToyWindowForCausalLM" not in registered_architectures():
+        register_architecture("ToyWindowForCausalLM", Cfg, build)
+    raw = {"architectures": ["ToyWindowForCausalLM"]}
+    (tmp_path / "config.json").write_text(json.dumps(raw))
+    tensors = random_tensors(DecoderModel(build(Cfg(raw))).weights(), seed=9, std=0.1)
+    save_file(tensors, str(tmp_path / "model.safetensors"))
+    w = {k: v.double().numpy() for k, v in tensors.items()}
+
+    toks = np.random.default_rng(3).integers(0, V, 150).tolist()
+    n = len(toks)
+    cos, sin = P.rope_cos_sin(np.arange(n), P.rope_inv_freq(D, 10000.0, None))
+    h = w["emb.weight"][toks]
+    for i, window in enumerate((WINDOW, None)):
+        p = f"l{i}."
+        x = P.rms_norm(h, w[p + "n1.weight"], 1e-5)
+        q = P.apply_rope((x @ w[p + "q.weight"].T).reshape(n, HQ, D), cos, sin)
+        k = P.apply_rope((x @ w[p + "k.weight"].T).reshape(n, HKV, D), cos, sin)
+        v = (x @ w[p + "v.weight"].T).reshape(n, HKV, D)
+        h = h + P.causal_attention(q, k, v, window).reshape(n, HQ * D) @ w[p + "o.weight"].T
+        x = P.rms_norm(h, w[p + "n2.weight"], 1e-5)
+        h = h + P.swiglu_mlp(x, w[p + "g.weight"], w[p + "u.weight"], w[p + "d.weight"])
+    want = P.rms_norm(h, w["norm.weight"], 1e-5) @ w["emb.weight"].T
+
+    for dtype, tol in (("float32", 1e-5), ("bfloat16", 4e-2)):
+        # group of the full layer: 10 pages (150 tokens); group of the window layer: 5 pages only
+        runner = ModelRunner(tmp_path, dtype=dtype, device="cuda:0", num_blocks=[5, 10], max_seq_len=160,
+                             max_num_seqs=2, use_graphs=True)
+        windows = runner.windows
+        assert sorted(windows, key=lambda x: (x is None, x)) == [WINDOW, None]
+        if windows[0] is None:                                     # group order follows the cache entries
+            runner = ModelRunner(tmp_path, dtype=dtype, device="cuda:0", num_blocks=[10, 5], max_seq_len=160,
+                                 max_num_seqs=2, use_graphs=True)
+        for cuts in ([16] * 9 + [6], [5, 2, 16, 1, 1, 1, 30, 3] + [1] * 40 + [16, 16, 16, 2, 1]):
+            assert sum(cuts) == n
+            rp = TraceReplayer(runner)
+            assert not rp.cache.prefix_cache                       # a window switches the prefix cache off
+            p0, worst = 0, 0.0
+            for kk, c in enumerate(cuts):
+                got = rp.run_step({"step": kk, "entries": [{"id": "a", "tokens": toks[p0:p0 + c], "want": list(range(c))}],
+                                   "end": ["a"] if p0 + c == n else []})
+                err = np.abs(got - want[p0:p0 + c]).max(-1) / np.abs(want[p0:p0 + c]).max(-1)
+                assert err.max() < tol, f"{dtype} positions {p0}..{p0 + c}: {err.max():.3e}"
+                p0 += c
+            assert all(rp.cache.num_free(g) == rp.cache.num_blocks(g) for g in range(2))
