@@ -103,26 +103,36 @@ __device__ __forceinline__ float silu_f(float g) { return g / (1.f + __expf(-g))
 // and receives C[4 * (l / 16) + v][l % 16], v = 0..3; C rows are rows of w, C columns are
 // tokens. MT = number of 16-token column tiles. SWIGLU: w is [gate; up] with n_out rows each
 // and the result is silu(gate) * up.
-template <int MT, bool SWIGLU, bool SPLIT, typename TO>
+// RT = 16-row tiles of w per wave (2 when there are more than 16 tokens: the tokens loaded
+// for a k-step then serve twice as many rows, halving the traffic for x, which for 64 tokens
+// would otherwise be four times that for w).
+template <int MT, int RT, bool SWIGLU, bool SPLIT, typename TO>
 __global__ __launch_bounds__(256) void skinny_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                           TO* __restrict__ out, int M, int n_out, int K) {
   constexpr int NACC = SWIGLU ? 2 * MT : MT;
-  constexpr int U = MT == 1 ? 8 : (MT == 2 ? 4 : 2);
+  constexpr int U = MT == 1 ? 8 : (MT * RT <= 2 ? 4 : 2);
   __shared__ f32x4 red[SPLIT ? 4 : 1][NACC][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int n0 = SPLIT ? blockIdx.x * 16 : (blockIdx.x * 4 + wave) * 16;
-  if (!SPLIT && n0 >= n_out) return;
+  const int tile0 = (SPLIT ? blockIdx.x : blockIdx.x * 4 + wave) * RT;
+  if (!SPLIT && tile0 * 16 >= n_out) return;
   const int r = lane & 15, g = lane >> 4;
-  const int row = min(n0 + r, n_out - 1);
-  const bf16_t* wrow = w + static_cast<int64_t>(row) * K + 8 * g;
-  const bf16_t* wrow_up = SWIGLU ? w + static_cast<int64_t>(n_out + row) * K + 8 * g : nullptr;
+  const bf16_t* wrow[RT];
+  const bf16_t* wrow_up[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int row = min((tile0 + rt) * 16 + r, n_out - 1);
+    wrow[rt] = w + static_cast<int64_t>(row) * K + 8 * g;
+    wrow_up[rt] = SWIGLU ? w + static_cast<int64_t>(n_out + row) * K + 8 * g : nullptr;
+  }
   const bf16_t* xrow[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) xrow[mt] = x + static_cast<int64_t>(min(mt * 16 + r, M - 1)) * K + 8 * g;
 
-  f32x4 acc[NACC];
+  f32x4 acc[RT][NACC];
 #pragma unroll
-  for (int i = 0; i < NACC; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int i = 0; i < NACC; ++i) acc[rt][i] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   const int steps = (K + 31) >> 5;
   const int per_wg = (steps + gridDim.y - 1) / gridDim.y;
@@ -131,19 +141,25 @@ __global__ __launch_bounds__(256) void skinny_mfma_kernel(const bf16_t* __restri
   const int s_full = min(s_end, K >> 5);          // steps that lie wholly inside K
   const int stride = SPLIT ? 4 : 1;
   for (int base = s_begin + (SPLIT ? wave : 0); base < s_full; base += stride * U) {
-    bf16x8 a[U], a_up[U], b[MT][U];
+    bf16x8 a[RT][U], a_up[RT][U], b[MT][U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int s = base + stride * u;
       if (s < s_full) {
         const int k = s << 5;
-        a[u] = load8(wrow + k);
-        if (SWIGLU) a_up[u] = load8(wrow_up + k);
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+          a[rt][u] = load8(wrow[rt] + k);
+          if (SWIGLU) a_up[rt][u] = load8(wrow_up[rt] + k);
+        }
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) b[mt][u] = load8(xrow[mt] + k);
       } else {
-        a[u] = zero8();
-        if (SWIGLU) a_up[u] = zero8();
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+          a[rt][u] = zero8();
+          if (SWIGLU) a_up[rt][u] = zero8();
+        }
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) b[mt][u] = zero8();
       }
@@ -151,9 +167,13 @@ __global__ __launch_bounds__(256) void skinny_mfma_kernel(const bf16_t* __restri
 #pragma unroll
     for (int u = 0; u < U; ++u) {
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b[mt][u], acc[mt], 0, 0, 0);
-        if (SWIGLU) acc[MT + mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_up[u], b[mt][u], acc[MT + mt], 0, 0, 0);
+      for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          acc[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[rt][u], b[mt][u], acc[rt][mt], 0, 0, 0);
+          if (SWIGLU)
+            acc[rt][MT + mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_up[rt][u], b[mt][u], acc[rt][MT + mt], 0, 0, 0);
+        }
       }
     }
   }
@@ -161,18 +181,21 @@ __global__ __launch_bounds__(256) void skinny_mfma_kernel(const bf16_t* __restri
   if (s_full < s_end && (!SPLIT || ((s_full - s_begin) & 3) == wave)) {
     const int k = s_full << 5;
     const bool in = k + 8 * g < K;
-    const bf16x8 a = in ? load8(wrow + k) : zero8();
-    bf16x8 a_up = zero8();
-    if (SWIGLU && in) a_up = load8(wrow_up + k);
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const bf16x8 b = in ? load8(xrow[mt] + k) : zero8();
-      acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mt], 0, 0, 0);
-      if (SWIGLU) acc[MT + mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_up, b, acc[MT + mt], 0, 0, 0);
+    for (int rt = 0; rt < RT; ++rt) {
+      const bf16x8 a = in ? load8(wrow[rt] + k) : zero8();
+      bf16x8 a_up = zero8();
+      if (SWIGLU && in) a_up = load8(wrow_up[rt] + k);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const bf16x8 b = in ? load8(xrow[mt] + k) : zero8();
+        acc[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[rt][mt], 0, 0, 0);
+        if (SWIGLU) acc[rt][MT + mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_up, b, acc[rt][MT + mt], 0, 0, 0);
+      }
     }
   }
 
-  auto finish = [&](int mt, f32x4 sum, f32x4 up) {
+  auto finish = [&](int rt, int mt, f32x4 sum, f32x4 up) {
     if (SWIGLU) {
 #pragma unroll
       for (int v = 0; v < 4; ++v) sum[v] = silu_f(sum[v]) * up[v];
@@ -182,41 +205,48 @@ __global__ __launch_bounds__(256) void skinny_mfma_kernel(const bf16_t* __restri
     TO* dst = out + (static_cast<int64_t>(blockIdx.y) * M + m) * n_out;
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
-      const int n = n0 + 4 * g + v;
+      const int n = (tile0 + rt) * 16 + 4 * g + v;
       if (n < n_out) dst[n] = from_float<TO>(sum[v]);
     }
   };
 
   if (!SPLIT) {
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) finish(mt, acc[mt], SWIGLU ? acc[MT + mt] : acc[mt]);
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) finish(rt, mt, acc[rt][mt], SWIGLU ? acc[rt][MT + mt] : acc[rt][mt]);
     return;
   }
 #pragma unroll
-  for (int i = 0; i < NACC; ++i) red[wave][i][lane] = acc[i];
-  __syncthreads();
-  // Wave `wave` finishes column tile `wave` (MT <= 4: at most one each).
-  if (wave >= MT) return;
-  const int mt = wave;
-  const f32x4 sum = red[0][mt][lane] + red[1][mt][lane] + red[2][mt][lane] + red[3][mt][lane];
-  f32x4 up = sum;
-  if (SWIGLU) up = red[0][MT + mt][lane] + red[1][MT + mt][lane] + red[2][MT + mt][lane] + red[3][MT + mt][lane];
-  finish(mt, sum, up);
+  for (int rt = 0; rt < RT; ++rt) {
+    if (rt > 0) __syncthreads();
+#pragma unroll
+    for (int i = 0; i < NACC; ++i) red[wave][i][lane] = acc[rt][i];
+    __syncthreads();
+    // Wave `wave` finishes column tile `wave` (MT <= 4: at most one each).
+    if (wave < MT) {
+      const int mt = wave;
+      const f32x4 sum = red[0][mt][lane] + red[1][mt][lane] + red[2][mt][lane] + red[3][mt][lane];
+      f32x4 up = sum;
+      if (SWIGLU) up = red[0][MT + mt][lane] + red[1][MT + mt][lane] + red[2][MT + mt][lane] + red[3][MT + mt][lane];
+      finish(rt, mt, sum, up);
+    }
+  }
 }
 
-template <int MT, bool SPLIT>
+template <int MT, int RT, bool SPLIT>
 static int launch_skinny2(hipStream_t s, const void* x, const void* w, void* out, int out_dtype, int M, int n_out,
                           int K, int epilogue, int ksplit) {
-  const int64_t tiles = ceil_div(n_out, 16);
-  const dim3 grid(static_cast<unsigned>(SPLIT ? tiles : ceil_div(tiles, 4)), static_cast<unsigned>(ksplit)), block(256);
+  const int64_t groups = ceil_div(ceil_div(n_out, 16), RT);
+  const dim3 grid(static_cast<unsigned>(SPLIT ? groups : ceil_div(groups, 4)), static_cast<unsigned>(ksplit)), block(256);
   const bf16_t* xp = static_cast<const bf16_t*>(x);
   const bf16_t* wp = static_cast<const bf16_t*>(w);
   if (epilogue == 1) {
-    skinny_mfma_kernel<MT, true, SPLIT, bf16_t><<<grid, block, 0, s>>>(xp, wp, static_cast<bf16_t*>(out), M, n_out, K);
+    skinny_mfma_kernel<MT, RT, true, SPLIT, bf16_t><<<grid, block, 0, s>>>(xp, wp, static_cast<bf16_t*>(out), M, n_out, K);
   } else if (out_dtype == kBF16) {
-    skinny_mfma_kernel<MT, false, SPLIT, bf16_t><<<grid, block, 0, s>>>(xp, wp, static_cast<bf16_t*>(out), M, n_out, K);
+    skinny_mfma_kernel<MT, RT, false, SPLIT, bf16_t><<<grid, block, 0, s>>>(xp, wp, static_cast<bf16_t*>(out), M, n_out, K);
   } else {
-    skinny_mfma_kernel<MT, false, SPLIT, float><<<grid, block, 0, s>>>(xp, wp, static_cast<float*>(out), M, n_out, K);
+    skinny_mfma_kernel<MT, RT, false, SPLIT, float><<<grid, block, 0, s>>>(xp, wp, static_cast<float*>(out), M, n_out, K);
   }
   return check_launch("psamd_linear_skinny");
 }
@@ -224,9 +254,10 @@ static int launch_skinny2(hipStream_t s, const void* x, const void* w, void* out
 template <int MT>
 static int launch_skinny(hipStream_t s, const void* x, const void* w, void* out, int out_dtype, int M, int n_out,
                          int K, int epilogue, int ksplit) {
-  // Enough 16-row tiles to fill the chip with one wave each: no need to split K inside a workgroup.
-  if (ceil_div(n_out, 16) >= 2048) return launch_skinny2<MT, false>(s, x, w, out, out_dtype, M, n_out, K, epilogue, ksplit);
-  return launch_skinny2<MT, true>(s, x, w, out, out_dtype, M, n_out, K, epilogue, ksplit);
+  constexpr int RT = MT >= 2 ? 2 : 1;
+  // Enough row groups to fill the chip with one wave each: no need to split K inside a workgroup.
+  if (ceil_div(ceil_div(n_out, 16), RT) >= 2048) return launch_skinny2<MT, RT, false>(s, x, w, out, out_dtype, M, n_out, K, epilogue, ksplit);
+  return launch_skinny2<MT, RT, true>(s, x, w, out, out_dtype, M, n_out, K, epilogue, ksplit);
 }
 
 // The q/k/v projection of a small step fused with what follows it: rotary encoding of q and

@@ -209,8 +209,8 @@ class HipOps:
         m, k = x.shape
         n = w.shape[0]
         if x.dtype == torch.bfloat16 and k % 8 == 0 and 0 < m <= self.SKINNY_MAX_ROWS:
-            tiles, steps = -(-n // 16), -(-k // 32)
-            ksplit = max(1, min(8, 512 // tiles, steps // 8))
+            groups, steps = -(-n // (16 if m <= 16 else 32)), -(-k // 32)   # workgroups before splitting K
+            ksplit = max(1, min(8, 512 // groups, steps // 8))
             if ksplit > 1:
                 self._need(w.shape[1] == k and x.is_contiguous() and w.is_contiguous(), "linear_to_residual: operands")
                 out = self.ws.get(name, (ksplit, m, n), torch.float32)
