@@ -118,22 +118,21 @@ class StepPacker:
         p_caps = [static_pages if static_pages is not None else p for p in pages]
         p_total = sum(p_caps)
 
-        # ---- host checks ----
-        for it, tk, n, e, pg in zip(items, toks, lens, ends, pages):
+        # ---- host checks (per item: cheap scalar ones; ranges of ids and pages: once per array below) ----
+        max_slot = max(self.num_slots, 1)
+        for it, n, e, pg in zip(items, lens, ends, pages):
             if it.start < 0 or e > self.max_position:
                 raise EngineError(f"{it.key}: positions [{it.start}, {e}) outside [0, {self.max_position})")
-            if int(tk.min()) < 0 or int(tk.max()) >= self.vocab_size:
-                raise EngineError(f"{it.key}: token id outside [0, {self.vocab_size})")
-            if not 0 <= int(it.slot) < max(self.num_slots, 1):
+            if not 0 <= it.slot < max_slot:
                 raise EngineError(f"{it.key}: state slot {it.slot} outside [0, {self.num_slots})")
             if len(it.block_tables) != g_n:
                 raise EngineError(f"{it.key}: {len(it.block_tables)} block tables for {g_n} layer groups")
             for w in it.want:
-                if not 0 <= int(w) < n:
+                if not 0 <= w < n:
                     raise EngineError(f"{it.key}: wanted place {w} outside its {n} tokens")
             if static_pages is not None and pg > static_pages:
                 raise EngineError(f"{it.key}: needs {pg} pages, static layout has {static_pages}")
-            for gi, (gm, table) in enumerate(zip(self.groups, it.block_tables)):
+            for gi, table in enumerate(it.block_tables):
                 if len(table) < pg:
                     raise EngineError(f"{it.key}: {len(table)} blocks in group {gi} for {e} tokens")
 
@@ -167,50 +166,56 @@ class StepPacker:
         item_start, item_pos0 = buf[sl["item_start"]], buf[sl["item_pos0"]]
         item_end, slots = buf[sl["item_end"]], buf[sl["slots"]]
         rows, dec, tiles = buf[sl["logit_rows"]], buf[sl["dec_items"]], buf[sl["pf_tiles"]]
+        # Absolute positions: a request that reused a prefix or resumes after preemption does
+        # not restart at 0 (prefixserve/llama_engine.py:190-193).
+        starts = [int(it.start) for it in items]
         item_start[0] = 0
-        t0 = r0 = d0 = q0 = 0
-        for i, (it, tk, n, e) in enumerate(zip(items, toks, lens, ends)):
-            ids[t0:t0 + n] = tk
-            # Absolute positions: a request that reused a prefix or resumes after
-            # preemption does not restart at 0 (prefixserve/llama_engine.py:190-193).
-            pos[t0:t0 + n] = np.arange(it.start, e, dtype=np.int32)
-            tok_item[t0:t0 + n] = i
-            item_start[i + 1] = t0 + n
-            item_pos0[i], item_end[i], slots[i] = it.start, e, it.slot
-            for w in it.want:
-                rows[r0] = t0 + int(w)
-                r0 += 1
-            if n == 1:
-                dec[d0] = i
-                d0 += 1
-            else:
-                for q in range(0, n, tile):
-                    tiles[2 * q0], tiles[2 * q0 + 1] = i, q
-                    q0 += 1
-            t0 += n
+        item_start[1:] = np.cumsum(lens)
+        item_pos0[:], item_end[:], slots[:] = starts, ends, [it.slot for it in items]
+        if n_dec == b:
+            ids[:] = [tk[0] for tk in toks]
+            pos[:] = starts
+            tok_item[:] = np.arange(b, dtype=np.int32)
+        else:
+            ids[:] = np.concatenate(toks)
+            tok_item[:] = np.repeat(np.arange(b, dtype=np.int32), lens)
+            pos[:] = item_pos0[tok_item] + (np.arange(t_n, dtype=np.int32) - item_start[tok_item])
+        dec[:] = [i for i, n in enumerate(lens) if n == 1]
+        tiles[:] = [x for i, n in enumerate(lens) if n > 1 for q in range(0, n, tile) for x in (i, q)]
+        rows[:] = [t0 + w for t0, it in zip(item_start[:-1].tolist(), items) for w in it.want]
+        if int(ids.min()) < 0 or int(ids.max()) >= self.vocab_size:
+            bad = next(it.key for it, tk in zip(items, toks) if int(tk.min()) < 0 or int(tk.max()) >= self.vocab_size)
+            raise EngineError(f"{bad}: token id outside [0, {self.vocab_size})")
 
         for gi, (gm, gs) in enumerate(zip(self.groups, gsl)):
             table_off, wslot, bids = buf[gs["table_off"]], buf[gs["write_slot"]], buf[gs["block_ids"]]
             table_off[0] = 0
-            p0 = t0 = 0
-            for i, (it, n, e, pg, cap) in enumerate(zip(items, lens, ends, pages, p_caps)):
-                table = np.asarray(it.block_tables[gi][:pg], dtype=np.int64)
+            table_off[1:] = np.cumsum(p_caps)
+            if static_pages is not None:
+                bids[:] = 0
+            p0 = 0
+            for it, s0, pg, cap in zip(items, starts, pages, p_caps):
+                table = it.block_tables[gi]
+                if not isinstance(table, np.ndarray):
+                    table = np.asarray(table[:pg], dtype=np.int64)
                 # Pages a token of this step can see or writes: all of them, or for a window
-                # group those from the window of the first new token on.
-                first_needed = 0
-                if gm.window is not None:
-                    first_needed = max(0, it.start - gm.window + 1) // PAGE
-                live = table[first_needed:]
-                if live.size and (int(live.min()) < 0 or int(live.max()) >= gm.num_blocks):
-                    raise EngineError(f"{it.key}: block id outside the pool of group {gi} (0..{gm.num_blocks - 1})")
-                bids[p0:p0 + pg] = np.where(table < 0, 0, table) if first_needed else table
-                if cap > pg:
-                    bids[p0 + pg:p0 + cap] = 0
-                p = np.arange(it.start, e)
-                wslot[t0:t0 + n] = table[p // PAGE] * PAGE + p % PAGE
+                # group those from the window of the first new token on; earlier entries may be
+                # -1 (given back) and are never read.
+                if gm.window is None:
+                    bids[p0:p0 + pg] = table[:pg]
+                else:
+                    first_needed = max(0, s0 - gm.window + 1) // PAGE
+                    bids[p0:p0 + first_needed] = 0
+                    bids[p0 + first_needed:p0 + pg] = table[first_needed:pg]
                 p0 += cap
-                t0 += n
-                table_off[i + 1] = p0
+            if int(bids.min()) < 0 or int(bids.max()) >= gm.num_blocks:
+                p0 = 0
+                for it, pg, cap in zip(items, pages, p_caps):        # name the request that brought it
+                    row = bids[p0:p0 + pg]
+                    if row.size and (int(row.min()) < 0 or int(row.max()) >= gm.num_blocks):
+                        raise EngineError(f"{it.key}: block id outside the pool of group {gi} (0..{gm.num_blocks - 1})")
+                    p0 += cap
+            wslot[:] = bids[table_off[tok_item] + pos // PAGE] * PAGE + pos % PAGE
 
         # ---- one copy ----
         if self.on_gpu:

@@ -10,6 +10,7 @@ from dataclasses import dataclass
 from pathlib import Path
 from typing import Any
 
+import numpy as np
 import torch
 
 from prefixserve_amd.cache.manager import CacheManager
@@ -44,6 +45,9 @@ class Engine:
         self.sampler = Sampler(self.runner.ops, self.runner.device, max(cfg.max_num_seqs, 1))
         self.capture_logits = False
         self.last_logits: dict[str, torch.Tensor] = {}
+        # req_id -> (preemption count, [(array, filled)] per group): block tables as arrays,
+        # extended as the lists grow, so a step does not convert whole lists again.
+        self._tables: dict[str, tuple[int, list[list]]] = {}
 
     @property
     def num_blocks(self) -> int:
@@ -69,6 +73,31 @@ class Engine:
                          chunk_size=chunk_size if chunk_size is not None else self.cfg.max_prefill_tokens,
                          stop_token_ids=self.stop_token_ids)
 
+    def _table_arrays(self, req) -> list:
+        """The request's block tables as int64 arrays. A request's tables only grow while it
+        runs; after a preemption it gets new ones, which the preemption count tells."""
+        entry = self._tables.get(req.req_id)
+        if entry is None or entry[0] != req.num_preemptions or len(entry[1]) != len(req.block_tables):
+            entry = (req.num_preemptions, [[np.empty(64, dtype=np.int64), 0] for _ in req.block_tables])
+            if len(self._tables) > 8 * self.cfg.max_num_seqs:
+                self._tables.clear()           # finished requests leave entries behind
+            self._tables[req.req_id] = entry
+        out = []
+        for slot, table in zip(entry[1], req.block_tables):
+            arr, filled = slot
+            n = len(table)
+            if n > arr.size:
+                grown = np.empty(max(n, 2 * arr.size), dtype=np.int64)
+                grown[:filled] = arr[:filled]
+                arr = slot[0] = grown
+            if n < filled:
+                filled = 0
+            if n > filled:
+                arr[filled:n] = table[filled:n]
+                slot[1] = n
+            out.append(arr[:n])
+        return out
+
     def step(self, batch: Batch) -> dict[str, int]:
         """Runs one batch; returns req_id -> next token for the items that sample."""
         if not batch.work:
@@ -81,7 +110,7 @@ class Engine:
             if w.end > self.cfg.max_seq_len:
                 raise EngineError(f"{req.req_id}: position {w.end} > max_seq_len {self.cfg.max_seq_len}")
             items.append(StepItem(key=req.req_id, tokens=req.tokens(w.start, w.end), start=w.start,
-                                  block_tables=req.block_tables, slot=max(req.slot, 0),
+                                  block_tables=self._table_arrays(req), slot=max(req.slot, 0),
                                   want=[n - 1] if w.samples else []))
             if w.samples:
                 sampling.append(req)

@@ -65,7 +65,7 @@ def test_packer_refuses_bad_batches():
     for change, needle in [
         (dict(block_tables=[[8]]), "outside the pool"), (dict(block_tables=[[-1]]), "outside the pool"),
         (dict(block_tables=[[]]), "blocks in group"), (dict(block_tables=[[0], [0]]), "block tables"),
-        (dict(tokens=[100]), "token id"), (dict(tokens=[]), "no tokens"), (dict(start=62), "positions"),
+        (dict(tokens=[100], want=[0]), "token id"), (dict(tokens=[]), "no tokens"), (dict(start=62), "positions"),
         (dict(want=[3]), "wanted place"), (dict(slot=2), "state slot"), (dict(start=-1), "positions"),
     ]:
         with pytest.raises(EngineError, match=needle):
