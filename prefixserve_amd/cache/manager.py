@@ -121,11 +121,14 @@ class CacheManager:
             first_visible = next_position - w + 1
             last_dead_page = first_visible // BLOCK_SIZE  # pages [0, last_dead_page) lie wholly before it
             table = tables[g]
-            for j in range(min(max(last_dead_page, 0), len(table))):
-                if table[j] >= 0:
-                    self.pools[g].decref(table[j])
-                    table[j] = -1
-                    freed += 1
+            # Pages go back in order, so the entries already given back are a prefix of the
+            # table: walk down from the newest dead page until one of them.
+            j = min(max(last_dead_page, 0), len(table)) - 1
+            while j >= 0 and table[j] >= 0:
+                self.pools[g].decref(table[j])
+                table[j] = -1
+                freed += 1
+                j -= 1
         return freed
 
     def evict_all(self) -> int:

@@ -7,7 +7,9 @@
 
 #include <pybind11/numpy.h>
 #include <pybind11/pybind11.h>
+#include <pybind11/stl.h>
 
+#include <deque>
 #include <memory>
 #include <stdexcept>
 #include <string>
@@ -15,6 +17,7 @@
 
 #include "block_pool.hpp"
 #include "prefix_tree.hpp"
+#include "step_pack.hpp"
 
 namespace py = pybind11;
 using namespace psamd;
@@ -78,6 +81,96 @@ class TreeHandle {
   PrefixTree tree_;
   std::vector<BlockId> found_;
 };
+
+using Longs = py::array_t<int64_t, py::array::c_style | py::array::forcecast>;
+
+// Integer sequences of a call as 64-bit spans: arrays are borrowed (converted if their type
+// differs), lists and tuples are copied. Everything lives until the holder dies.
+struct Borrowed {
+  std::vector<Longs> arrays;
+  std::deque<std::vector<int64_t>> copies;
+
+  Span of(const py::handle& seq, const char* name) {
+    PyObject* o = seq.ptr();
+    if (PyList_Check(o) || PyTuple_Check(o)) {
+      const Py_ssize_t n = PySequence_Fast_GET_SIZE(o);
+      PyObject** elems = PySequence_Fast_ITEMS(o);
+      std::vector<int64_t>& v = copies.emplace_back(static_cast<size_t>(n));
+      for (Py_ssize_t i = 0; i < n; ++i) {
+        v[static_cast<size_t>(i)] = PyLong_AsLongLong(elems[i]);
+        if (v[static_cast<size_t>(i)] == -1 && PyErr_Occurred()) {
+          PyErr_Clear();
+          // Not plain Python integers (numpy scalars, say): let numpy convert the lot.
+          copies.pop_back();
+          return of_array(seq, name);
+        }
+      }
+      return Span{v.data(), static_cast<int64_t>(n)};
+    }
+    return of_array(seq, name);
+  }
+
+  Span of_array(const py::handle& seq, const char* name) {
+    Longs a = Longs::ensure(seq);
+    if (!a) {
+      PyErr_Clear();
+      throw py::value_error(std::string(name) + " must be a sequence of integers");
+    }
+    if (a.ndim() != 1) a = a.attr("reshape")(-1).cast<Longs>();
+    arrays.push_back(a);
+    return Span{a.data(), static_cast<int64_t>(a.size())};
+  }
+};
+
+// pack_step(buffer, items, groups, vocab_size, max_position, num_slots, prefill_tile,
+// static_pages) -> None if the buffer is too small, in which case only the first number
+// of the result counts, else the layout as a tuple of integers.
+py::tuple pack_step(py::array_t<int32_t, py::array::c_style> buffer, const py::sequence& items,
+                    const std::vector<std::pair<int64_t, py::object>>& groups, int64_t vocab_size,
+                    int64_t max_position, int64_t num_slots, int64_t prefill_tile, const py::object& static_pages) {
+  std::vector<PackGroup> gs;
+  for (const auto& g : groups) gs.push_back(PackGroup{g.first, g.second.is_none() ? -1 : g.second.cast<int64_t>()});
+  PackLimits lim;
+  lim.vocab_size = vocab_size;
+  lim.max_position = max_position;
+  lim.num_slots = num_slots;
+  lim.prefill_tile = prefill_tile;
+  lim.static_pages = static_pages.is_none() ? -1 : static_pages.cast<int64_t>();
+
+  Borrowed keep;
+  std::vector<PackItem> its;
+  const size_t n_items = py::len(items);
+  its.reserve(n_items);
+  keep.arrays.reserve(n_items * (2 + gs.size()));
+  // Attribute names as Python strings made once: this runs for every item of every step.
+  static const py::str k_tokens("tokens"), k_start("start"), k_slot("slot"), k_tables("block_tables"), k_want("want");
+  for (const py::handle& obj : items) {
+    PackItem it;
+    it.tokens = keep.of(obj.attr(k_tokens), "tokens");
+    it.start = obj.attr(k_start).cast<int64_t>();
+    it.slot = obj.attr(k_slot).cast<int64_t>();
+    it.tables.reserve(gs.size());
+    for (const py::handle& table : obj.attr(k_tables)) it.tables.push_back(keep.of(table, "a block table"));
+    it.want = keep.of(obj.attr(k_want), "want");
+    its.push_back(std::move(it));
+  }
+  try {
+    const PackLayout lay = plan_step(its, gs, lim);
+    const bool fits = lay.total <= buffer.size();
+    if (fits) fill_step(its, gs, lim, lay, buffer.mutable_data());
+    py::list group_offsets;
+    for (const GroupLayout& g : lay.groups) group_offsets.append(py::make_tuple(g.table_off, g.write_slot, g.block_ids));
+    return py::make_tuple(fits, lay.total, lay.tokens, lay.items, lay.logit_rows, lay.decode_items,
+                          lay.prefill_tiles, lay.pages, lay.max_kv_len,
+                          py::make_tuple(lay.token_ids, lay.positions, lay.tok_item, lay.item_start, lay.item_pos0,
+                                         lay.item_end, lay.slots, lay.logit_rows_off, lay.dec_items, lay.pf_tiles),
+                          group_offsets);
+  } catch (const PackError& e) {
+    std::string who;
+    if (e.item >= 0) who = py::str(items[static_cast<size_t>(e.item)].attr("key")).cast<std::string>() + ": ";
+    throw py::value_error(who + e.what());
+  }
+}
 
 }  // namespace
 
@@ -144,6 +237,10 @@ PYBIND11_MODULE(_core, m) {
       .def("is_cached", &TreeHandle::is_cached, py::arg("block_id"))
       .def_property_readonly("num_cached_blocks", &TreeHandle::cached)
       .def("check_invariants", &TreeHandle::check);
+
+  m.def("pack_step", &pack_step, py::arg("buffer"), py::arg("items"), py::arg("groups"), py::arg("vocab_size"),
+        py::arg("max_position"), py::arg("num_slots"), py::arg("prefill_tile"), py::arg("static_pages") = py::none(),
+        "Checks a step's items and lays their integer arrays out in one buffer.");
 
   py::class_<StateSlots>(m, "StateSlots")
       .def(py::init<int32_t, int64_t>(), py::arg("num_slots"), py::arg("bytes_per_slot") = 0)

@@ -23,16 +23,41 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __r
   const float* row = logits + static_cast<int64_t>(blockIdx.x) * vocab;
   const float temp = temperature[blockIdx.x];
 
-  // ---- max and its first index
+  // ---- max and its first index. The body of the row is read as aligned groups of four,
+  // several loads in flight per thread; a row need not start on a 16-byte boundary.
   float best = -INFINITY;
   int32_t best_i = 0x7fffffff;
-  for (int i = tid; i < vocab; i += kSampleThreads) {
-    const float v = row[i];
+  auto take = [&](float v, int32_t i) {
     if (v > best || (v == best && i < best_i)) {
       best = v;
       best_i = i;
     }
+  };
+  const int head = min(vocab, static_cast<int>((4 - ((reinterpret_cast<uintptr_t>(row) >> 2) & 3)) & 3));
+  const int quads = (vocab - head) / 4;
+  if (tid < head) take(row[tid], tid);
+  const float4* body = reinterpret_cast<const float4*>(row + head);
+  constexpr int kInFlight = 4;
+  for (int q0 = tid; q0 < quads; q0 += kSampleThreads * kInFlight) {
+    float4 v[kInFlight];
+#pragma unroll
+    for (int u = 0; u < kInFlight; ++u) {
+      const int q = q0 + u * kSampleThreads;
+      v[u] = body[min(q, quads - 1)];
+    }
+#pragma unroll
+    for (int u = 0; u < kInFlight; ++u) {
+      const int q = q0 + u * kSampleThreads;
+      if (q < quads) {
+        const int i = head + 4 * q;
+        take(v[u].x, i);
+        take(v[u].y, i + 1);
+        take(v[u].z, i + 2);
+        take(v[u].w, i + 3);
+      }
+    }
   }
+  for (int i = head + 4 * quads + tid; i < vocab; i += kSampleThreads) take(row[i], i);
 #pragma unroll
   for (int o = kWave / 2; o > 0; o >>= 1) {
     const float ob = __shfl_xor(best, o, kWave);

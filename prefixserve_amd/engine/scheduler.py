@@ -95,13 +95,14 @@ class Request:
             return self.prompt
         return np.concatenate((self.prompt, np.asarray(self.output, dtype=np.int32)))
 
-    def tokens(self, start: int, end: int) -> np.ndarray:
-        """seq[start:end] without building the whole sequence."""
+    def tokens(self, start: int, end: int) -> np.ndarray | list[int]:
+        """seq[start:end] without building the whole sequence: an array, or a list when all
+        of it is output (every decode step asks for that; a slice of a list costs least)."""
         n = len(self.prompt)
         if end <= n:
             return self.prompt[start:end]
         if start >= n:
-            return np.asarray(self.output[start - n:end - n], dtype=np.int32)
+            return self.output[start - n:end - n]
         return np.concatenate((self.prompt[start:], np.asarray(self.output[:end - n], dtype=np.int32)))
 
 

@@ -50,10 +50,15 @@ class Sampler:
 
     def _alloc(self, rows: int) -> None:
         pin = self.device.type == "cuda"
-        self._host = torch.empty((2, rows), dtype=torch.float32, pin_memory=pin)
-        self._dev = torch.empty((2, rows), dtype=torch.float32, device=self.device)
+        # Temperatures, then uniform numbers: one contiguous host-to-device copy.
+        self._host = torch.empty(2 * rows, dtype=torch.float32, pin_memory=pin)
+        self._host_np = self._host.numpy()
+        self._dev = torch.zeros(2 * rows, dtype=torch.float32, device=self.device)
         self._out = torch.empty(rows, dtype=torch.int32, device=self.device)
+        self._out_host = torch.empty(rows, dtype=torch.int32, pin_memory=pin)
+        self._out_np = self._out_host.numpy()
         self.max_rows = rows
+        self._greedy_rows = rows     # leading rows of the device copy known to hold temperature 0
 
     def sample(self, logits: torch.Tensor, temperatures: Sequence[float], uniforms: Sequence[float]) -> list[int]:
         rows = logits.shape[0]
@@ -61,9 +66,21 @@ class Sampler:
             raise ValueError("one temperature and one uniform number per logits row")
         if rows > self.max_rows:
             self._alloc(max(rows, 2 * self.max_rows))
-        self._host[0, :rows] = torch.tensor(temperatures, dtype=torch.float32)
-        self._host[1, :rows] = torch.tensor(uniforms, dtype=torch.float32)
-        self._dev[:, :rows].copy_(self._host[:, :rows], non_blocking=True)
+        n = self.max_rows
+        greedy = not any(t > 0 for t in temperatures)
+        if not (greedy and self._greedy_rows >= rows):     # an all-greedy batch reads zeros already there
+            self._host_np[:rows] = temperatures
+            self._host_np[n:n + rows] = uniforms
+            if self.device.type == "cuda":
+                self._dev[:n + rows].copy_(self._host[:n + rows], non_blocking=True)
+            else:
+                self._dev[:n + rows] = self._host[:n + rows]
+            self._greedy_rows = rows if greedy else 0
         out = self._out[:rows]
-        self.ops.sample(logits, self._dev[0, :rows], self._dev[1, :rows], out)
-        return out.tolist()   # the step's one device-to-host wait
+        self.ops.sample(logits, self._dev[:rows], self._dev[n:n + rows], out)
+        # The step's one device-to-host wait.
+        if self.device.type == "cuda":
+            self._out_host[:rows].copy_(out, non_blocking=True)
+            torch.cuda.current_stream(self.device).synchronize()
+            return self._out_np[:rows].tolist()
+        return out.tolist()
