@@ -37,6 +37,22 @@ LLAMA_1B = {
 }
 
 
+def _llama3(hidden, inter, layers, heads, kv, dim, factor, tied):
+    cfg = dict(LLAMA_1B)
+    cfg.update(hidden_size=hidden, intermediate_size=inter, num_hidden_layers=layers, num_attention_heads=heads,
+               num_key_value_heads=kv, head_dim=dim, tie_word_embeddings=tied,
+               rope_scaling=dict(LLAMA_1B["rope_scaling"], factor=factor))
+    return cfg
+
+
+# The default is the 1B shape; the two larger ones show the kernels at another head size and width.
+SHAPES = {
+    "llama-3.2-1b": LLAMA_1B,
+    "llama-3.2-3b": _llama3(3072, 8192, 28, 24, 8, 128, 32.0, True),
+    "llama-3.1-8b": _llama3(4096, 14336, 32, 32, 8, 128, 8.0, False),
+}
+
+
 def prefill_flops(cfg: dict, layers: int, tokens: int) -> float:
     h, i, v = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
     hq, hkv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
@@ -59,6 +75,7 @@ def main() -> int:
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--prefill-reps", type=int, default=5, help="timed repetitions of the 2,048-token prefill")
     ap.add_argument("--model", default=None, help="use this model folder instead of writing random weights")
+    ap.add_argument("--shape", choices=sorted(SHAPES), default="llama-3.2-1b", help="layer sizes of the random model")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -70,7 +87,9 @@ def main() -> int:
     from prefixserve_amd import Engine, EngineConfig
     from prefixserve_amd.weights import write_random_model
 
-    cfg = dict(LLAMA_1B)
+    cfg = dict(SHAPES[args.shape])
+    if args.model is not None:
+        cfg = json.loads((Path(args.model) / "config.json").read_text())
     layers_full = cfg["num_hidden_layers"]
     if args.layers is not None:
         cfg["num_hidden_layers"] = args.layers
@@ -156,11 +175,11 @@ def main() -> int:
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
         "data": "synthetic: seeded uniform-random token ids, seeded random weights",
         "config": {
-            "model": "llama-3.2-1b-shape", "layers": layers_full, "layers_run": layers, "hidden": cfg["hidden_size"],
+            "model": (args.shape if args.model is None else Path(args.model).name) + "-shape", "layers": layers_full, "layers_run": layers, "hidden": cfg["hidden_size"],
             "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
             "intermediate": cfg["intermediate_size"], "vocab": vocab, "rope_theta": cfg["rope_theta"],
-            "rope_factor": cfg["rope_scaling"]["factor"], "rms_norm_eps": cfg["rms_norm_eps"],
-            "tied": cfg["tie_word_embeddings"], "global_batch": args.batch, "seq_len": args.context,
+            "rope_factor": (cfg.get("rope_scaling") or {}).get("factor"), "rms_norm_eps": cfg["rms_norm_eps"],
+            "tied": cfg.get("tie_word_embeddings", False), "global_batch": args.batch, "seq_len": args.context,
             "prompt_len": args.prompt_len, "page_tokens": 16, "parallelism": "none",
         },
         "prefill": prefill,
