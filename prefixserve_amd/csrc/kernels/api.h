@@ -39,6 +39,7 @@ int psamd_linear(void* stream, const void* x, int x_dtype, const void* w, int w_
 
 // bfloat16 product for M <= 64 on the matrix cores. epilogue 1: w = [gate; up], out = silu(gate) * up.
 // ksplit > 1: out receives ksplit float32 partial sums [ksplit][M, n_out] (plain epilogue only).
+int psamd_linear_skinny_ksplit(int M, int n_out, int K);
 int psamd_linear_skinny(void* stream, const void* x, const void* w, void* out, int out_dtype, int M, int n_out, int K,
                         int epilogue, int ksplit);
 

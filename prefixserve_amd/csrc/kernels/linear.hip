@@ -9,6 +9,8 @@
 //   16x16x32 matrix-core instruction with the M tokens as the other operand. Optional
 //   epilogue: SwiGLU over a fused [gate; up] matrix, or float32 output for logits.
 
+#include <algorithm>
+
 #include "api.h"
 #include "common.h"
 
@@ -106,14 +108,17 @@ __device__ __forceinline__ float silu_f(float g) { return g / (1.f + __expf(-g))
 // RT = 16-row tiles of w per wave (2 when there are more than 16 tokens: the tokens loaded
 // for a k-step then serve twice as many rows, halving the traffic for x, which for 64 tokens
 // would otherwise be four times that for w).
-template <int MT, int RT, bool SWIGLU, bool SPLIT, typename TO>
-__global__ __launch_bounds__(256) void skinny_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+// WV = waves of a workgroup (8 with many tokens: more k-slices in flight per workgroup).
+// U = k-steps whose loads are in flight together.
+constexpr int skinny_depth(int mt, int rt) { return mt == 1 ? 8 : (mt * rt <= 2 ? 4 : (mt * rt <= 8 ? 2 : 1)); }
+
+template <int MT, int RT, int WV, bool SWIGLU, bool SPLIT, typename TO, int U = skinny_depth(MT, RT)>
+__global__ __launch_bounds__(64 * WV) void skinny_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                           TO* __restrict__ out, int M, int n_out, int K) {
   constexpr int NACC = SWIGLU ? 2 * MT : MT;
-  constexpr int U = MT == 1 ? 8 : (MT * RT <= 2 ? 4 : 2);
-  __shared__ f32x4 red[SPLIT ? 4 : 1][NACC][64];
+  __shared__ f32x4 red[SPLIT ? WV : 1][NACC][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int tile0 = (SPLIT ? blockIdx.x : blockIdx.x * 4 + wave) * RT;
+  const int tile0 = (SPLIT ? blockIdx.x : blockIdx.x * WV + wave) * RT;
   if (!SPLIT && tile0 * 16 >= n_out) return;
   const int r = lane & 15, g = lane >> 4;
   const bf16_t* wrow[RT];
@@ -139,7 +144,7 @@ __global__ __launch_bounds__(256) void skinny_mfma_kernel(const bf16_t* __restri
   const int s_begin = blockIdx.y * per_wg;
   const int s_end = min(s_begin + per_wg, steps);
   const int s_full = min(s_end, K >> 5);          // steps that lie wholly inside K
-  const int stride = SPLIT ? 4 : 1;
+  const int stride = SPLIT ? WV : 1;
   for (int base = s_begin + (SPLIT ? wave : 0); base < s_full; base += stride * U) {
     bf16x8 a[RT][U], a_up[RT][U], b[MT][U];
 #pragma unroll
@@ -178,7 +183,7 @@ __global__ __launch_bounds__(256) void skinny_mfma_kernel(const bf16_t* __restri
     }
   }
   // K % 32 in {8, 16, 24}: the last step is partial; lane groups past the end contribute zeros.
-  if (s_full < s_end && (!SPLIT || ((s_full - s_begin) & 3) == wave)) {
+  if (s_full < s_end && (!SPLIT || ((s_full - s_begin) % WV) == wave)) {
     const int k = s_full << 5;
     const bool in = k + 8 * g < K;
 #pragma unroll
@@ -226,38 +231,58 @@ __global__ __launch_bounds__(256) void skinny_mfma_kernel(const bf16_t* __restri
     // Wave `wave` finishes column tile `wave` (MT <= 4: at most one each).
     if (wave < MT) {
       const int mt = wave;
-      const f32x4 sum = red[0][mt][lane] + red[1][mt][lane] + red[2][mt][lane] + red[3][mt][lane];
+      f32x4 sum = red[0][mt][lane];
+#pragma unroll
+      for (int w2 = 1; w2 < WV; ++w2) sum += red[w2][mt][lane];
       f32x4 up = sum;
-      if (SWIGLU) up = red[0][MT + mt][lane] + red[1][MT + mt][lane] + red[2][MT + mt][lane] + red[3][MT + mt][lane];
+      if (SWIGLU) {
+        up = red[0][MT + mt][lane];
+#pragma unroll
+        for (int w2 = 1; w2 < WV; ++w2) up += red[w2][MT + mt][lane];
+      }
       finish(rt, mt, sum, up);
     }
   }
 }
 
-template <int MT, int RT, bool SPLIT>
+template <int MT, int RT, int WV, bool SWIGLU, bool SPLIT>
 static int launch_skinny2(hipStream_t s, const void* x, const void* w, void* out, int out_dtype, int M, int n_out,
-                          int K, int epilogue, int ksplit) {
+                          int K, int ksplit) {
   const int64_t groups = ceil_div(ceil_div(n_out, 16), RT);
-  const dim3 grid(static_cast<unsigned>(SPLIT ? groups : ceil_div(groups, 4)), static_cast<unsigned>(ksplit)), block(256);
+  const dim3 grid(static_cast<unsigned>(SPLIT ? groups : ceil_div(groups, WV)), static_cast<unsigned>(ksplit)), block(64 * WV);
   const bf16_t* xp = static_cast<const bf16_t*>(x);
   const bf16_t* wp = static_cast<const bf16_t*>(w);
-  if (epilogue == 1) {
-    skinny_mfma_kernel<MT, RT, true, SPLIT, bf16_t><<<grid, block, 0, s>>>(xp, wp, static_cast<bf16_t*>(out), M, n_out, K);
+  if constexpr (SWIGLU) {
+    skinny_mfma_kernel<MT, RT, WV, true, SPLIT, bf16_t><<<grid, block, 0, s>>>(xp, wp, static_cast<bf16_t*>(out), M, n_out, K);
   } else if (out_dtype == kBF16) {
-    skinny_mfma_kernel<MT, RT, false, SPLIT, bf16_t><<<grid, block, 0, s>>>(xp, wp, static_cast<bf16_t*>(out), M, n_out, K);
+    skinny_mfma_kernel<MT, RT, WV, false, SPLIT, bf16_t><<<grid, block, 0, s>>>(xp, wp, static_cast<bf16_t*>(out), M, n_out, K);
   } else {
-    skinny_mfma_kernel<MT, RT, false, SPLIT, float><<<grid, block, 0, s>>>(xp, wp, static_cast<float*>(out), M, n_out, K);
+    skinny_mfma_kernel<MT, RT, WV, false, SPLIT, float><<<grid, block, 0, s>>>(xp, wp, static_cast<float*>(out), M, n_out, K);
   }
   return check_launch("psamd_linear_skinny");
+}
+
+// Row tiles per wave and waves per workgroup for MT column tiles of tokens. With more than
+// 32 tokens the tokens are most of a k-step's loads: a wave then takes four row tiles (the
+// SwiGLU form two of gate and two of up) and a workgroup eight k-slices.
+constexpr int skinny_rt(int mt, bool swiglu) { return mt == 1 ? 1 : (mt == 2 || swiglu ? 2 : 4); }
+constexpr int skinny_wv(int mt) { return mt <= 2 ? 4 : 8; }
+
+template <int MT, bool SWIGLU>
+static int launch_skinny1(hipStream_t s, const void* x, const void* w, void* out, int out_dtype, int M, int n_out,
+                          int K, int ksplit) {
+  constexpr int RT = skinny_rt(MT, SWIGLU), WV = skinny_wv(MT);
+  // Enough row groups to fill the chip with one wave each: no need to split K inside a workgroup.
+  if (ceil_div(ceil_div(n_out, 16), RT) >= 2048)
+    return launch_skinny2<MT, RT, WV, SWIGLU, false>(s, x, w, out, out_dtype, M, n_out, K, ksplit);
+  return launch_skinny2<MT, RT, WV, SWIGLU, true>(s, x, w, out, out_dtype, M, n_out, K, ksplit);
 }
 
 template <int MT>
 static int launch_skinny(hipStream_t s, const void* x, const void* w, void* out, int out_dtype, int M, int n_out,
                          int K, int epilogue, int ksplit) {
-  constexpr int RT = MT >= 2 ? 2 : 1;
-  // Enough row groups to fill the chip with one wave each: no need to split K inside a workgroup.
-  if (ceil_div(ceil_div(n_out, 16), RT) >= 2048) return launch_skinny2<MT, RT, false>(s, x, w, out, out_dtype, M, n_out, K, epilogue, ksplit);
-  return launch_skinny2<MT, RT, true>(s, x, w, out, out_dtype, M, n_out, K, epilogue, ksplit);
+  if (epilogue == 1) return launch_skinny1<MT, true>(s, x, w, out, out_dtype, M, n_out, K, ksplit);
+  return launch_skinny1<MT, false>(s, x, w, out, out_dtype, M, n_out, K, ksplit);
 }
 
 // The q/k/v projection of a small step fused with what follows it: rotary encoding of q and
@@ -268,39 +293,50 @@ static int launch_skinny(hipStream_t s, const void* x, const void* w, void* out,
 // first-half elements and groups 2-3 their partners, one shuffle apart.
 // qkv_out[m] receives the rotated q and k and v (the layout the attention kernels read q
 // from); k and v also go to page slot write_slot[m] when a cache is given.
-template <int MT>
-__global__ __launch_bounds__(256) void qkv_rope_append_kernel(
+// RT such tiles per workgroup and WV waves, as in skinny_mfma_kernel.
+template <int MT, int RT, int WV>
+__global__ __launch_bounds__(64 * WV) void qkv_rope_append_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, bf16_t* __restrict__ qkv_out, int M, int K, int hq,
     int hkv, int d, const int32_t* __restrict__ positions, const float2* __restrict__ table,
     bf16_t* __restrict__ kv, const int32_t* __restrict__ write_slot) {
-  __shared__ f32x4 red[4][MT][64];
+  __shared__ f32x4 red[WV][MT][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
   const int half = d >> 1;
   const int tiles_per_head = d >> 4;
-  const int head = blockIdx.x / tiles_per_head;
-  const int p = (blockIdx.x - head * tiles_per_head) << 3;          // first of 8 pair indices
-  const int row = head * d + (r < 8 ? p + r : half + p + r - 8);
-  const bf16_t* wrow = w + static_cast<int64_t>(row) * K + 8 * g;
+  const int n_tiles = (hq + 2 * hkv) * tiles_per_head;
+  const bf16_t* wrow[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int t = min(static_cast<int>(blockIdx.x) * RT + rt, n_tiles - 1);
+    const int head = t / tiles_per_head;
+    const int p = (t - head * tiles_per_head) << 3;                 // first of 8 pair indices
+    const int row = head * d + (r < 8 ? p + r : half + p + r - 8);
+    wrow[rt] = w + static_cast<int64_t>(row) * K + 8 * g;
+  }
   const bf16_t* xrow[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) xrow[mt] = x + static_cast<int64_t>(min(mt * 16 + r, M - 1)) * K + 8 * g;
-  f32x4 acc[MT];
+  f32x4 acc[RT][MT];
 #pragma unroll
-  for (int i = 0; i < MT; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int i = 0; i < MT; ++i) acc[rt][i] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int s_full = K >> 5;
-  constexpr int U = MT == 1 ? 8 : (MT == 2 ? 4 : 2);   // steps whose loads are in flight together
-  for (int base = wave; base < s_full; base += 4 * U) {
-    bf16x8 a[U], b[MT][U];
+  constexpr int U = MT == 1 ? 8 : (MT * RT <= 2 ? 4 : 2);   // steps whose loads are in flight together
+  for (int base = wave; base < s_full; base += WV * U) {
+    bf16x8 a[RT][U], b[MT][U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int s = base + 4 * u;
+      const int s = base + WV * u;
       if (s < s_full) {
-        a[u] = load8(wrow + (s << 5));
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) a[rt][u] = load8(wrow[rt] + (s << 5));
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) b[mt][u] = load8(xrow[mt] + (s << 5));
       } else {
-        a[u] = zero8();
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) a[rt][u] = zero8();
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) b[mt][u] = zero8();
       }
@@ -308,62 +344,93 @@ __global__ __launch_bounds__(256) void qkv_rope_append_kernel(
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b[mt][u], acc[mt], 0, 0, 0);
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          acc[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[rt][u], b[mt][u], acc[rt][mt], 0, 0, 0);
   }
-  if ((K & 31) != 0 && (s_full & 3) == wave) {
+  if ((K & 31) != 0 && (s_full % WV) == wave) {
     const int k = s_full << 5;
     const bool in = k + 8 * g < K;
-    const bf16x8 a = in ? load8(wrow + k) : zero8();
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const bf16x8 b = in ? load8(xrow[mt] + k) : zero8();
-      acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mt], 0, 0, 0);
+    for (int rt = 0; rt < RT; ++rt) {
+      const bf16x8 a = in ? load8(wrow[rt] + k) : zero8();
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const bf16x8 b = in ? load8(xrow[mt] + k) : zero8();
+        acc[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[rt][mt], 0, 0, 0);
+      }
     }
   }
 #pragma unroll
-  for (int i = 0; i < MT; ++i) red[wave][i][lane] = acc[i];
-  __syncthreads();
-  if (wave >= MT) return;
-  const int mt = wave;
-  const f32x4 own = red[0][mt][lane] + red[1][mt][lane] + red[2][mt][lane] + red[3][mt][lane];
-  const int m = mt * 16 + r;
-  const int mc = min(m, M - 1);
-  const bool second = g >= 2;
-  const bool rotate = table != nullptr && head < hq + hkv;
-  const int pos = positions[mc];
-  f32x4 res;
+  for (int rt = 0; rt < RT; ++rt) {
+    if (rt > 0) __syncthreads();
 #pragma unroll
-  for (int v = 0; v < 4; ++v) {
-    const float other = __shfl_xor(own[v], 32, kWave);              // the pair's other half
-    float val = own[v];
-    if (rotate) {
-      const float2 cs = table[static_cast<int64_t>(pos) * half + p + 4 * (g & 1) + v];
-      val = second ? own[v] * cs.x + other * cs.y : own[v] * cs.x - other * cs.y;
+    for (int i = 0; i < MT; ++i) red[wave][i][lane] = acc[rt][i];
+    __syncthreads();
+    const int t = static_cast<int>(blockIdx.x) * RT + rt;
+    if (wave >= MT || t >= n_tiles) continue;
+    const int head = t / tiles_per_head;
+    const int p = (t - head * tiles_per_head) << 3;
+    const int mt = wave;
+    f32x4 own = red[0][mt][lane];
+#pragma unroll
+    for (int w2 = 1; w2 < WV; ++w2) own += red[w2][mt][lane];
+    const int m = mt * 16 + r;
+    const int mc = min(m, M - 1);
+    const bool second = g >= 2;
+    const bool rotate = table != nullptr && head < hq + hkv;
+    const int pos = positions[mc];
+    f32x4 res;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const float other = __shfl_xor(own[v], 32, kWave);              // the pair's other half
+      float val = own[v];
+      if (rotate) {
+        const float2 cs = table[static_cast<int64_t>(pos) * half + p + 4 * (g & 1) + v];
+        val = second ? own[v] * cs.x + other * cs.y : own[v] * cs.x - other * cs.y;
+      }
+      res[v] = val;
     }
-    res[v] = val;
+    if (m >= M) continue;
+    const int e0 = (second ? half : 0) + p + 4 * (g & 1);              // element of the head, 4 consecutive
+    ushort4 pk;
+    pk.x = float_to_bf16(res[0]);
+    pk.y = float_to_bf16(res[1]);
+    pk.z = float_to_bf16(res[2]);
+    pk.w = float_to_bf16(res[3]);
+    *reinterpret_cast<ushort4*>(qkv_out + static_cast<int64_t>(m) * ((hq + 2 * hkv) * d) + head * d + e0) = pk;
+    if (kv == nullptr || head < hq) continue;
+    const int slot = write_slot[m];
+    const int64_t page_elems = 2LL * hkv * kPage * d;
+    bf16_t* page = kv + static_cast<int64_t>(slot / kPage) * page_elems;
+    const int off = slot % kPage;
+    if (head < hq + hkv) {                                             // key row [16][D]
+      *reinterpret_cast<ushort4*>(page + (static_cast<int64_t>(head - hq) * kPage + off) * d + e0) = pk;
+    } else {                                                           // value, transposed [D][16]
+      bf16_t* vp = page + static_cast<int64_t>(hkv) * kPage * d + (static_cast<int64_t>(head - hq - hkv) * d + e0) * kPage + off;
+      vp[0] = pk.x;
+      vp[kPage] = pk.y;
+      vp[2 * kPage] = pk.z;
+      vp[3 * kPage] = pk.w;
+    }
   }
-  if (m >= M) return;
-  const int e0 = (second ? half : 0) + p + 4 * (g & 1);              // element of the head, 4 consecutive
-  ushort4 pk;
-  pk.x = float_to_bf16(res[0]);
-  pk.y = float_to_bf16(res[1]);
-  pk.z = float_to_bf16(res[2]);
-  pk.w = float_to_bf16(res[3]);
-  *reinterpret_cast<ushort4*>(qkv_out + static_cast<int64_t>(m) * ((hq + 2 * hkv) * d) + head * d + e0) = pk;
-  if (kv == nullptr || head < hq) return;
-  const int slot = write_slot[m];
-  const int64_t page_elems = 2LL * hkv * kPage * d;
-  bf16_t* page = kv + static_cast<int64_t>(slot / kPage) * page_elems;
-  const int off = slot % kPage;
-  if (head < hq + hkv) {                                             // key row [16][D]
-    *reinterpret_cast<ushort4*>(page + (static_cast<int64_t>(head - hq) * kPage + off) * d + e0) = pk;
-  } else {                                                           // value, transposed [D][16]
-    bf16_t* vp = page + static_cast<int64_t>(hkv) * kPage * d + (static_cast<int64_t>(head - hq - hkv) * d + e0) * kPage + off;
-    vp[0] = pk.x;
-    vp[kPage] = pk.y;
-    vp[2 * kPage] = pk.z;
-    vp[3 * kPage] = pk.w;
+}
+
+// One tile per workgroup keeps the most workgroups, and K cannot be split over workgroups
+// here (the rotation needs whole sums); two tiles halve the traffic for the tokens once there
+// are many tokens and still enough workgroups for every compute unit.
+template <int MT>
+static void launch_qkv(hipStream_t s, const bf16_t* x, const bf16_t* w, bf16_t* out, int M, int K, int hq, int hkv, int d,
+                       const int32_t* positions, const float2* table, bf16_t* kv, const int32_t* write_slot) {
+  const int n_tiles = (hq + 2 * hkv) * (d / 16);
+  if (MT >= 3 && n_tiles >= 384) {
+    constexpr int RT = MT >= 3 ? 2 : 1;
+    qkv_rope_append_kernel<MT, RT, 4><<<dim3(static_cast<unsigned>(ceil_div(n_tiles, RT))), dim3(256), 0, s>>>(
+        x, w, out, M, K, hq, hkv, d, positions, table, kv, write_slot);
+  } else {
+    qkv_rope_append_kernel<MT, 1, 4><<<dim3(static_cast<unsigned>(n_tiles)), dim3(256), 0, s>>>(
+        x, w, out, M, K, hq, hkv, d, positions, table, kv, write_slot);
   }
 }
 
@@ -383,6 +450,18 @@ int psamd_linear(void* stream, const void* x, int x_dtype, const void* w, int w_
   if (x_dtype == kBF16 && w_dtype == kBF16 && out_dtype == kBF16) return launch_tiled<bf16_t, bf16_t, bf16_t>(s, x, w, out, M, N, K);
   if (x_dtype == kBF16 && w_dtype == kBF16 && out_dtype == kF32) return launch_tiled<bf16_t, bf16_t, float>(s, x, w, out, M, N, K);
   return fail("psamd_linear: supported types are (f32,f32)->f32, (bf16,bf16)->bf16 and (bf16,bf16)->f32");
+}
+
+// The K-split that fills the chip for a linear product of M <= 64 tokens whose float32 partial
+// sums a consumer adds up: as many workgroups as there are compute units to spare, each wave
+// keeping at least two k-steps.
+int psamd_linear_skinny_ksplit(int M, int n_out, int K) {
+  if (M < 1 || M > 64 || n_out < 1 || K < 1) return 1;
+  const int mt = static_cast<int>(ceil_div(M, 16));
+  const int64_t groups = ceil_div(ceil_div(n_out, 16), skinny_rt(mt, false));
+  const int64_t steps = ceil_div(K, 32);
+  const int64_t split = std::min<int64_t>({8, 512 / std::max<int64_t>(groups, 1), steps / (2 * skinny_wv(mt))});
+  return static_cast<int>(std::max<int64_t>(split, 1));
 }
 
 // out[ksplit][M, n_out]; epilogue 0: n_out = rows of w; epilogue 1 (SwiGLU): w has 2 * n_out rows.
@@ -419,17 +498,16 @@ int psamd_qkv_rope_append(void* stream, const void* x, const void* w, void* qkv_
   PSAMD_REQUIRE(positions != nullptr, "positions are needed");
   PSAMD_REQUIRE(kv == nullptr || write_slot != nullptr, "a cache needs write slots");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const dim3 grid(static_cast<unsigned>((hq + 2 * hkv) * (head_dim / 16))), block(256);
   const bf16_t* xp = static_cast<const bf16_t*>(x);
   const bf16_t* wp = static_cast<const bf16_t*>(w);
   bf16_t* op = static_cast<bf16_t*>(qkv_out);
   const float2* tab = reinterpret_cast<const float2*>(table);
   bf16_t* kvp = static_cast<bf16_t*>(kv);
   switch (static_cast<int>(ceil_div(M, 16))) {
-    case 1: qkv_rope_append_kernel<1><<<grid, block, 0, s>>>(xp, wp, op, M, K, hq, hkv, head_dim, positions, tab, kvp, write_slot); break;
-    case 2: qkv_rope_append_kernel<2><<<grid, block, 0, s>>>(xp, wp, op, M, K, hq, hkv, head_dim, positions, tab, kvp, write_slot); break;
-    case 3: qkv_rope_append_kernel<3><<<grid, block, 0, s>>>(xp, wp, op, M, K, hq, hkv, head_dim, positions, tab, kvp, write_slot); break;
-    default: qkv_rope_append_kernel<4><<<grid, block, 0, s>>>(xp, wp, op, M, K, hq, hkv, head_dim, positions, tab, kvp, write_slot); break;
+    case 1: launch_qkv<1>(s, xp, wp, op, M, K, hq, hkv, head_dim, positions, tab, kvp, write_slot); break;
+    case 2: launch_qkv<2>(s, xp, wp, op, M, K, hq, hkv, head_dim, positions, tab, kvp, write_slot); break;
+    case 3: launch_qkv<3>(s, xp, wp, op, M, K, hq, hkv, head_dim, positions, tab, kvp, write_slot); break;
+    default: launch_qkv<4>(s, xp, wp, op, M, K, hq, hkv, head_dim, positions, tab, kvp, write_slot); break;
   }
   return check_launch("psamd_qkv_rope_append");
 }

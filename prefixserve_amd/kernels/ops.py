@@ -44,6 +44,7 @@ _SIGNATURES = {
     "psamd_rope_kv_append": [_vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp, _vp, _vp, _vp],
     "psamd_linear": [_vp, _vp, _i32, _vp, _i32, _vp, _i32, _i64, _i32, _i32],
     "psamd_linear_skinny": [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32],
+    "psamd_linear_skinny_ksplit": [_i32, _i32, _i32],
     "psamd_qkv_rope_append": [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp],
     "psamd_attention_generic": [_vp, _vp, _i32, _vp, _vp, _i32, _i64, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _f32, _i32],
     "psamd_attention_mfma_supports": [_i32, _i32, _i32],
@@ -209,8 +210,7 @@ class HipOps:
         m, k = x.shape
         n = w.shape[0]
         if x.dtype == torch.bfloat16 and k % 8 == 0 and 0 < m <= self.SKINNY_MAX_ROWS:
-            groups, steps = -(-n // (16 if m <= 16 else 32)), -(-k // 32)   # workgroups before splitting K
-            ksplit = max(1, min(8, 512 // groups, steps // 8))
+            ksplit = self.lib.psamd_linear_skinny_ksplit(m, n, k)
             if ksplit > 1:
                 self._need(w.shape[1] == k and x.is_contiguous() and w.is_contiguous(), "linear_to_residual: operands")
                 out = self.ws.get(name, (ksplit, m, n), torch.float32)
