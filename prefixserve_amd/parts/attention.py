@@ -8,8 +8,7 @@ from typing import TYPE_CHECKING, Any, Mapping
 
 import torch
 
-from .base import CacheNeed, Mixer, PositionEncoding, Runtime, WeightWant, register_mixer
-from .rope import RotaryEmbedding
+from .base import CacheNeed, Mixer, PositionEncoding, RotaryTable, Runtime, WeightWant, register_mixer
 
 if TYPE_CHECKING:
     from prefixserve_amd.engine.batch import StepContext
@@ -49,9 +48,9 @@ class PagedAttention(Mixer):
         self.window = None if window is None else int(window)
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
         self.pos = positions[position] if position is not None else None
-        if self.pos is not None and not isinstance(self.pos, RotaryEmbedding):
-            raise ValueError("PagedAttention applies rotary encodings; other encodings belong to their own mixer")
-        if isinstance(self.pos, RotaryEmbedding) and self.pos.head_dim != self.head_dim:
+        if self.pos is not None and not isinstance(self.pos, RotaryTable):
+            raise ValueError("PagedAttention applies rotation tables; other encodings belong to their own mixer")
+        if isinstance(self.pos, RotaryTable) and self.pos.head_dim != self.head_dim:
             raise ValueError("rotary head_dim differs from the attention head_dim")
         self.q_size = self.num_heads * self.head_dim
         self.kv_size = self.num_kv_heads * self.head_dim

@@ -133,6 +133,16 @@ class PositionEncoding(Part):
         """Build tables for positions [0, max_position)."""
 
 
+class RotaryTable(PositionEncoding):
+    """A position encoding that rotates the pairs (i, i + D/2) of every query and key head by
+    an angle that depends on the position and on i. It has ``head_dim`` and, once ``prepare``
+    ran, ``table``: float32 ``[max_position, head_dim / 2, 2]`` = (cos, sin) on the device.
+    How the angles come about is the subclass's business; attention only reads the table."""
+
+    head_dim: int
+    table: torch.Tensor | None = None
+
+
 class Mixer(Part):
     """Mixes information between positions (attention here)."""
 

@@ -7,7 +7,7 @@ from typing import Any, Mapping
 
 import torch
 
-from .base import PositionEncoding, Runtime, register_position
+from .base import RotaryTable, Runtime, register_position
 
 
 def rope_inv_freq(head_dim: int, theta: float, scaling: Mapping[str, Any] | None) -> torch.Tensor:
@@ -33,7 +33,7 @@ def rope_inv_freq(head_dim: int, theta: float, scaling: Mapping[str, Any] | None
     return inv.to(torch.float32)
 
 
-class RotaryEmbedding(PositionEncoding):
+class RotaryEmbedding(RotaryTable):
     """Pairs (i, i + D/2) of every head are rotated by angle = position * inv_freq[i]
     (prefixserve/model/llama.py:72-77). The angle is a float32 product as in the
     reference's table (llama.py:56-58); its cosine and sine are kept in float32 whatever

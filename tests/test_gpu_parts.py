@@ -346,3 +346,150 @@ def test_windowed_attention_through_the_engine(tmp_path):
                 assert err.max() < tol, f"{dtype} positions {p0}..{p0 + c}: {err.max():.3e}"
                 p0 += c
             assert all(rp.cache.num_free(g) == rp.cache.num_blocks(g) for g in range(2))
+
+
+def test_a_toy_position_encoding_and_a_routed_feed_forward(tmp_path):
+    """Two more parts defined and registered from this test only: a position encoding whose
+    rotation angle is position * (i + 1) / 50 (another rule than rope's, through the same
+    rotation table), and a feed-forward that sends every token to one of three SwiGLU experts
+    by the largest router logit and scales the result by that logit's softmax weight. Layer 0
+    uses both; layer 1 is an ordinary rope + dense layer: the parts are chosen per layer.
+    Compared with the plain functions, whole and in portions, in both dtypes."""
+    import json
+
+    from safetensors.torch import save_file
+
+    from prefixserve_amd.config import register_architecture, registered_architectures
+    from prefixserve_amd.engine.replay import TraceReplayer
+    from prefixserve_amd.engine.runner import ModelRunner
+    from prefixserve_amd.parts import (DecoderModel, FeedForward, LayerRun, LayerSpec, ModelSpec, PartSpec, RotaryTable,
+                                       WeightWant, register_feed_forward, register_position)
+    from prefixserve_amd.weights import random_tensors
+
+    H, HQ, HKV, D, INNER, V, E = 80, 5, 1, 32, 48, 90, 3
+
+    class LinearAngles(RotaryTable):
+        def __init__(self, head_dim, slope):
+            self.head_dim, self.slope = int(head_dim), float(slope)
+
+        def prepare(self, max_position):
+            i = torch.arange(self.head_dim // 2, dtype=torch.float64)
+            angle = torch.outer(torch.arange(max_position, dtype=torch.float64), (i + 1.0) * self.slope)
+            self.table = torch.stack((angle.cos(), angle.sin()), -1).float().contiguous().to(self.rt.device)
+
+    class Top1Experts(FeedForward):
+        def __init__(self, hidden_size, inner, experts):
+            self.h, self.inner, self.e = hidden_size, inner, experts
+
+        def weights(self):
+            want = {"router.weight": WeightWant((self.e, self.h))}
+            for e in range(self.e):
+                want[f"e{e}.gate_up.weight"] = WeightWant((2 * self.inner, self.h))
+                want[f"e{e}.down.weight"] = WeightWant((self.h, self.inner))
+            return want
+
+        def bind(self, tensors, rt):
+            super().bind(tensors, rt)
+            self.router = tensors["router.weight"].float().to(rt.device)        # router logits in 32-bit
+            self.gate_up = [rt.ops.prepare_matrix(tensors[f"e{e}.gate_up.weight"], rt) for e in range(self.e)]
+            self.down = [rt.ops.prepare_matrix(tensors[f"e{e}.down.weight"], rt) for e in range(self.e)]
+
+        def forward(self, x, ctx):
+            ops = self.rt.ops
+            logits = x.float() @ self.router.T
+            weight, choice = torch.softmax(logits, -1).max(-1)
+            out = torch.zeros_like(x)
+            for e in range(self.e):
+                rows = (choice == e).nonzero().flatten()
+                if rows.numel() == 0:
+                    continue
+                xe = x[rows].contiguous()
+                act = torch.empty(rows.numel(), self.inner, dtype=x.dtype, device=x.device)
+                ops.linear_swiglu(xe, self.gate_up[e], act)
+                ye = torch.empty(rows.numel(), self.h, dtype=x.dtype, device=x.device)
+                ops.linear(act, self.down[e], ye)
+                out[rows] = (ye.float() * weight[rows, None]).to(x.dtype)
+            return out
+
+    class Cfg:
+        def __init__(self, raw):
+            self.raw = raw
+
+        @classmethod
+        def from_dicts(cls, raw, gen=None):
+            return cls(dict(raw))
+
+    def build(cfg):
+        def attn(position):
+            return PartSpec("paged_attention", {"num_heads": HQ, "num_kv_heads": HKV, "head_dim": D, "position": position,
+                                                "names": {"q": "q.weight", "k": "k.weight", "v": "v.weight", "o": "o.weight"}})
+        dense = PartSpec("swiglu", {"intermediate_size": INNER, "names": {"gate": "g.weight", "up": "u.weight", "down": "d.weight"}})
+        routed = PartSpec("test_top1_experts", {"inner": INNER, "experts": E})
+        norm = lambda nm: PartSpec("rmsnorm", {"eps": 1e-6, "name": nm})
+        layers = (LayerSpec(prefix="l0.", mixer=attn("linear"), feed_forward=routed, mixer_norm=norm("n1.weight"),
+                            feed_forward_norm=norm("n2.weight")),
+                  LayerSpec(prefix="l1.", mixer=attn("rope"), feed_forward=dense, mixer_norm=norm("n1.weight"),
+                            feed_forward_norm=norm("n2.weight")))
+        return ModelSpec(vocab_size=V, hidden_size=H, embedding="emb.weight", layers=layers,
+                         order=(LayerRun(0, 0), LayerRun(1, 1)), final_norm=norm("norm.weight"), final_norm_prefix="",
+                         head="head.weight",
+                         positions={"rope": PartSpec("rope", {"head_dim": D, "theta": 10000.0}),
+                                    "linear": PartSpec("test_linear_angles", {"head_dim": D, "slope": 0.02})},
+                         max_position=256)
+
+    if "ToyRoutedForCausalLM" not in registered_architectures():
+        register_position("test_linear_angles", LinearAngles)
+        register_feed_forward("test_top1_experts", Top1Experts)
+        register_architecture("ToyRoutedForCausalLM", Cfg, build)
+    raw = {"architectures": ["ToyRoutedForCausalLM"]}
+    (tmp_path / "config.json").write_text(json.dumps(raw))
+    tensors = random_tensors(DecoderModel(build(Cfg(raw))).weights(), seed=11, std=0.1)
+    tensors["l0.router.weight"] = tensors["l0.router.weight"] * 8.0        # clear choices, far from ties
+    save_file(tensors, str(tmp_path / "model.safetensors"))
+    w = {k: v.double().numpy() for k, v in tensors.items()}
+
+    toks = np.random.default_rng(5).integers(0, V, 100).tolist()
+    n = len(toks)
+    pos = np.arange(n)
+    angle = np.outer(pos, (np.arange(D // 2) + 1.0) * 0.02)
+    angle = np.concatenate([angle, angle], -1)                            # both halves of a pair share the angle
+    tables = [(np.cos(angle), np.sin(angle)), P.rope_cos_sin(pos, P.rope_inv_freq(D, 10000.0, None))]
+    h = w["emb.weight"][toks]
+    used = set()
+    for i, (cos, sin) in enumerate(tables):
+        p = f"l{i}."
+        x = P.rms_norm(h, w[p + "n1.weight"], 1e-6)
+        q = P.apply_rope((x @ w[p + "q.weight"].T).reshape(n, HQ, D), cos, sin)
+        k = P.apply_rope((x @ w[p + "k.weight"].T).reshape(n, HKV, D), cos, sin)
+        v = (x @ w[p + "v.weight"].T).reshape(n, HKV, D)
+        h = h + P.causal_attention(q, k, v).reshape(n, HQ * D) @ w[p + "o.weight"].T
+        x = P.rms_norm(h, w[p + "n2.weight"], 1e-6)
+        if i == 0:
+            logits = x @ w[p + "router.weight"].T
+            prob = np.exp(logits - logits.max(-1, keepdims=True))
+            prob /= prob.sum(-1, keepdims=True)
+            y = np.zeros_like(x)
+            for t in range(n):
+                e = int(prob[t].argmax())
+                used.add(e)
+                gu = w[p + f"e{e}.gate_up.weight"]
+                y[t] = prob[t, e] * P.swiglu_mlp(x[t:t + 1], gu[:INNER], gu[INNER:], w[p + f"e{e}.down.weight"])[0]
+            h = h + y
+        else:
+            h = h + P.swiglu_mlp(x, w[p + "g.weight"], w[p + "u.weight"], w[p + "d.weight"])
+    assert used == set(range(E))                                           # every expert had tokens
+    want = P.rms_norm(h, w["norm.weight"], 1e-6) @ w["head.weight"].T
+
+    for dtype, tol in (("float32", 1e-5), ("bfloat16", 4e-2)):
+        runner = ModelRunner(tmp_path, dtype=dtype, device="cuda:0", num_blocks=8, max_seq_len=112, max_num_seqs=2,
+                             use_graphs=False)
+        for cuts in ([n], [3, 2, 40, 1, 1, 1, 17, 35]):
+            assert sum(cuts) == n
+            rp = TraceReplayer(runner)
+            p0 = 0
+            for kk, c in enumerate(cuts):
+                got = rp.run_step({"step": kk, "entries": [{"id": "a", "tokens": toks[p0:p0 + c], "want": list(range(c))}],
+                                   "end": ["a"] if p0 + c == n else []})
+                err = np.abs(got - want[p0:p0 + c]).max(-1) / np.abs(want[p0:p0 + c]).max(-1)
+                assert err.max() < tol, f"{dtype} positions {p0}..{p0 + c}: {err.max():.3e}"
+                p0 += c
