@@ -108,3 +108,37 @@ def test_pool_is_sized_from_free_memory(model_dirs):
 
     eng = Engine(EngineConfig(model_path=model_dirs["A"], dtype="bfloat16", max_seq_len=512, reserve_bytes=200 << 30))
     assert eng.num_blocks > 10_000
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_hundred_requests_decode_together(dtype, model_dirs, plain_models):
+    """More decoding requests in one step than the small-step kernels take (64): the step falls
+    back to the general product and the decode attention runs over 100 block tables."""
+    from prefixserve_amd import Engine, EngineConfig, generate
+
+    name = "B"
+    rng = np.random.default_rng(12)
+    prompts = [rng.integers(3, 512, int(n)).tolist() for n in rng.integers(1, 40, 100)]
+    eng = Engine(EngineConfig(model_path=model_dirs[name], dtype=dtype, max_num_seqs=100, max_prefill_tokens=256,
+                              max_seq_len=64, num_blocks=100 * 4))
+    widest, step = [0], eng.step
+
+    def counting_step(batch):
+        widest[0] = max(widest[0], sum(1 for w in batch.work if w.end - w.start == 1))
+        return step(batch)
+
+    eng.step = counting_step
+    outs, stats = generate(eng, prompts, 10, ignore_eos=True)
+    assert stats.preemptions == 0 and widest[0] == 100
+    for p, o in list(zip(prompts, outs))[::7]:
+        if dtype == "float32":
+            assert o.tokens == plain_models[name].greedy(p, 10)[0]
+            continue
+        seq = list(p)
+        for tok in o.tokens:                                  # teacher-forced: equal, or a near-tie
+            row = plain_models[name].logits(seq)[-1]
+            best = int(np.argmax(row))
+            if tok != best:
+                assert row[best] - row[tok] < 0.05 * np.abs(row).max(), "left the plain model at a clear margin"
+                break
+            seq.append(tok)

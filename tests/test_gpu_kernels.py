@@ -311,6 +311,16 @@ def test_paged_attention_window(ops, act, window):
 
 
 @pytest.mark.parametrize("act", [torch.float32, torch.bfloat16])
+def test_paged_attention_long_contexts(ops, act):
+    """Tens of thousands of cached positions: the decode kernel at its widest split, a portion
+    on top of a long prefix, and short requests beside them in the same batch."""
+    got, want = paged_case(ops, act, 8, 2, 64, [1, 300, 1, 1, 5], [20000, 9000, 3, 33000, 0], seed=5, num_blocks=4096)
+    assert rel(got, want) < (2e-5 if act == torch.float32 else 2e-2)
+    got, want = paged_case(ops, act, 4, 4, 128, [1, 40], [16383, 16384], seed=6, num_blocks=2100)
+    assert rel(got, want) < (2e-5 if act == torch.float32 else 2e-2)
+
+
+@pytest.mark.parametrize("act", [torch.float32, torch.bfloat16])
 def test_attention_finds_one_far_key_among_hundreds(ops, act):
     """One old key is made to match the query strongly; the output must be that key's value,
     wherever its page lies. A kernel that skips or misplaces a page cannot pass."""
