@@ -263,6 +263,198 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
   }
 }
 
+// ------------------------------------------------------------------ prefill, query heads of a kv head together
+
+// The same 32 queries for up to 4 query heads that share a kv head: one head per wave, all
+// keys, no merge. The 32-key tile of K and of V^T is brought into LDS ONCE per workgroup
+// (16-byte loads, whole contiguous pages) and read from there by the 4 waves: the texture
+// path, which bounded the kernel above (a wave's operand loads there touch 32 rows of 32
+// bytes each, and every head loads the same keys again), carries a quarter of the bytes in
+// full lines. Two LDS stages: the next tile's global loads are in flight while the current
+// tile is multiplied, one barrier per tile.
+// LDS rows are padded (keys by 8 elements, V^T rows by 4) so that a wave's operand reads
+// spread over all banks.
+template <int NS>
+__global__ __launch_bounds__(256) void attn_prefill_grouped_kernel(
+    const bf16_t* __restrict__ qkv, int q_stride, bf16_t* __restrict__ out, const bf16_t* __restrict__ kv,
+    const int32_t* __restrict__ pf_tiles, const int32_t* __restrict__ item_start,
+    const int32_t* __restrict__ item_pos0, const int32_t* __restrict__ table_off,
+    const int32_t* __restrict__ block_ids, int hq, int hkv, int table_pages, float scale, int window) {
+  constexpr int D = 16 * NS;
+  constexpr int DT = (D + 31) / 32;
+  constexpr int KS = D + 8;                      // elements per key row in LDS
+  constexpr int VS = kPage + 4;                  // elements per V^T row of one page in LDS
+  constexpr int CHUNKS = 4 * D;                  // 16-byte pieces of a K tile (and of a V tile)
+  constexpr int CPT = (CHUNKS + 255) / 256;      // pieces per thread
+  constexpr int K_STAGE = 32 * KS, V_STAGE = 2 * D * VS;
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  bf16_t* k_lds = reinterpret_cast<bf16_t*>(smem_raw);
+  bf16_t* v_lds = k_lds + 2 * K_STAGE;
+  int32_t* table = reinterpret_cast<int32_t*>(v_lds + 2 * V_STAGE);
+
+  const int group = hq / hkv;
+  const int wg_per_kv = (group + 3) >> 2;
+  // Late tiles of a prompt see the most keys: start them first.
+  const int tile = gridDim.x - 1 - blockIdx.x;
+  const int kvh = blockIdx.y / wg_per_kv;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int head_in_group = (blockIdx.y - kvh * wg_per_kv) * 4 + wave;
+  const bool head_valid = head_in_group < group;       // a spare wave repeats the last head and writes nothing
+  const int h = kvh * group + min(head_in_group, group - 1);
+  const int item = pf_tiles[2 * tile];
+  const int q_off = pf_tiles[2 * tile + 1];
+  const int t0 = item_start[item];
+  const int n = item_start[item + 1] - t0;
+  const int pos0 = item_pos0[item];
+  const int col = lane & 31, hi = lane >> 5;
+
+  const int qi = min(q_off + col, n - 1);          // lanes past the end repeat the last query
+  const bool q_valid = q_off + col < n;
+  const int q_pos = pos0 + qi;
+  const int first_pos = pos0 + q_off;
+  const int last_pos = pos0 + min(q_off + 31, n - 1);
+  const int k_lo_q = window > 0 ? max(0, q_pos - window + 1) : 0;
+  const int k_begin = window > 0 ? (max(0, first_pos - window + 1) & ~31) : 0;
+  const float c = scale * 1.44269504088896340736f;  // scores are exponentiated in base 2
+  {
+    const int32_t* gtable = block_ids + table_off[item];
+    for (int i = threadIdx.x; i <= (last_pos >> 4); i += blockDim.x) table[i] = gtable[i];
+  }
+  __syncthreads();
+
+  bf16x8 qf[NS];
+  {
+    const bf16_t* qp = qkv + static_cast<int64_t>(t0 + qi) * q_stride + h * D + 8 * hi;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) qf[s] = ld8(qp + 16 * s);
+  }
+  f32x16 o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) o[dt][v] = 0.f;
+  float m = -INFINITY, l = 0.f;       // m in base-2 units (score * c)
+
+  const int64_t page_elems = 2LL * hkv * kPage * D;
+  const int64_t khead = static_cast<int64_t>(kvh) * kPage * D;
+  const int64_t vhead = static_cast<int64_t>(hkv) * kPage * D + static_cast<int64_t>(kvh) * D * kPage;
+
+  // Piece p of a tile lies in page p / (2 D) at element 8 * (p % (2 D)) of the head's keys
+  // (and likewise of its values): both halves of a page are contiguous per head.
+  uint4 kreg[CPT], vreg[CPT];
+  auto load_global = [&](int k0) {
+    const int64_t base0 = static_cast<int64_t>(table[k0 >> 4]) * page_elems;
+    const int64_t base1 = static_cast<int64_t>(table[min(k0 + 16, last_pos) >> 4]) * page_elems;
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) {
+      const int p = threadIdx.x + 256 * i;
+      if (CHUNKS % 256 == 0 || p < CHUNKS) {
+        const int page = p >= 2 * D, rem = p - page * 2 * D;
+        const bf16_t* src = kv + (page ? base1 : base0) + 8 * rem;
+        kreg[i] = *reinterpret_cast<const uint4*>(src + khead);
+        vreg[i] = *reinterpret_cast<const uint4*>(src + vhead);
+      }
+    }
+  };
+  auto store_lds = [&](int stage) {
+    bf16_t* kd = k_lds + stage * K_STAGE;
+    bf16_t* vd = v_lds + stage * V_STAGE;
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) {
+      const int p = threadIdx.x + 256 * i;
+      if (CHUNKS % 256 == 0 || p < CHUNKS) {
+        const int key = p / (D / 8), part = p - key * (D / 8);
+        *reinterpret_cast<uint4*>(kd + key * KS + 8 * part) = kreg[i];
+        const int row = p >> 1, half = p & 1;                     // row = page * D + d
+        uint2* dst = reinterpret_cast<uint2*>(vd + row * VS + 8 * half);
+        dst[0] = uint2{vreg[i].x, vreg[i].y};
+        dst[1] = uint2{vreg[i].z, vreg[i].w};
+      }
+    }
+  };
+  auto compute = [&](int stage, int k0) {
+    const bf16_t* kd = k_lds + stage * K_STAGE + col * KS + 8 * hi;
+    const bf16_t* vd = v_lds + stage * V_STAGE + 4 * hi;
+    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    f32x16 s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ld8(kd), qf[0], zero, 0, 0, 0);
+#pragma unroll
+    for (int i = 1; i < NS; ++i) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ld8(kd + 16 * i), qf[i], s, 0, 0, 0);
+    // A tile whose last key is not after the first query, with no window, needs no mask.
+    if (window > 0 || k0 + 31 > first_pos) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int key = k0 + 8 * (v >> 2) + 4 * hi + (v & 3);
+        s[v] = (key <= q_pos && key >= k_lo_q) ? s[v] : -INFINITY;
+      }
+    }
+    float mx = s[0];
+#pragma unroll
+    for (int v = 1; v < 16; ++v) mx = fmaxf(mx, s[v]);
+    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave)) * c;
+    // The running maximum is only raised (and the accumulators rescaled) when some query's
+    // scores outgrow it by more than 2^8 (see the kernel above).
+    if (__any(mx > m + 8.f)) {
+      const float m_new = fmaxf(m, mx);
+      const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m - m_new);
+      l *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o[dt][v] *= alpha;
+      m = m_new;
+    }
+    const float m_use = m == -INFINITY ? 0.f : m;
+    float rowsum = 0.f;
+    bf16x8 pb[2];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const float p = __builtin_amdgcn_exp2f(fmaf(s[v], c, -m_use));
+      rowsum += p;
+      pb[v >> 3][v & 7] = static_cast<__bf16>(p);
+    }
+    l += rowsum + __shfl_xor(rowsum, 32, kWave);
+#pragma unroll
+    for (int cpage = 0; cpage < 2; ++cpage)
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        const bf16_t* vr = vd + (cpage * D + min(32 * dt + col, D - 1)) * VS;
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(join(ld4(vr), ld4(vr + 8)), pb[cpage], o[dt], 0, 0, 0);
+      }
+  };
+
+  {
+    int stage = 0;
+    load_global(k_begin);
+    for (int k0 = k_begin; k0 <= last_pos; k0 += 32) {
+      store_lds(stage);
+      if (k0 + 32 <= last_pos) load_global(k0 + 32);
+      // Every wave is past the tile that last used this stage: it had to finish it to reach
+      // the previous barrier.
+      __syncthreads();
+      compute(stage, k0);
+      stage ^= 1;
+    }
+  }
+
+  if (!head_valid || !q_valid) return;
+  const float inv = 1.f / l;
+  bf16_t* op = out + static_cast<int64_t>(t0 + qi) * (static_cast<int64_t>(hq) * D) + h * D;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int v4 = 0; v4 < 4; ++v4) {
+      const int d = 32 * dt + 8 * v4 + 4 * hi;
+      if (d < D) {
+        ushort4 pk;
+        pk.x = float_to_bf16(o[dt][4 * v4 + 0] * inv);
+        pk.y = float_to_bf16(o[dt][4 * v4 + 1] * inv);
+        pk.z = float_to_bf16(o[dt][4 * v4 + 2] * inv);
+        pk.w = float_to_bf16(o[dt][4 * v4 + 3] * inv);
+        *reinterpret_cast<ushort4*>(op + d) = pk;
+      }
+    }
+}
+
 // ------------------------------------------------------------------ decode (split keys)
 
 // NS = D / 16, CT = ceil(group / 16) column tiles of query heads.
@@ -454,10 +646,25 @@ __global__ __launch_bounds__(64) void attn_decode_merge_kernel(
   }
 }
 
+// Bytes of LDS the grouped kernel needs for head size D and a block table of table_pages entries.
+static size_t grouped_smem(int D, int table_pages) {
+  return sizeof(bf16_t) * 2 * (32 * static_cast<size_t>(D + 8) + 2 * static_cast<size_t>(D) * (kPage + 4)) +
+         sizeof(int32_t) * static_cast<size_t>(table_pages);
+}
+
 template <int NS>
 static int launch_prefill(hipStream_t s, const void* qkv, int q_stride, void* out, const void* kv,
                           const int32_t* pf_tiles, int n_tiles, int table_pages, const int32_t* item_start, const int32_t* item_pos0,
                           const int32_t* table_off, const int32_t* block_ids, int hq, int hkv, float scale, int window) {
+  const int group = hq / hkv;
+  const size_t smem = grouped_smem(16 * NS, table_pages);
+  // Three or more query heads per kv head: they share the keys and values through LDS.
+  if (group >= 3 && smem <= 64 * 1024) {
+    attn_prefill_grouped_kernel<NS><<<dim3(n_tiles, hkv * ((group + 3) / 4)), dim3(256), smem, s>>>(
+        static_cast<const bf16_t*>(qkv), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(kv), pf_tiles,
+        item_start, item_pos0, table_off, block_ids, hq, hkv, table_pages, scale, window);
+    return check_launch("psamd_attention_prefill");
+  }
   attn_prefill_mfma_kernel<NS><<<dim3(n_tiles, hq), dim3(256), sizeof(int32_t) * static_cast<size_t>(table_pages), s>>>(
       static_cast<const bf16_t*>(qkv), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(kv), pf_tiles,
       item_start, item_pos0, table_off, block_ids, hq, hkv, scale, window);
