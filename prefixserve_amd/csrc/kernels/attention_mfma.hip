@@ -18,6 +18,8 @@
 // Softmax statistics, scaling and masks are float. Page layout per layer:
 // [num_blocks][2][kv_heads][16 * D], half 0 keys [16][D], half 1 values [D][16].
 
+#include <algorithm>
+
 #include "api.h"
 #include "common.h"
 
@@ -274,19 +276,21 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
 // tile is multiplied, one barrier per tile.
 // LDS rows are padded (keys by 8 elements, V^T rows by 4) so that a wave's operand reads
 // spread over all banks.
-template <int NS>
-__global__ __launch_bounds__(256) void attn_prefill_grouped_kernel(
+template <int NS, int KT, int KP>
+__global__ __launch_bounds__(256 * KP) void attn_prefill_grouped_kernel(
     const bf16_t* __restrict__ qkv, int q_stride, bf16_t* __restrict__ out, const bf16_t* __restrict__ kv,
     const int32_t* __restrict__ pf_tiles, const int32_t* __restrict__ item_start,
     const int32_t* __restrict__ item_pos0, const int32_t* __restrict__ table_off,
-    const int32_t* __restrict__ block_ids, int hq, int hkv, int table_pages, float scale, int window) {
+    const int32_t* __restrict__ block_ids, int n_tiles, int hq, int hkv, int table_pages, float scale, int window) {
   constexpr int D = 16 * NS;
   constexpr int DT = (D + 31) / 32;
   constexpr int KS = D + 8;                      // elements per key row in LDS
   constexpr int VS = kPage + 4;                  // elements per V^T row of one page in LDS
-  constexpr int CHUNKS = 4 * D;                  // 16-byte pieces of a K tile (and of a V tile)
-  constexpr int CPT = (CHUNKS + 255) / 256;      // pieces per thread
-  constexpr int K_STAGE = 32 * KS, V_STAGE = 2 * D * VS;
+  constexpr int THREADS = 256 * KP;
+  constexpr int KEYS = 32 * KT * KP;             // keys per iteration
+  constexpr int CHUNKS = 4 * D * KT * KP;        // 16-byte pieces of an iteration's keys (and of its values)
+  constexpr int CPT = (CHUNKS + THREADS - 1) / THREADS;   // pieces per thread
+  constexpr int K_STAGE = KEYS * KS, V_STAGE = (KEYS / kPage) * D * VS;
   extern __shared__ __align__(16) unsigned char smem_raw[];
   bf16_t* k_lds = reinterpret_cast<bf16_t*>(smem_raw);
   bf16_t* v_lds = k_lds + 2 * K_STAGE;
@@ -294,13 +298,21 @@ __global__ __launch_bounds__(256) void attn_prefill_grouped_kernel(
 
   const int group = hq / hkv;
   const int wg_per_kv = (group + 3) >> 2;
-  // Late tiles of a prompt see the most keys: start them first.
-  const int tile = gridDim.x - 1 - blockIdx.x;
   const int kvh = blockIdx.y / wg_per_kv;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int head_in_group = (blockIdx.y - kvh * wg_per_kv) * 4 + wave;
+  const int part = wave >> 2;                           // which of the iteration's KP runs of keys
+  const int head_in_group = (blockIdx.y - kvh * wg_per_kv) * 4 + (wave & 3);
   const bool head_valid = head_in_group < group;       // a spare wave repeats the last head and writes nothing
   const int h = kvh * group + min(head_in_group, group - 1);
+  // A workgroup takes two tiles, one after the other: the b-th from the end and the b-th from
+  // the start. In a causal prompt the first sees the most keys and the second the fewest, so
+  // all workgroups get the same amount of work and none is left running alone at the end.
+  for (int phase = 0; phase < 2; ++phase) {
+  const int tile = phase == 0 ? n_tiles - 1 - static_cast<int>(blockIdx.x) : static_cast<int>(blockIdx.x);
+  if (phase == 1) {
+    if (tile >= n_tiles - 1 - static_cast<int>(blockIdx.x)) break;     // the middle tile is taken once
+    __syncthreads();                                                   // LDS is used again from the start
+  }
   const int item = pf_tiles[2 * tile];
   const int q_off = pf_tiles[2 * tile + 1];
   const int t0 = item_start[item];
@@ -314,7 +326,7 @@ __global__ __launch_bounds__(256) void attn_prefill_grouped_kernel(
   const int first_pos = pos0 + q_off;
   const int last_pos = pos0 + min(q_off + 31, n - 1);
   const int k_lo_q = window > 0 ? max(0, q_pos - window + 1) : 0;
-  const int k_begin = window > 0 ? (max(0, first_pos - window + 1) & ~31) : 0;
+  const int k_begin = window > 0 ? (max(0, first_pos - window + 1) & ~(KEYS - 1)) : 0;
   const float c = scale * 1.44269504088896340736f;  // scores are exponentiated in base 2
   {
     const int32_t* gtable = block_ids + table_off[item];
@@ -341,55 +353,69 @@ __global__ __launch_bounds__(256) void attn_prefill_grouped_kernel(
 
   // Piece p of a tile lies in page p / (2 D) at element 8 * (p % (2 D)) of the head's keys
   // (and likewise of its values): both halves of a page are contiguous per head.
-  uint4 kreg[CPT], vreg[CPT];
-  auto load_global = [&](int k0) {
-    const int64_t base0 = static_cast<int64_t>(table[k0 >> 4]) * page_elems;
-    const int64_t base1 = static_cast<int64_t>(table[min(k0 + 16, last_pos) >> 4]) * page_elems;
+  struct Pieces {
+    uint4 k[CPT], v[CPT];
+  };
+  auto load_global = [&](Pieces& r, int k0) {
 #pragma unroll
     for (int i = 0; i < CPT; ++i) {
-      const int p = threadIdx.x + 256 * i;
-      if (CHUNKS % 256 == 0 || p < CHUNKS) {
-        const int page = p >= 2 * D, rem = p - page * 2 * D;
-        const bf16_t* src = kv + (page ? base1 : base0) + 8 * rem;
-        kreg[i] = *reinterpret_cast<const uint4*>(src + khead);
-        vreg[i] = *reinterpret_cast<const uint4*>(src + vhead);
+      const int p = threadIdx.x + THREADS * i;
+      if (CHUNKS % THREADS == 0 || p < CHUNKS) {
+        const int page = p / (2 * D), rem = p - page * 2 * D;
+        const int64_t base = static_cast<int64_t>(table[min(k0 + 16 * page, last_pos) >> 4]) * page_elems;
+        const bf16_t* src = kv + base + 8 * rem;
+        r.k[i] = *reinterpret_cast<const uint4*>(src + khead);
+        r.v[i] = *reinterpret_cast<const uint4*>(src + vhead);
       }
     }
   };
-  auto store_lds = [&](int stage) {
+  auto store_lds = [&](const Pieces& r, int stage) {
     bf16_t* kd = k_lds + stage * K_STAGE;
     bf16_t* vd = v_lds + stage * V_STAGE;
 #pragma unroll
     for (int i = 0; i < CPT; ++i) {
-      const int p = threadIdx.x + 256 * i;
-      if (CHUNKS % 256 == 0 || p < CHUNKS) {
+      const int p = threadIdx.x + THREADS * i;
+      if (CHUNKS % THREADS == 0 || p < CHUNKS) {
         const int key = p / (D / 8), part = p - key * (D / 8);
-        *reinterpret_cast<uint4*>(kd + key * KS + 8 * part) = kreg[i];
+        *reinterpret_cast<uint4*>(kd + key * KS + 8 * part) = r.k[i];
         const int row = p >> 1, half = p & 1;                     // row = page * D + d
         uint2* dst = reinterpret_cast<uint2*>(vd + row * VS + 8 * half);
-        dst[0] = uint2{vreg[i].x, vreg[i].y};
-        dst[1] = uint2{vreg[i].z, vreg[i].w};
+        dst[0] = uint2{r.v[i].x, r.v[i].y};
+        dst[1] = uint2{r.v[i].z, r.v[i].w};
       }
     }
   };
-  auto compute = [&](int stage, int k0) {
-    const bf16_t* kd = k_lds + stage * K_STAGE + col * KS + 8 * hi;
-    const bf16_t* vd = v_lds + stage * V_STAGE + 4 * hi;
+  auto compute = [&](int stage, int k_iter) {
+    const int k0 = k_iter + 32 * KT * part;          // this wave's keys of the iteration
+    if (k0 > last_pos) return;                       // all after the last query (the loads were clamped)
+    const bf16_t* kd = k_lds + stage * K_STAGE + (32 * KT * part + col) * KS + 8 * hi;
+    const bf16_t* vd = v_lds + stage * V_STAGE + 2 * KT * part * D * VS + 4 * hi;
     const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    f32x16 s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ld8(kd), qf[0], zero, 0, 0, 0);
+    // The KT score tiles are independent chains of matrix instructions: one runs while the
+    // other's results are being exponentiated.
+    f32x16 s[KT];
 #pragma unroll
-    for (int i = 1; i < NS; ++i) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ld8(kd + 16 * i), qf[i], s, 0, 0, 0);
-    // A tile whose last key is not after the first query, with no window, needs no mask.
-    if (window > 0 || k0 + 31 > first_pos) {
+    for (int t = 0; t < KT; ++t) {
+      s[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ld8(kd + t * 32 * KS), qf[0], zero, 0, 0, 0);
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int key = k0 + 8 * (v >> 2) + 4 * hi + (v & 3);
-        s[v] = (key <= q_pos && key >= k_lo_q) ? s[v] : -INFINITY;
-      }
+      for (int i = 1; i < NS; ++i)
+        s[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ld8(kd + t * 32 * KS + 16 * i), qf[i], s[t], 0, 0, 0);
     }
-    float mx = s[0];
+    // Keys that are not after the first query, with no window, need no mask.
+    if (window > 0 || k0 + 32 * KT - 1 > first_pos) {
 #pragma unroll
-    for (int v = 1; v < 16; ++v) mx = fmaxf(mx, s[v]);
+      for (int t = 0; t < KT; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int key = k0 + 32 * t + 8 * (v >> 2) + 4 * hi + (v & 3);
+          s[t][v] = (key <= q_pos && key >= k_lo_q) ? s[t][v] : -INFINITY;
+        }
+    }
+    float mx = s[0][0];
+#pragma unroll
+    for (int t = 0; t < KT; ++t)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[t][v]);
     mx = fmaxf(mx, __shfl_xor(mx, 32, kWave)) * c;
     // The running maximum is only raised (and the accumulators rescaled) when some query's
     // scores outgrow it by more than 2^8 (see the kernel above).
@@ -405,38 +431,96 @@ __global__ __launch_bounds__(256) void attn_prefill_grouped_kernel(
     }
     const float m_use = m == -INFINITY ? 0.f : m;
     float rowsum = 0.f;
-    bf16x8 pb[2];
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const float p = __builtin_amdgcn_exp2f(fmaf(s[v], c, -m_use));
-      rowsum += p;
-      pb[v >> 3][v & 7] = static_cast<__bf16>(p);
+    for (int t = 0; t < KT; ++t) {
+      bf16x8 pb[2];
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const float p = __builtin_amdgcn_exp2f(fmaf(s[t][v], c, -m_use));
+        rowsum += p;
+        pb[v >> 3][v & 7] = static_cast<__bf16>(p);
+      }
+#pragma unroll
+      for (int cpage = 0; cpage < 2; ++cpage)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          const bf16_t* vr = vd + ((2 * t + cpage) * D + min(32 * dt + col, D - 1)) * VS;
+          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(join(ld4(vr), ld4(vr + 8)), pb[cpage], o[dt], 0, 0, 0);
+        }
     }
     l += rowsum + __shfl_xor(rowsum, 32, kWave);
-#pragma unroll
-    for (int cpage = 0; cpage < 2; ++cpage)
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        const bf16_t* vr = vd + (cpage * D + min(32 * dt + col, D - 1)) * VS;
-        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(join(ld4(vr), ld4(vr + 8)), pb[cpage], o[dt], 0, 0, 0);
-      }
   };
 
   {
-    int stage = 0;
-    load_global(k_begin);
-    for (int k0 = k_begin; k0 <= last_pos; k0 += 32) {
-      store_lds(stage);
-      if (k0 + 32 <= last_pos) load_global(k0 + 32);
-      // Every wave is past the tile that last used this stage: it had to finish it to reach
-      // the previous barrier.
+    // Global loads run two iterations ahead in two register sets, issued whether or not the
+    // keys exist (page lookups are clamped to the last key): memory that missed the L2 takes
+    // longer than one iteration, and with no branch around the loads the wait in front of a
+    // store to LDS counts exactly the older set and leaves the newer one in flight.
+    Pieces ra, rb;
+    int k0 = k_begin, stage = 0;
+    load_global(ra, k0);
+    load_global(rb, k0 + KEYS);
+    while (true) {
+      store_lds(ra, stage);
+      load_global(ra, k0 + 2 * KEYS);
+      // Every wave is past the iteration that last used this stage: it had to finish it to
+      // reach the previous barrier.
       __syncthreads();
       compute(stage, k0);
       stage ^= 1;
+      k0 += KEYS;
+      if (k0 > last_pos) break;
+      store_lds(rb, stage);
+      load_global(rb, k0 + 2 * KEYS);
+      __syncthreads();
+      compute(stage, k0);
+      stage ^= 1;
+      k0 += KEYS;
+      if (k0 > last_pos) break;
     }
   }
 
-  if (!head_valid || !q_valid) return;
+  if (KP > 1) {
+    // Merge the KP runs of keys by log-sum-exp; the K/V stages are free now.
+    constexpr int O_FLOATS = DT * 16 * 64;
+    float* mg = reinterpret_cast<float*>(smem_raw);
+    __syncthreads();
+    if (part > 0) {
+      float* dst = mg + ((part - 1) * 4 + (wave & 3)) * (O_FLOATS + 64);
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) dst[(dt * 16 + v) * 64 + lane] = o[dt][v];
+      if (hi == 0) {
+        dst[O_FLOATS + col] = m;
+        dst[O_FLOATS + 32 + col] = l;
+      }
+    }
+    __syncthreads();
+    if (part == 0) {
+    float mm = m;
+#pragma unroll
+    for (int p = 1; p < KP; ++p) mm = fmaxf(mm, mg[((p - 1) * 4 + wave) * (O_FLOATS + 64) + O_FLOATS + col]);
+    const float f0 = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - mm);
+    l *= f0;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) o[dt][v] *= f0;
+#pragma unroll
+    for (int p = 1; p < KP; ++p) {
+      const float* src = mg + ((p - 1) * 4 + wave) * (O_FLOATS + 64);
+      const float mp = src[O_FLOATS + col];
+      const float f = mp == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mp - mm);
+      l += f * src[O_FLOATS + 32 + col];
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o[dt][v] += f * src[(dt * 16 + v) * 64 + lane];
+    }
+    }
+  }
+  if (part != 0 || !head_valid || !q_valid) continue;
   const float inv = 1.f / l;
   bf16_t* op = out + static_cast<int64_t>(t0 + qi) * (static_cast<int64_t>(hq) * D) + h * D;
 #pragma unroll
@@ -453,6 +537,7 @@ __global__ __launch_bounds__(256) void attn_prefill_grouped_kernel(
         *reinterpret_cast<ushort4*>(op + d) = pk;
       }
     }
+  }
 }
 
 // ------------------------------------------------------------------ decode (split keys)
@@ -646,10 +731,22 @@ __global__ __launch_bounds__(64) void attn_decode_merge_kernel(
   }
 }
 
-// Bytes of LDS the grouped kernel needs for head size D and a block table of table_pages entries.
-static size_t grouped_smem(int D, int table_pages) {
-  return sizeof(bf16_t) * 2 * (32 * static_cast<size_t>(D + 8) + 2 * static_cast<size_t>(D) * (kPage + 4)) +
-         sizeof(int32_t) * static_cast<size_t>(table_pages);
+// Bytes of LDS the grouped kernel needs for head size D, kt 32-key tiles per wave and
+// iteration, kp waves per head and a block table of table_pages entries.
+static size_t grouped_smem(int D, int kt, int kp, int table_pages) {
+  const size_t stages = sizeof(bf16_t) * 2 * kt * kp * (32 * static_cast<size_t>(D + 8) + 2 * static_cast<size_t>(D) * (kPage + 4)) +
+                        sizeof(int32_t) * static_cast<size_t>(table_pages);
+  const size_t merge = sizeof(float) * (kp - 1) * 4 * (static_cast<size_t>((D + 31) / 32) * 16 * 64 + 64);
+  return std::max(stages, merge);
+}
+
+// More than 64 KB of dynamic LDS has to be asked for, kernel by kernel.
+template <typename Kernel>
+static bool lds_allowed(Kernel kernel, size_t bytes) {
+  if (bytes <= 64 * 1024) return true;
+  if (bytes > 160 * 1024) return false;
+  return hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                             static_cast<int>(bytes)) == hipSuccess;
 }
 
 template <int NS>
@@ -657,13 +754,26 @@ static int launch_prefill(hipStream_t s, const void* qkv, int q_stride, void* ou
                           const int32_t* pf_tiles, int n_tiles, int table_pages, const int32_t* item_start, const int32_t* item_pos0,
                           const int32_t* table_off, const int32_t* block_ids, int hq, int hkv, float scale, int window) {
   const int group = hq / hkv;
-  const size_t smem = grouped_smem(16 * NS, table_pages);
-  // Three or more query heads per kv head: they share the keys and values through LDS.
-  if (group >= 3 && smem <= 64 * 1024) {
-    attn_prefill_grouped_kernel<NS><<<dim3(n_tiles, hkv * ((group + 3) / 4)), dim3(256), smem, s>>>(
-        static_cast<const bf16_t*>(qkv), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(kv), pf_tiles,
-        item_start, item_pos0, table_off, block_ids, hq, hkv, table_pages, scale, window);
-    return check_launch("psamd_attention_prefill");
+  // Three or more query heads per kv head: they share the keys and values through LDS, two
+  // waves per head (each its own run of keys) if the stages fit, else one.
+  if (group >= 3) {
+    const dim3 grid((n_tiles + 1) / 2, hkv * ((group + 3) / 4));
+#define PSAMD_GROUPED(KP_)                                                                                         \
+  {                                                                                                               \
+    const size_t smem = grouped_smem(16 * NS, 1, KP_, table_pages);                                               \
+    if (lds_allowed(attn_prefill_grouped_kernel<NS, 1, KP_>, smem)) {                                             \
+      attn_prefill_grouped_kernel<NS, 1, KP_><<<grid, dim3(256 * KP_), smem, s>>>(                                \
+          static_cast<const bf16_t*>(qkv), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(kv),   \
+          pf_tiles, item_start, item_pos0, table_off, block_ids, n_tiles, hq, hkv, table_pages, scale, window);   \
+      return check_launch("psamd_attention_prefill");                                                             \
+    }                                                                                                             \
+  }
+#ifdef PSAMD_PF_KP4
+    PSAMD_GROUPED(4)
+#endif
+    PSAMD_GROUPED(2)
+    PSAMD_GROUPED(1)
+#undef PSAMD_GROUPED
   }
   attn_prefill_mfma_kernel<NS><<<dim3(n_tiles, hq), dim3(256), sizeof(int32_t) * static_cast<size_t>(table_pages), s>>>(
       static_cast<const bf16_t*>(qkv), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(kv), pf_tiles,
