@@ -289,7 +289,8 @@ def paged_case(ops, act, hq, hkv, d, lens_new, lens_old, window=None, seed=0, nu
     return out.view(t, hq, d), want
 
 
-SHAPES = [(4, 2, 16), (3, 1, 32), (8, 2, 64), (32, 8, 64), (6, 6, 96), (8, 1, 128), (40, 2, 64), (2, 2, 256), (6, 3, 48), (2, 1, 80)]
+SHAPES = [(4, 2, 16), (3, 1, 32), (8, 2, 64), (32, 8, 64), (6, 6, 96), (8, 1, 128), (40, 2, 64), (2, 2, 256), (6, 3, 48), (2, 1, 80),
+          (6, 2, 256), (12, 4, 128), (5, 1, 32), (9, 3, 96)]
 
 
 @pytest.mark.parametrize("hq,hkv,d", SHAPES)
