@@ -73,6 +73,8 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / batch 64 points")
     ap.add_argument("--no-graphs", action="store_true")
+    ap.add_argument("--decode-steps", type=int, default=8,
+                    help="decode steps per scheduler round (the host reads the tokens once per round)")
     ap.add_argument("--prefill-reps", type=int, default=5, help="timed repetitions of the 2,048-token prefill")
     ap.add_argument("--model", default=None, help="use this model folder instead of writing random weights")
     ap.add_argument("--shape", choices=sorted(SHAPES), default="llama-3.2-1b", help="layer sizes of the random model")
@@ -129,10 +131,12 @@ def main() -> int:
         kv_start = sum(r.num_computed for r in sched._requests.values())
         sync()
         t0 = time.perf_counter()
-        for _ in range(steps):
-            bt = sched.schedule_step(args.prompt_len, batch)
+        done = 0
+        while done < steps:
+            bt = sched.schedule_step(args.prompt_len, batch, min(args.decode_steps, steps - done))
             assert len(bt.work) == batch and bt.num_tokens == batch
             sched.commit(bt, engine.step(bt))
+            done += bt.decode_steps
         sync()
         dt = time.perf_counter() - t0
         kv_end = sum(r.num_computed for r in sched._requests.values())
@@ -180,7 +184,7 @@ def main() -> int:
             "intermediate": cfg["intermediate_size"], "vocab": vocab, "rope_theta": cfg["rope_theta"],
             "rope_factor": (cfg.get("rope_scaling") or {}).get("factor"), "rms_norm_eps": cfg["rms_norm_eps"],
             "tied": cfg.get("tie_word_embeddings", False), "global_batch": args.batch, "seq_len": args.context,
-            "prompt_len": args.prompt_len, "page_tokens": 16, "parallelism": "none",
+            "prompt_len": args.prompt_len, "page_tokens": 16, "decode_steps": args.decode_steps, "parallelism": "none",
         },
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": main_run["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",

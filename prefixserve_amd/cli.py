@@ -30,6 +30,8 @@ def _add_engine_options(p: argparse.ArgumentParser) -> None:
     p.add_argument("--chunked-prefill-size", type=int, default=512)
     p.add_argument("--disable-prefix-cache", action="store_true")
     p.add_argument("--no-graphs", action="store_true", help="do not capture decode steps as HIP graphs")
+    p.add_argument("--decode-steps", type=int, default=1,
+                   help="decode steps a batch of decoding requests runs before the host looks at the tokens")
 
 
 def _generate(args: argparse.Namespace) -> int:
@@ -40,7 +42,8 @@ def _generate(args: argparse.Namespace) -> int:
 
     cfg = EngineConfig(model_path=Path(args.model), dtype=args.dtype, max_num_seqs=args.max_running_requests,
                        max_prefill_tokens=args.chunked_prefill_size, max_seq_len=args.max_seq_len,
-                       num_blocks=args.num_blocks, use_graphs=not args.no_graphs, sample_seed=args.sample_seed)
+                       num_blocks=args.num_blocks, use_graphs=not args.no_graphs, sample_seed=args.sample_seed,
+                       decode_steps=args.decode_steps)
     engine = Engine(cfg)
     prompts: list[list[int]] = [[int(t) for t in s.split(",") if t.strip()] for s in (args.prompt_ids or [])]
     if args.prompt_len:

@@ -33,6 +33,11 @@ class EngineConfig:
     reserve_bytes: int = 1 << 30
     use_graphs: bool = True              # replay decode-only steps as captured HIP graphs
     sample_seed: int = 0
+    # Decode steps a batch of decoding requests may run before the host looks at the tokens
+    # (1 = after every step). More hides the host's work behind the device's; a request that
+    # meets a stop token in between has computed up to decode_steps - 1 tokens for nothing, and
+    # a request that arrives waits until the running batch has finished its steps.
+    decode_steps: int = 1
 
 
 class Engine:
@@ -98,10 +103,38 @@ class Engine:
             out.append(arr[:n])
         return out
 
+    def _decode_steps(self, batch: Batch) -> dict[str, list[int]]:
+        """``batch.decode_steps`` steps in a row for a batch of decoding requests. The token a
+        step samples stays on the device and is the next step's input there; the host packs
+        the next step's integers while the device runs the current one and waits once, at the
+        end, for all tokens."""
+        k, reqs = batch.decode_steps, [w.req for w in batch.work]
+        for w in batch.work:
+            if w.start + k > self.cfg.max_seq_len:
+                raise EngineError(f"{w.req.req_id}: position {w.start + k} > max_seq_len {self.cfg.max_seq_len}")
+        temps = [r.temperature for r in reqs]
+        uniforms = [[uniform_for(self.cfg.sample_seed ^ r.seed, request_key(r.req_id), len(r.output) + j)
+                     if r.temperature > 0 else 0.0 for r in reqs] for j in range(k)]
+        t_dev, u_dev, out_dev = self.sampler.stage_steps(temps, uniforms)
+        tables = [self._table_arrays(r) for r in reqs]
+        first = [r.tokens(w.start, w.end) for r, w in zip(reqs, batch.work)]
+        for j in range(k):
+            items = [StepItem(key=r.req_id, tokens=first[i] if j == 0 else (0,), start=w.start + j,
+                              block_tables=tables[i], slot=max(r.slot, 0), want=(0,))
+                     for i, (r, w) in enumerate(zip(reqs, batch.work))]
+            logits = self.runner.step(items, token_feed=out_dev[j - 1] if j else None)
+            assert logits is not None
+            self.sampler.sample_into(logits, t_dev, u_dev[j], out_dev[j])
+        rows = self.sampler.fetch(k, len(reqs))
+        return {r.req_id: [rows[j][i] for j in range(k)] for i, r in enumerate(reqs)}
+
     def step(self, batch: Batch) -> dict[str, int]:
-        """Runs one batch; returns req_id -> next token for the items that sample."""
+        """Runs one batch; returns req_id -> next token for the items that sample (a list of
+        tokens each for a batch of several decode steps)."""
         if not batch.work:
             return {}
+        if batch.decode_steps > 1:
+            return self._decode_steps(batch)
         if len(batch.work) > self.cfg.max_num_seqs:
             raise EngineError(f"batch of {len(batch.work)} requests is over max_num_seqs {self.cfg.max_num_seqs}")
         items, sampling = [], []

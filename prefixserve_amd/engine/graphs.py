@@ -24,12 +24,14 @@ if TYPE_CHECKING:
     from prefixserve_amd.engine.runner import ModelRunner
 
 
-def graphed_decode_step(runner: "ModelRunner", items: Sequence[StepItem]) -> Any:
+def graphed_decode_step(runner: "ModelRunner", items: Sequence[StepItem], token_feed: Any = None) -> Any:
     wanted = sum(len(it.want) for it in items)
     key = (len(items), wanted)
     static_pages = -(-runner.max_seq_len // PAGE)
     ops, ws, packer = runner.ops, runner.workspace, runner.packer
     ctx = packer.pack(items, static_pages=static_pages)
+    if token_feed is not None:
+        ctx.token_ids.copy_(token_feed)    # in stream order after the packed integers, before the graph
     entry = runner._graphs.get(key)
     if entry is not None and entry[2] == (packer.version, ws.version):
         entry[0].replay()

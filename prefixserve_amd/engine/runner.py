@@ -140,18 +140,24 @@ class ModelRunner:
     # ------------------------------------------------------------------ step
 
     @torch.inference_mode()
-    def step(self, items: Sequence[StepItem]) -> torch.Tensor | None:
+    def step(self, items: Sequence[StepItem], token_feed: torch.Tensor | None = None) -> torch.Tensor | None:
         """One step: runs exactly the given tokens as one batch from the cache that earlier
         steps left, and returns float32 logits ``[S, vocab]`` in the order of the items and
         of their ``want`` (None if nothing is wanted). Steps run strictly in order on the
-        current stream, so step N+1 reads what step N wrote."""
+        current stream, so step N+1 reads what step N wrote.
+
+        ``token_feed``: int32 ``[T]`` on the device, taken for the step's token ids instead of
+        the items' own (which must still be valid ids): the tokens an earlier step sampled and
+        the host has not seen yet."""
         if self.use_graphs and all(len(it.tokens) == 1 for it in items):
             from prefixserve_amd.engine.graphs import graphed_decode_step
 
-            out = graphed_decode_step(self, items)
+            out = graphed_decode_step(self, items, token_feed)
             if out is not NotImplemented:
                 return out
         ctx = self.packer.pack(items)
+        if token_feed is not None:
+            ctx.token_ids.copy_(token_feed)
         return self.model.step(ctx)
 
     def pack(self, items: Sequence[StepItem]) -> StepContext:

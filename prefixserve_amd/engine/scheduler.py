@@ -120,8 +120,13 @@ class WorkItem:
 
 @dataclass(frozen=True)
 class Batch:
+    """``decode_steps`` > 1: every item is a decoding request and the engine runs that many
+    steps in a row for them (item j of a request starts at ``start + j``), feeding each step's
+    token to the next on the device; ``commit`` then takes a list of tokens per request."""
+
     work: list[WorkItem]
     preempted: list[str]
+    decode_steps: int = 1
 
     @property
     def num_tokens(self) -> int:
@@ -130,8 +135,12 @@ class Batch:
 
 @dataclass(frozen=True)
 class StepResult:
+    """``new_tokens``: the last token each request got in this commit; ``tokens``: all of
+    them in order (more than one after a batch of several decode steps)."""
+
     new_tokens: dict[str, int]
     finished: dict[str, FinishReason]
+    tokens: dict[str, list[int]] = field(default_factory=dict)
 
 
 @dataclass(frozen=True)
@@ -196,8 +205,14 @@ class Scheduler:
         self._prompt_tokens += len(checked)
         return AddResult.ACCEPTED
 
-    def schedule_step(self, max_prefill_tokens: int, max_decode_seqs: int) -> Batch:
-        """Chooses this step's work. ``commit`` must follow before the next call."""
+    def schedule_step(self, max_prefill_tokens: int, max_decode_seqs: int, decode_steps: int = 1) -> Batch:
+        """Chooses this step's work. ``commit`` must follow before the next call.
+
+        ``decode_steps`` > 1 lets a batch that holds nothing but decoding requests, with nobody
+        waiting, run up to that many steps before the host looks at the tokens (fewer if a
+        request would pass its ``max_tokens`` or the free pages do not reach). A request that
+        meets a stop token in between finishes there; what was computed for it after that is
+        dropped. Nothing else changes: the pages for those positions are taken now."""
         if self._inflight is not None:
             raise SchedulerError("commit() the previous batch before scheduling another")
         if max_prefill_tokens < 1 or max_decode_seqs < 1:
@@ -235,7 +250,22 @@ class Scheduler:
                 budget -= item.end - item.start
             work.append(item)
 
-        batch = Batch(work=work, preempted=preempted)
+        steps = 1
+        if (decode_steps > 1 and work and not self._waiting and not preempted
+                and all(w.end - w.start == 1 and w.samples for w in work)):
+            steps = min(decode_steps, min(w.req.max_tokens - len(w.req.output) for w in work))
+            for w in work:
+                if steps == 1:
+                    break
+                need = [max(blocks_for(w.start + steps) - len(t), 0) for t in w.req.block_tables]
+                if any(need):
+                    fresh = self.cache.allocate(need)
+                    if fresh is None:
+                        steps = 1        # pages already taken for others stay theirs: they will be used
+                    else:
+                        for table, new in zip(w.req.block_tables, fresh):
+                            table.extend(new)
+        batch = Batch(work=work, preempted=preempted, decode_steps=steps)
         self._inflight = batch
         elapsed = time.perf_counter() - started
         if elapsed > SLOW_STEP_SECONDS:
@@ -248,38 +278,47 @@ class Scheduler:
             raise SchedulerError("commit() got a batch that isn't the one in flight")
         self._inflight = None
         new_tokens: dict[str, int] = {}
+        all_tokens: dict[str, list[int]] = {}
         finished: dict[str, FinishReason] = {}
         for w in batch.work:
             req = w.req
             if req.num_computed != w.start:
                 raise SchedulerError(f"{req.req_id}: batch is stale")
-            reached_end = w.samples
-            req.num_computed = w.end
-            self.cache.trim_windows(req.block_tables, req.num_computed)
-            if not reached_end:
+            if not w.samples:
+                req.num_computed = w.end
+                self.cache.trim_windows(req.block_tables, req.num_computed)
                 continue
             if req.req_id not in sampled:
                 raise SchedulerError(f"engine returned no token for {req.req_id}")
-            token = int(sampled[req.req_id])
-            if not req.prompt_cached:      # prompt complete for the first time: share it now
-                self._cache(req)
-                req.prompt_cached = True
-            req.output.append(token)
-            new_tokens[req.req_id] = token
-            if req.abort_pending:
-                continue
-            if token in self._stop and not req.ignore_eos:
-                self._finish(req, FinishReason.STOP)
-                finished[req.req_id] = FinishReason.STOP
-            elif len(req.output) >= req.max_tokens:
-                self._finish(req, FinishReason.LENGTH)
-                finished[req.req_id] = FinishReason.LENGTH
+            got = sampled[req.req_id]
+            tokens = [int(got)] if isinstance(got, (int, np.integer)) else [int(t) for t in got]
+            if len(tokens) != batch.decode_steps:
+                raise SchedulerError(f"{req.req_id}: {len(tokens)} tokens for {batch.decode_steps} decode steps")
+            for j, token in enumerate(tokens):
+                req.num_computed = w.end + j
+                self.cache.trim_windows(req.block_tables, req.num_computed)
+                if not req.prompt_cached:      # prompt complete for the first time: share it now
+                    self._cache(req)
+                    req.prompt_cached = True
+                req.output.append(token)
+                new_tokens[req.req_id] = token
+                all_tokens.setdefault(req.req_id, []).append(token)
+                if req.abort_pending:
+                    break
+                if token in self._stop and not req.ignore_eos:
+                    self._finish(req, FinishReason.STOP)
+                    finished[req.req_id] = FinishReason.STOP
+                    break
+                if len(req.output) >= req.max_tokens:
+                    self._finish(req, FinishReason.LENGTH)
+                    finished[req.req_id] = FinishReason.LENGTH
+                    break
         for req in self._pending_aborts:   # safe now: the batch that wrote their pages is done
             if req.state is ReqState.RUNNING:
                 self._finish(req, FinishReason.ABORT)
                 finished[req.req_id] = FinishReason.ABORT
         self._pending_aborts.clear()
-        return StepResult(new_tokens=new_tokens, finished=finished)
+        return StepResult(new_tokens=new_tokens, finished=finished, tokens=all_tokens)
 
     def free_request(self, req_id: str) -> bool:
         """Aborts a request. False for an unknown id or a second call."""

@@ -27,8 +27,11 @@ class Generation:
 def generate(engine: Engine, prompts: Sequence[Iterable[int]], max_tokens: int, *, temperature: float = 0.0,
              seed: int = 0, ignore_eos: bool = False, scheduler: Scheduler | None = None,
              max_prefill_tokens: int | None = None, max_running_requests: int | None = None,
-             enable_prefix_cache: bool = True) -> tuple[list[Generation], SchedulerStats]:
-    """Generates up to ``max_tokens`` tokens for every prompt (token ids in, token ids out)."""
+             enable_prefix_cache: bool = True, decode_steps: int | None = None) -> tuple[list[Generation], SchedulerStats]:
+    """Generates up to ``max_tokens`` tokens for every prompt (token ids in, token ids out).
+    ``decode_steps``: how many decode steps a batch of decoding requests may run before the
+    host looks at the tokens (default: the engine configuration's)."""
+    steps = decode_steps if decode_steps is not None else engine.cfg.decode_steps
     budget = max_prefill_tokens if max_prefill_tokens is not None else engine.cfg.max_prefill_tokens
     running = max_running_requests if max_running_requests is not None else engine.cfg.max_num_seqs
     sched = scheduler if scheduler is not None else engine.make_scheduler(
@@ -44,14 +47,14 @@ def generate(engine: Engine, prompts: Sequence[Iterable[int]], max_tokens: int, 
             raise ValueError(f"{rid} rejected: {res.value}")
         results[rid] = Generation(rid, ids)
     while sched.has_work():
-        batch = sched.schedule_step(budget, running)
+        batch = sched.schedule_step(budget, running, steps)
         if not batch.work:
             raise RuntimeError("the scheduler has work but could schedule none of it (pool too small?)")
         tracked = {w.req.req_id: w.req for w in batch.work}
         sampled = engine.step(batch)
         step = sched.commit(batch, sampled)
-        for rid, tok in step.new_tokens.items():
-            results[rid].tokens.append(tok)
+        for rid, toks in step.tokens.items():
+            results[rid].tokens.extend(toks)
         for rid, why in step.finished.items():
             g, r = results[rid], tracked.get(rid)
             g.finish_reason = why

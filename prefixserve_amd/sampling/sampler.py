@@ -84,3 +84,45 @@ class Sampler:
             torch.cuda.current_stream(self.device).synchronize()
             return self._out_np[:rows].tolist()
         return out.tolist()
+
+    # ---- several steps in a row: nothing here waits for the device but ``fetch``
+
+    def stage_steps(self, temperatures: Sequence[float], uniforms: Sequence[Sequence[float]]):
+        """Device copies of the temperatures and of one row of uniform numbers per step, made
+        with one host-to-device copy; and a device buffer for ``len(uniforms)`` rows of tokens."""
+        rows, steps = len(temperatures), len(uniforms)
+        need = (steps + 1) * rows
+        if getattr(self, "_steps_cap", 0) < need:
+            pin = self.device.type == "cuda"
+            self._steps_host = torch.empty(need, dtype=torch.float32, pin_memory=pin)
+            self._steps_dev = torch.zeros(need, dtype=torch.float32, device=self.device)
+            self._steps_out = torch.empty(need, dtype=torch.int32, device=self.device)
+            self._steps_out_host = torch.empty(need, dtype=torch.int32, pin_memory=pin)
+            self._steps_cap = need
+            self._steps_greedy = need
+        greedy = not any(t > 0 for t in temperatures)
+        if not (greedy and self._steps_greedy >= need):
+            host = self._steps_host.numpy()
+            host[:rows] = temperatures
+            for j, u in enumerate(uniforms):
+                host[(j + 1) * rows:(j + 2) * rows] = u
+            self._steps_dev[:need].copy_(self._steps_host[:need], non_blocking=True)
+            self._steps_greedy = need if greedy else 0
+        temps = self._steps_dev[:rows]
+        return temps, [self._steps_dev[(j + 1) * rows:(j + 2) * rows] for j in range(steps)], \
+            [self._steps_out[j * rows:(j + 1) * rows] for j in range(steps)]
+
+    def sample_into(self, logits: torch.Tensor, temperatures: torch.Tensor, uniforms: torch.Tensor,
+                    out: torch.Tensor) -> None:
+        self.ops.sample(logits, temperatures, uniforms, out)
+
+    def fetch(self, steps: int, rows: int) -> list[list[int]]:
+        """The tokens of ``stage_steps``' output rows: the one device-to-host wait."""
+        n = steps * rows
+        if self.device.type == "cuda":
+            self._steps_out_host[:n].copy_(self._steps_out[:n], non_blocking=True)
+            torch.cuda.current_stream(self.device).synchronize()
+            flat = self._steps_out_host.numpy()[:n]
+        else:
+            flat = self._steps_out[:n].numpy()
+        return flat.reshape(steps, rows).tolist()

@@ -156,3 +156,27 @@ def test_engine_refuses_without_kernels_on_cpu(model_dirs):
 
     with pytest.raises(KernelError, match="GPU only"):
         ModelRunner(model_dirs["A"], dtype="float32", device="cpu", num_blocks=4, max_seq_len=64)
+
+
+@pytest.mark.parametrize("temperature", [0.0, 0.8])
+def test_several_decode_steps_give_the_same_tokens(temperature, model_dirs, plain_models):
+    """Running four decode steps before the host reads the tokens changes no token, greedy or
+    sampled: each step's token reaches the next on the device, the draws depend only on
+    (seed, request, output index). A stop token inside the four ends the request there."""
+    eng = Engine(EngineConfig(model_path=model_dirs["A"], dtype="float32", device="cpu", max_num_seqs=4,
+                              max_prefill_tokens=64, max_seq_len=128, num_blocks=32, use_graphs=False, sample_seed=2),
+                 ops=EmulatedOps())
+    rng = np.random.default_rng(11)
+    prompts = [rng.integers(3, 256, n).tolist() for n in (12, 30, 7)]
+    one, _ = generate(eng, prompts, 11, temperature=temperature, ignore_eos=True)
+    four, _ = generate(eng, prompts, 11, temperature=temperature, ignore_eos=True, decode_steps=4)
+    assert [o.tokens for o in one] == [o.tokens for o in four]
+    if temperature == 0.0:
+        assert one[0].tokens == plain_models["A"].greedy(prompts[0], 11)[0]
+        sched = eng.make_scheduler()
+        sched._stop = frozenset({one[1].tokens[5]})
+        stopped, _ = generate(eng, prompts, 11, scheduler=sched, decode_steps=4)
+        for o, full in zip(stopped, one):
+            cut = next((i for i, t in enumerate(full.tokens) if t in sched._stop), None)
+            assert o.tokens == (full.tokens if cut is None else full.tokens[:cut + 1])
+    assert eng.make_cache().num_free(0) == 32

@@ -142,3 +142,23 @@ def test_a_hundred_requests_decode_together(dtype, model_dirs, plain_models):
                 assert row[best] - row[tok] < 0.05 * np.abs(row).max(), "left the plain model at a clear margin"
                 break
             seq.append(tok)
+
+
+def test_several_decode_steps_before_the_host_reads(model_dirs, plain_models):
+    """Five decode steps per scheduler round through captured graphs: the same tokens as one
+    step per round, greedy (equal to the plain model's) and sampled, with a pool so small
+    that rounds fall back to single steps now and then."""
+    from prefixserve_amd import Engine, EngineConfig, generate
+
+    name = "B"
+    rng = np.random.default_rng(21)
+    prompts = [rng.integers(3, 512, n).tolist() for n in (33, 5, 18, 47)]
+    eng = Engine(EngineConfig(model_path=model_dirs[name], dtype="float32", max_num_seqs=4, max_prefill_tokens=64,
+                              max_seq_len=128, num_blocks=20, sample_seed=4, decode_steps=5))
+    many, stats = generate(eng, prompts, 23, ignore_eos=True)
+    for p, o in zip(prompts, many):
+        assert o.tokens == plain_models[name].greedy(p, 23)[0]
+    one_t, _ = generate(eng, prompts, 23, temperature=0.7, ignore_eos=True, decode_steps=1)
+    many_t, _ = generate(eng, prompts, 23, temperature=0.7, ignore_eos=True)
+    assert [o.tokens for o in one_t] == [o.tokens for o in many_t]
+    assert [o.tokens for o in one_t] != [o.tokens for o in many]

@@ -296,3 +296,42 @@ def test_random_load_keeps_the_ref_count_invariant():
         s.cache.check_invariants()
     run_until_done(s, budget=24, max_seqs=4)
     assert_clean(s)
+
+
+def test_several_decode_steps_in_one_batch():
+    """A batch of nothing but decodes, nobody waiting: up to decode_steps steps, bounded by
+    max_tokens and by the free pages; commit takes that many tokens per request and stops a
+    request at its stop token."""
+    s = Scheduler(num_blocks=16, stop_token_ids=[7])
+    s.add_request("a", toks(20), 9, ignore_eos=True)
+    s.add_request("b", toks(30, 50), 30)
+    first = s.schedule_step(2048, 8, decode_steps=4)
+    assert first.decode_steps == 1                                     # prompts: one step
+    s.commit(first, {"a": 1, "b": 1})
+    batch = s.schedule_step(2048, 8, decode_steps=4)
+    assert batch.decode_steps == 4 and [(w.start, w.end) for w in batch.work] == [(20, 21), (30, 31)]
+    assert len(s.get_request("a").block_table) == 2 and len(s.get_request("b").block_table) == 3   # 24 and 34 positions
+    res = s.commit(batch, {"a": [2, 3, 4, 5], "b": [2, 7, 8, 9]})      # b meets its stop token at the second step
+    assert res.tokens == {"a": [2, 3, 4, 5], "b": [2, 7]} and res.finished == {"b": FinishReason.STOP}
+    assert s.get_request("a").num_computed == 24 and s.get_request("a").output == [1, 2, 3, 4, 5]
+    batch = s.schedule_step(2048, 8, decode_steps=8)
+    assert batch.decode_steps == 4                                     # max_tokens 9, 5 made
+    res = s.commit(batch, {"a": [6, 7, 8, 9]})                         # ignore_eos: 7 does not stop it
+    assert res.finished == {"a": FinishReason.LENGTH} and not s.has_work()
+    assert_clean(s)
+
+
+def test_decode_steps_fall_back_to_one():
+    s = Scheduler(num_blocks=4)                                        # 64 positions in all
+    s.add_request("a", toks(30), 20, ignore_eos=True)
+    s.add_request("b", toks(30, 40), 20, ignore_eos=True)
+    step(s)
+    batch = s.schedule_step(2048, 8, decode_steps=8)                   # 32 + 8 positions each: no pages for that
+    assert batch.decode_steps == 1
+    s.commit(batch, sample(batch))
+    s.add_request("c", toks(5, 90), 4)
+    batch = s.schedule_step(2048, 1, decode_steps=2)                   # somebody waits: one step at a time
+    assert batch.decode_steps == 1 and s.stats().num_waiting == 1
+    s.commit(batch, sample(batch))
+    run_until_done(s)
+    assert_clean(s)
