@@ -10,6 +10,7 @@ every 32-bit product and every product with at most 64 rows is a kernel of this 
 
 from __future__ import annotations
 
+import os
 import ctypes
 from typing import Any
 
@@ -261,7 +262,7 @@ class HipOps:
                 kv_len = self.decode_split_kv_len or ctx.max_kv_len
                 if win:
                     kv_len = min(kv_len, win)
-                nsplit = max(1, min(64, 1024 // (ctx.num_decode * hkv), -(-kv_len // 128)))
+                nsplit = max(1, min(64, 512 // (ctx.num_decode * hkv), -(-kv_len // 128)))
                 part_o = self.ws.get("attn.part_o", (ctx.num_decode * hq * nsplit * d,), torch.float32)
                 part_ml = self.ws.get("attn.part_ml", (ctx.num_decode * hq * nsplit * 2,), torch.float32)
                 self._ok(self.lib.psamd_attention_decode(
