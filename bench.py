@@ -76,6 +76,7 @@ def main() -> int:
     ap.add_argument("--decode-steps", type=int, default=8,
                     help="decode steps per scheduler round (the host reads the tokens once per round)")
     ap.add_argument("--prefill-reps", type=int, default=5, help="timed repetitions of the 2,048-token prefill")
+    ap.add_argument("--no-peaks", action="store_true", help="skip measuring the copy bandwidth and a large library product")
     ap.add_argument("--model", default=None, help="use this model folder instead of writing random weights")
     ap.add_argument("--shape", choices=sorted(SHAPES), default="llama-3.2-1b", help="layer sizes of the random model")
     args = ap.parse_args()
@@ -166,6 +167,26 @@ def main() -> int:
         return {"value": n / (ms / 1e3), "tokens": n, "ms": ms,
                 "frac": flops / (ms / 1e3) / (MFMA_PEAK_TFLOPS[args.dtype] * 1e12)}
 
+    def measured_peaks() -> dict:
+        """What this GPU delivers on the two simplest workloads, to set beside the published
+        peaks: a 1 GiB device copy (bytes read + written per second) and an 8192^3 library product."""
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        a = torch.randn(8192, 8192, device="cuda").to(torch.bfloat16 if args.dtype == "bfloat16" else torch.float32)
+        out = {}
+        for name, fn, work in (("copy_gbs", lambda: dst.copy_(src), 2 * src.numel() / 1e9),
+                               ("product_tflops", lambda: torch.matmul(a, a), 2 * 8192 ** 3 / 1e12)):
+            for _ in range(2):
+                fn()
+            sync()
+            t0 = time.perf_counter()
+            for _ in range(5):
+                fn()
+            sync()
+            out[name] = work * 5 / (time.perf_counter() - t0)
+        return out
+
+    peaks = {} if args.no_peaks else measured_peaks()
     prefill = prefill_run(reps=args.prefill_reps)
     main_run = decode_run(args.batch, args.steps, args.warmup)
     points = {}
@@ -190,6 +211,7 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": main_run["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": main_run["gbs"] / HBM_PEAK_GBS},
         "points": points,
+        "measured_peaks": peaks,
     }
     print(json.dumps(line), flush=True)
     if tmp is not None:

@@ -48,8 +48,11 @@ def _generate(args: argparse.Namespace) -> int:
     prompts: list[list[int]] = [[int(t) for t in s.split(",") if t.strip()] for s in (args.prompt_ids or [])]
     if args.prompt_len:
         rng = np.random.default_rng(args.seed)
-        prompts += [rng.integers(0, engine.runner.vocab_size, args.prompt_len).tolist()
-                    for _ in range(args.num_prompts)]
+        shared = rng.integers(0, engine.runner.vocab_size, min(args.shared_prefix_len, args.prompt_len)).tolist()
+        for i in range(args.num_prompts):
+            own = rng.integers(0, engine.runner.vocab_size, args.prompt_len).tolist()
+            # every second random prompt starts with the shared prefix
+            prompts.append(shared + own[len(shared):] if shared and i % 2 == 0 else own)
     if not prompts:
         print("give --prompt-ids or --prompt-len", file=sys.stderr)
         return 2
@@ -62,7 +65,8 @@ def _generate(args: argparse.Namespace) -> int:
     dt = time.perf_counter() - t0
     new = sum(len(o.tokens) for o in outs)
     print(json.dumps({
-        "outputs": [{"id": o.req_id, "tokens": o.tokens, "finish_reason": o.finish_reason.value if o.finish_reason else None,
+        "outputs": [] if args.quiet else
+                   [{"id": o.req_id, "tokens": o.tokens, "finish_reason": o.finish_reason.value if o.finish_reason else None,
                      "cached_tokens": o.cached_tokens, "preemptions": o.preemptions} for o in outs],
         "stats": {"seconds": dt, "new_tokens": new, "tokens_per_second": new / dt if dt > 0 else None,
                   "prompt_tokens": stats.prompt_tokens, "cached_prompt_tokens": stats.cached_prompt_tokens,
@@ -96,6 +100,9 @@ def main(argv: list[str] | None = None) -> int:
     g.add_argument("--prompt-ids", action="append", help="comma-separated token ids; may be repeated")
     g.add_argument("--prompt-len", type=int, default=0, help="make random prompts of this many ids")
     g.add_argument("--num-prompts", type=int, default=1)
+    g.add_argument("--shared-prefix-len", type=int, default=0,
+                   help="every second random prompt starts with the same ids of this length")
+    g.add_argument("--quiet", action="store_true", help="print the statistics only, not the tokens")
     g.add_argument("--seed", type=int, default=0, help="seed of the random prompt ids")
     g.set_defaults(run=_generate)
 
