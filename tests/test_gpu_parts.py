@@ -347,6 +347,34 @@ def test_windowed_attention_through_the_engine(tmp_path):
                 p0 += c
             assert all(rp.cache.num_free(g) == rp.cache.num_blocks(g) for g in range(2))
 
+    # The same architecture through the scheduler: pages of the window group go back while the
+    # requests run, also when several decode steps are taken per round.
+    from prefixserve_amd import Engine, EngineConfig, generate
+
+    prompts = [toks[:70], toks[40:75], toks[90:97]]
+    eng = Engine(EngineConfig(model_path=tmp_path, dtype="float32", max_num_seqs=3, max_prefill_tokens=32, max_seq_len=160,
+                              num_blocks=12))
+    one, _ = generate(eng, prompts, 40, ignore_eos=True)
+    four, _ = generate(eng, prompts, 40, ignore_eos=True, decode_steps=4)
+    assert [o.tokens for o in one] == [o.tokens for o in four]
+    seq = list(prompts[2])
+    for tok in one[2].tokens[:6]:                                  # against the plain functions, token by token
+        hh = w["emb.weight"][seq]
+        nn = len(seq)
+        cs, sn = P.rope_cos_sin(np.arange(nn), P.rope_inv_freq(D, 10000.0, None))
+        for i, window in enumerate((WINDOW, None)):
+            pp = f"l{i}."
+            x = P.rms_norm(hh, w[pp + "n1.weight"], 1e-5)
+            q = P.apply_rope((x @ w[pp + "q.weight"].T).reshape(nn, HQ, D), cs, sn)
+            k = P.apply_rope((x @ w[pp + "k.weight"].T).reshape(nn, HKV, D), cs, sn)
+            v = (x @ w[pp + "v.weight"].T).reshape(nn, HKV, D)
+            hh = hh + P.causal_attention(q, k, v, window).reshape(nn, HQ * D) @ w[pp + "o.weight"].T
+            x = P.rms_norm(hh, w[pp + "n2.weight"], 1e-5)
+            hh = hh + P.swiglu_mlp(x, w[pp + "g.weight"], w[pp + "u.weight"], w[pp + "d.weight"])
+        row = P.rms_norm(hh[-1:], w["norm.weight"], 1e-5) @ w["emb.weight"].T
+        assert tok == int(np.argmax(row[0]))
+        seq.append(tok)
+
 
 def test_a_toy_position_encoding_and_a_routed_feed_forward(tmp_path):
     """Two more parts defined and registered from this test only: a position encoding whose
