@@ -178,3 +178,55 @@ def test_trace_run_program(dtype, model_dirs, plain_models, tmp_path):
     finally:
         if proc.poll() is None:
             proc.kill()
+
+
+def _random_config(rng):
+    """A configuration the architecture allows, drawn so that every kernel path is met over a
+    few seeds: head sizes with and without a matrix-core kernel, groups of 1 to 8, widths and
+    vocabularies that are no multiple of 8 (the small-step products then refuse and the
+    general one runs), rope scaling on or off, tied or not."""
+    d = int(rng.choice([16, 32, 48, 64, 80, 96, 112, 128]))
+    hkv = int(rng.choice([1, 2, 3]))
+    group = int(rng.choice([1, 2, 3, 4, 5, 8]))
+    hidden = int(rng.choice([40, 72, 100, 136, 200]))
+    cfg = dict(architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=int(rng.integers(90, 700)),
+               hidden_size=hidden, intermediate_size=int(rng.choice([44, 96, 150, 264])),
+               num_hidden_layers=int(rng.integers(1, 4)), num_attention_heads=hkv * group, num_key_value_heads=hkv,
+               head_dim=d, rms_norm_eps=float(rng.choice([1e-5, 1e-6, 3e-4])), rope_theta=float(rng.choice([1e4, 5e5])),
+               max_position_embeddings=1024, tie_word_embeddings=bool(rng.integers(0, 2)))
+    if rng.integers(0, 2):
+        cfg["rope_scaling"] = dict(rope_type="llama3", factor=float(rng.choice([4.0, 8.0, 32.0])), low_freq_factor=1.0,
+                                   high_freq_factor=4.0, original_max_position_embeddings=int(rng.choice([32, 64, 256])))
+    return cfg
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2, 3, 4, 5, 6, 7])
+def test_random_configurations_in_both_dtypes(seed, tmp_path):
+    from configs import INIT_STD
+    from plain.llama_plain import PlainLlama
+    from prefixserve_amd.weights import write_random_model
+
+    rng = np.random.default_rng(1000 + seed)
+    cfg = _random_config(rng)
+    write_random_model(tmp_path, cfg, seed=seed, std=INIT_STD)
+    plain = PlainLlama(tmp_path)
+    reqs = [rng.integers(0, cfg["vocab_size"], n).tolist() for n in (75, 40, 97, 18, 66)]
+    truth = [plain.logits(t) for t in reqs]
+    rough = PlainLlama(tmp_path, bf16=True).logits(reqs[0])
+    yardstick = float(np.mean(np.abs(rough - truth[0]).max(-1) / np.abs(truth[0]).max(-1)))
+    for dtype in ("float32", "bfloat16"):
+        runner = runner_for(tmp_path, dtype, 32)
+        errors = []
+        for build in (traces.decode_tail, traces.portions):
+            steps, expect = build(reqs)
+            traces.compare(TraceReplayer(runner).run_step, steps, expect, truth, TOL[dtype], errors)
+        steps, expect, peak = traces.mixed(reqs, seed=seed)
+        small = runner_for(tmp_path, dtype, peak // 16)
+        small.pools.tensors[0].fill_(1e30)
+        worst = traces.compare(TraceReplayer(small).run_step, steps, expect, truth, TOL[dtype], errors)
+        print(seed, dtype, {k: cfg[k] for k in ("hidden_size", "num_attention_heads", "num_key_value_heads", "head_dim")},
+              f"worst {worst:.2e} mean {np.mean(errors):.2e} (plain bf16 {yardstick:.2e})")
+        if dtype == "float32":
+            assert max(errors) < 2e-5
+        else:
+            assert np.mean(errors) <= 1.5 * yardstick, f"{np.mean(errors):.3e} > 1.5 x {yardstick:.3e}"
