@@ -68,8 +68,9 @@ int psamd_attention_decode(void* stream, const void* qkv, int q_stride, void* ou
                            int hkv, int head_dim, int nsplit, float scale, int window);
 
 // out[r] = argmax (temperature[r] <= 0) or the inverse-CDF draw with uniform[r] in [0, 1).
+int64_t psamd_sample_scratch_floats(int rows);
 int psamd_sample(void* stream, const float* logits, const float* temperature, const float* uniform, int32_t* out,
-                 int rows, int vocab);
+                 float* scratch, int rows, int vocab);
 
 #ifdef __cplusplus
 }

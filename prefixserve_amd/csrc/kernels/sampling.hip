@@ -2,71 +2,46 @@
 // temperature sampling by inverse CDF of softmax(logits / T) in vocabulary order. The
 // uniform number of each row comes from the host, a function of (seed, request, output
 // index) only, so a recomputed request draws the same token.
+//
+// Two kernels, because one workgroup per row reads a 128k-entry row far below what the
+// memory can deliver: the first cuts every row into up to 32 runs of the vocabulary, one
+// workgroup each, and leaves per run (maximum, its first index, sum of exp((x - max) / T));
+// the second, one workgroup per row, combines the runs (that is already the greedy answer),
+// finds the run in which the cumulative sum passes the target and scans only that run.
+
+#include <algorithm>
 
 #include "api.h"
 #include "common.h"
 
 namespace psamd {
 
-constexpr int kSampleThreads = 1024;
+constexpr int kSampleThreads = 256;
+constexpr int kMaxRuns = 32;
 
-// One block per row. Thread t owns the contiguous segment [t * seg, (t + 1) * seg).
-__global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __restrict__ logits,
-                                                                const float* __restrict__ temperature,
-                                                                const float* __restrict__ uniform,
-                                                                int32_t* __restrict__ out, int vocab) {
-  __shared__ float red[kSampleThreads / kWave];
-  __shared__ int32_t red_i[kSampleThreads / kWave];
-  __shared__ float seg_sum[kSampleThreads];
-  __shared__ int32_t chosen;
-  const int tid = threadIdx.x;
-  const float* row = logits + static_cast<int64_t>(blockIdx.x) * vocab;
-  const float temp = temperature[blockIdx.x];
+struct RunStat {
+  float max;
+  int32_t arg;
+  float sum;
+  float pad;
+};
 
-  // ---- max and its first index. The body of the row is read as aligned groups of four,
-  // several loads in flight per thread; a row need not start on a 16-byte boundary.
-  float best = -INFINITY;
-  int32_t best_i = 0x7fffffff;
-  auto take = [&](float v, int32_t i) {
-    if (v > best || (v == best && i < best_i)) {
-      best = v;
-      best_i = i;
-    }
-  };
-  const int head = min(vocab, static_cast<int>((4 - ((reinterpret_cast<uintptr_t>(row) >> 2) & 3)) & 3));
-  const int quads = (vocab - head) / 4;
-  if (tid < head) take(row[tid], tid);
-  const float4* body = reinterpret_cast<const float4*>(row + head);
-  constexpr int kInFlight = 4;
-  for (int q0 = tid; q0 < quads; q0 += kSampleThreads * kInFlight) {
-    float4 v[kInFlight];
-#pragma unroll
-    for (int u = 0; u < kInFlight; ++u) {
-      const int q = q0 + u * kSampleThreads;
-      v[u] = body[min(q, quads - 1)];
-    }
-#pragma unroll
-    for (int u = 0; u < kInFlight; ++u) {
-      const int q = q0 + u * kSampleThreads;
-      if (q < quads) {
-        const int i = head + 4 * q;
-        take(v[u].x, i);
-        take(v[u].y, i + 1);
-        take(v[u].z, i + 2);
-        take(v[u].w, i + 3);
-      }
-    }
+__device__ __forceinline__ void take_max(float v, int32_t i, float& best, int32_t& best_i) {
+  if (v > best || (v == best && i < best_i)) {
+    best = v;
+    best_i = i;
   }
-  for (int i = head + 4 * quads + tid; i < vocab; i += kSampleThreads) take(row[i], i);
+}
+
+// Block-wide (max, first index) by shuffles and one LDS round.
+__device__ __forceinline__ void block_argmax(float& best, int32_t& best_i, float* red, int32_t* red_i) {
 #pragma unroll
   for (int o = kWave / 2; o > 0; o >>= 1) {
     const float ob = __shfl_xor(best, o, kWave);
     const int32_t oi = __shfl_xor(best_i, o, kWave);
-    if (ob > best || (ob == best && oi < best_i)) {
-      best = ob;
-      best_i = oi;
-    }
+    take_max(ob, oi, best, best_i);
   }
+  const int tid = threadIdx.x;
   if ((tid & (kWave - 1)) == 0) {
     red[tid / kWave] = best;
     red_i[tid / kWave] = best_i;
@@ -74,40 +49,130 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __r
   __syncthreads();
   best = red[0];
   best_i = red_i[0];
-  for (int w = 1; w < kSampleThreads / kWave; ++w) {
-    if (red[w] > best || (red[w] == best && red_i[w] < best_i)) {
-      best = red[w];
-      best_i = red_i[w];
+#pragma unroll
+  for (int w = 1; w < kSampleThreads / kWave; ++w) take_max(red[w], red_i[w], best, best_i);
+  __syncthreads();
+}
+
+__device__ __forceinline__ float block_sum(float v, float* red) {
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  const int tid = threadIdx.x;
+  if ((tid & (kWave - 1)) == 0) red[tid / kWave] = v;
+  __syncthreads();
+  float total = 0.f;
+#pragma unroll
+  for (int w = 0; w < kSampleThreads / kWave; ++w) total += red[w];   // every thread the same order
+  __syncthreads();
+  return total;
+}
+
+// Applies f(value, index) to row[lo, hi): aligned groups of four as 16-byte loads, several in
+// flight per thread, the ragged ends one by one. A run need not start on a 16-byte boundary.
+template <typename F>
+__device__ __forceinline__ void for_each_in_run(const float* __restrict__ row, int lo, int hi, F f) {
+  const int tid = threadIdx.x;
+  const int head = min(hi - lo, static_cast<int>((4 - ((reinterpret_cast<uintptr_t>(row + lo) >> 2) & 3)) & 3));
+  const int quads = (hi - lo - head) / 4;
+  if (tid < head) f(row[lo + tid], lo + tid);
+  const float4* body = reinterpret_cast<const float4*>(row + lo + head);
+  constexpr int kInFlight = 4;
+  for (int q0 = tid; q0 < quads; q0 += kSampleThreads * kInFlight) {
+    float4 v[kInFlight];
+#pragma unroll
+    for (int u = 0; u < kInFlight; ++u) v[u] = body[min(q0 + u * kSampleThreads, quads - 1)];
+#pragma unroll
+    for (int u = 0; u < kInFlight; ++u) {
+      const int q = q0 + u * kSampleThreads;
+      if (q < quads) {
+        const int i = lo + head + 4 * q;
+        f(v[u].x, i);
+        f(v[u].y, i + 1);
+        f(v[u].z, i + 2);
+        f(v[u].w, i + 3);
+      }
     }
   }
+  for (int i = lo + head + 4 * quads + tid; i < hi; i += kSampleThreads) f(row[i], i);
+}
+
+// grid (runs, rows): statistics of one run of one row.
+__global__ __launch_bounds__(kSampleThreads) void sample_runs_kernel(const float* __restrict__ logits,
+                                                                    const float* __restrict__ temperature,
+                                                                    RunStat* __restrict__ stats, int vocab, int run_len) {
+  __shared__ float red[kSampleThreads / kWave];
+  __shared__ int32_t red_i[kSampleThreads / kWave];
+  const int run = blockIdx.x, r = blockIdx.y;
+  const float* row = logits + static_cast<int64_t>(r) * vocab;
+  const int lo = run * run_len, hi = min(lo + run_len, vocab);
+  float best = -INFINITY;
+  int32_t best_i = 0x7fffffff;
+  for_each_in_run(row, lo, hi, [&](float v, int32_t i) { take_max(v, i, best, best_i); });
+  block_argmax(best, best_i, red, red_i);
+  const float temp = temperature[r];
+  float total = 0.f;
+  if (temp > 0.f) {
+    const float inv_t = 1.f / temp;
+    float mine = 0.f;
+    // The run was just read: this second pass comes from cache.
+    for_each_in_run(row, lo, hi, [&](float v, int32_t) { mine += expf((v - best) * inv_t); });
+    total = block_sum(mine, red);
+  }
+  if (threadIdx.x == 0) stats[static_cast<int64_t>(r) * gridDim.x + run] = RunStat{best, best_i, total, 0.f};
+}
+
+// grid (rows): combines the runs; for a positive temperature walks the cumulative sum.
+__global__ __launch_bounds__(kSampleThreads) void sample_pick_kernel(const float* __restrict__ logits,
+                                                                    const float* __restrict__ temperature,
+                                                                    const float* __restrict__ uniform,
+                                                                    const RunStat* __restrict__ stats,
+                                                                    int32_t* __restrict__ out, int vocab, int run_len,
+                                                                    int runs) {
+  __shared__ float seg_sum[kSampleThreads];
+  __shared__ int32_t chosen;
+  const int tid = threadIdx.x, r = blockIdx.x;
+  const RunStat* st = stats + static_cast<int64_t>(r) * runs;
+  float best = -INFINITY;
+  int32_t best_i = 0x7fffffff;
+  for (int c = 0; c < runs; ++c) take_max(st[c].max, st[c].arg, best, best_i);   // runs in index order: first wins
+  const float temp = temperature[r];
   if (!(temp > 0.f)) {
-    if (tid == 0) out[blockIdx.x] = best_i;
+    if (tid == 0) out[r] = best_i;
     return;
   }
-
-  // ---- segment sums of exp((x - max) / T)
   const float inv_t = 1.f / temp;
-  const int seg = (vocab + kSampleThreads - 1) / kSampleThreads;
-  const int lo = min(tid * seg, vocab), hi = min(lo + seg, vocab);
-  float mine = 0.f;
-  for (int i = lo; i < hi; ++i) mine += expf((row[i] - best) * inv_t);
-  seg_sum[tid] = mine;
-  if (tid == 0) chosen = vocab - 1;
-  __syncthreads();
-  // Exclusive prefix over the 1024 segment sums, in index order (every thread the same way).
-  float before = 0.f, total = 0.f;
-  for (int t = 0; t < kSampleThreads; ++t) {
-    if (t == tid) before = total;
-    total += seg_sum[t];
+  // Mass of every run relative to the row's maximum, summed in index order.
+  float total = 0.f;
+  for (int c = 0; c < runs; ++c) total += st[c].sum * expf((st[c].max - best) * inv_t);
+  const float target = uniform[r] * total;
+  float before = 0.f;
+  int pick_run = runs - 1;
+  for (int c = 0; c < runs; ++c) {
+    const float mass = st[c].sum * expf((st[c].max - best) * inv_t);
+    if (target < before + mass) {
+      pick_run = c;
+      break;
+    }
+    if (c < runs - 1) before += mass;
   }
-  const float target = uniform[blockIdx.x] * total;
-  // The segment in which the running sum first exceeds the target rescans itself.
-  if (before <= target && target < before + mine) {
-    float run = before;
-    int pick = hi - 1;
-    for (int i = lo; i < hi; ++i) {
-      run += expf((row[i] - best) * inv_t);
-      if (run > target) {
+  // Within the run: thread t owns the contiguous segment [lo + t * seg, lo + (t + 1) * seg).
+  const float* row = logits + static_cast<int64_t>(r) * vocab;
+  const int lo = pick_run * run_len, hi = min(lo + run_len, vocab);
+  const int seg = (hi - lo + kSampleThreads - 1) / kSampleThreads;
+  const int s_lo = min(lo + tid * seg, hi), s_hi = min(s_lo + seg, hi);
+  float mine = 0.f;
+  for (int i = s_lo; i < s_hi; ++i) mine += expf((row[i] - best) * inv_t);
+  seg_sum[tid] = mine;
+  if (tid == 0) chosen = hi - 1;
+  __syncthreads();
+  float start = before;
+  for (int t = 0; t < tid; ++t) start += seg_sum[t];          // exclusive prefix, every thread in index order
+  if (start <= target && target < start + mine) {
+    float run_sum = start;
+    int pick = s_hi - 1;
+    for (int i = s_lo; i < s_hi; ++i) {
+      run_sum += expf((row[i] - best) * inv_t);
+      if (run_sum > target) {
         pick = i;
         break;
       }
@@ -115,18 +180,35 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __r
     atomicMin(&chosen, pick);
   }
   __syncthreads();
-  if (tid == 0) out[blockIdx.x] = chosen;
+  if (tid == 0) out[r] = chosen;
 }
 
 }  // namespace psamd
 
 using namespace psamd;
 
-extern "C" int psamd_sample(void* stream, const float* logits, const float* temperature, const float* uniform,
-                            int32_t* out, int rows, int vocab) {
+extern "C" {
+
+// Floats of scratch ``psamd_sample`` needs for this many rows.
+int64_t psamd_sample_scratch_floats(int rows) { return static_cast<int64_t>(rows) * kMaxRuns * 4; }
+
+int psamd_sample(void* stream, const float* logits, const float* temperature, const float* uniform, int32_t* out,
+                 float* scratch, int rows, int vocab) {
   PSAMD_REQUIRE(rows >= 0 && vocab > 0, "bad sizes");
+  PSAMD_REQUIRE(rows <= 65535, "too many rows for one launch");
   if (rows == 0) return 0;
-  sample_kernel<<<dim3(rows), dim3(kSampleThreads), 0, static_cast<hipStream_t>(stream)>>>(logits, temperature,
-                                                                                           uniform, out, vocab);
-  return check_launch("psamd_sample");
+  PSAMD_REQUIRE(scratch != nullptr, "sampling needs its scratch buffer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // Runs of at least 1024 entries, a multiple of 4 long, at most kMaxRuns of them.
+  int run_len = static_cast<int>(ceil_div(vocab, kMaxRuns));
+  run_len = std::max(1024, (run_len + 3) & ~3);
+  const int runs = static_cast<int>(ceil_div(vocab, run_len));
+  RunStat* stats = reinterpret_cast<RunStat*>(scratch);
+  sample_runs_kernel<<<dim3(runs, rows), dim3(kSampleThreads), 0, s>>>(logits, temperature, stats, vocab, run_len);
+  if (int rc = check_launch("psamd_sample(runs)")) return rc;
+  sample_pick_kernel<<<dim3(rows), dim3(kSampleThreads), 0, s>>>(logits, temperature, uniform, stats, out, vocab, run_len,
+                                                                runs);
+  return check_launch("psamd_sample(pick)");
 }
+
+}  // extern "C"

@@ -53,7 +53,7 @@ _SIGNATURES = {
                                 _i32],
     "psamd_attention_decode": [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32,
                                _i32, _f32, _i32],
-    "psamd_sample": [_vp, _vp, _vp, _vp, _vp, _i32, _i32],
+    "psamd_sample": [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32],
 }
 
 
@@ -73,7 +73,10 @@ class HipOps:
             fn.argtypes = argtypes
             fn.restype = ctypes.c_int
         self.lib.psamd_last_error.restype = ctypes.c_char_p
+        self.lib.psamd_sample_scratch_floats.argtypes = [ctypes.c_int]
+        self.lib.psamd_sample_scratch_floats.restype = ctypes.c_int64
         self.ws = workspace
+        self._sample_scratch: torch.Tensor | None = None
         self.decode_split_kv_len: int | None = None   # fixed key length to size splits by (graph capture)
 
     # ---------------------------------------------------------------- helpers
@@ -283,8 +286,12 @@ class HipOps:
         self._need(temperatures.dtype == torch.float32 and uniforms.dtype == torch.float32 and
                    temperatures.numel() == rows and uniforms.numel() == rows, "sample: one temperature and uniform per row")
         self._need(out.dtype == torch.int32 and out.numel() == rows, "sample: output must be int32 [rows]")
+        need = int(self.lib.psamd_sample_scratch_floats(rows))
+        if self._sample_scratch is None or self._sample_scratch.numel() < need:
+            # Kept apart from the workspace: growing it must not drop captured graphs.
+            self._sample_scratch = torch.empty(max(need, 64 * 128), dtype=torch.float32, device=self.device)
         self._ok(self.lib.psamd_sample(self._stream(), logits.data_ptr(), temperatures.data_ptr(), uniforms.data_ptr(),
-                                       out.data_ptr(), rows, vocab))
+                                       out.data_ptr(), self._sample_scratch.data_ptr(), rows, vocab))
 
     def argmax(self, logits, out) -> None:
         rows = logits.shape[0]

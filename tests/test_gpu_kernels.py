@@ -355,18 +355,26 @@ def test_attention_finds_one_far_key_among_hundreds(ops, act):
 
 # --------------------------------------------------------------------- sampling
 
-def test_sampling_kernel(ops):
+@pytest.mark.parametrize("vocab", [1237, 50257, 3])
+def test_sampling_kernel(ops, vocab):
+    """One run of the vocabulary, many runs of a length that is no multiple of 4 (so rows and
+    runs start at odd alignments), and a vocabulary smaller than anything the kernel tiles by."""
     from plain.llama_plain import sample_plain
 
-    rows, vocab = 6, 1237
+    rows = 6
     logits = rnd(rows, vocab, seed=4, scale=3.0)
-    logits[0, 77] = logits[0, 900] = 50.0                           # a tie: the lowest index wins
+    if vocab == 3:
+        logits[0, 1] = logits[0, 2] = 50.0
+        logits_tie = 1
+    else:
+        logits[0, 77] = logits[0, 900] = 50.0                       # a tie: the lowest index wins
+        logits_tie = 77
     temps = torch.tensor([0.0, 0.0, 0.8, 0.8, 1.5, 0.3], device=DEV)
     us = torch.tensor([0.0, 0.5, 0.1234, 0.9999, 0.5, 0.0], device=DEV)
     out = torch.empty(rows, dtype=torch.int32, device=DEV)
     ops.sample(logits, temps, us, out)
     got = out.tolist()
-    assert got[0] == 77 and got[1] == int(torch.argmax(logits[1]))
+    assert got[0] == logits_tie and got[1] == int(torch.argmax(logits[1]))
     lg = logits.cpu().numpy()
     for r in range(2, rows):
         want = sample_plain(lg[r], float(temps[r]), float(us[r]))
@@ -378,7 +386,7 @@ def test_sampling_kernel(ops):
             assert hi - lo == 1 and abs(c[lo] - target) < 1e-5 * c[-1]
     out2 = torch.empty(rows, dtype=torch.int32, device=DEV)
     ops.argmax(logits, out2)
-    assert out2.tolist() == [77] + torch.argmax(logits[1:], -1).tolist()
+    assert out2.tolist() == [logits_tie] + torch.argmax(logits[1:], -1).tolist()
 
 
 def test_sampling_frequencies(ops):
