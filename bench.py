@@ -186,13 +186,14 @@ def main() -> int:
             out[name] = work * 5 / (time.perf_counter() - t0)
         return out
 
-    peaks = {} if args.no_peaks else measured_peaks()
     prefill = prefill_run(reps=args.prefill_reps)
     main_run = decode_run(args.batch, args.steps, args.warmup)
     points = {}
     if not args.no_points:
         points["decode_b1"] = decode_run(1, max(16, args.steps // 2), max(4, args.warmup // 2))["tok_s"]
         points["decode_b64"] = decode_run(64, max(16, args.steps // 4), max(4, args.warmup // 4))["tok_s"]
+
+    peaks = {} if args.no_peaks else measured_peaks()      # last: a long product changes the clocks of what follows
 
     line = {
         "metric": "decode_tokens_per_second", "value": main_run["tok_s"], "unit": "tok/s", "n_gpus": 1,

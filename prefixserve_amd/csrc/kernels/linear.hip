@@ -453,14 +453,14 @@ int psamd_linear(void* stream, const void* x, int x_dtype, const void* w, int w_
 }
 
 // The K-split that fills the chip for a linear product of M <= 64 tokens whose float32 partial
-// sums a consumer adds up: as many workgroups as there are compute units to spare, each wave
-// keeping at least two k-steps.
+// sums a consumer adds up: as many workgroups as there are compute units to spare.
 int psamd_linear_skinny_ksplit(int M, int n_out, int K) {
   if (M < 1 || M > 64 || n_out < 1 || K < 1) return 1;
   const int mt = static_cast<int>(ceil_div(M, 16));
   const int64_t groups = ceil_div(ceil_div(n_out, 16), skinny_rt(mt, false));
   const int64_t steps = ceil_div(K, 32);
-  const int64_t split = std::min<int64_t>({8, 512 / std::max<int64_t>(groups, 1), steps / (2 * skinny_wv(mt))});
+  // Up to 32 tokens a wave keeps at least two k-steps; above, one is enough (measured).
+  const int64_t split = std::min<int64_t>({8, 512 / std::max<int64_t>(groups, 1), steps / ((mt <= 2 ? 2 : 1) * skinny_wv(mt))});
   return static_cast<int>(std::max<int64_t>(split, 1));
 }
 
