@@ -3,6 +3,8 @@
 // cache pages. Each is templated on the activation type (bfloat16 or float); statistics,
 // rotation and the residual sum are always float.
 
+#include <algorithm>
+
 #include "api.h"
 #include "common.h"
 
@@ -274,6 +276,82 @@ __global__ void rope_kv_append_kernel(A* __restrict__ qkv, int hq, int hkv, int 
   }
 }
 
+// bfloat16 with a head size that is a multiple of 16: one block per 16 tokens of the step.
+// q and k are rotated eight pairs per thread with 16-byte accesses. The values of the 16
+// tokens pass through LDS so that lanes 0..15 write the same (head, dim) of 16 tokens: when
+// the tokens follow each other in one page, as the tokens of a prompt do, that is one 32-byte
+// run of the transposed page instead of 16 scattered 2-byte stores.
+__global__ __launch_bounds__(256) void rope_kv_append_vec_kernel(bf16_t* __restrict__ qkv, int tokens, int hq, int hkv,
+                                                                 int d, const int32_t* __restrict__ positions,
+                                                                 const float2* __restrict__ table,
+                                                                 bf16_t* __restrict__ kv,
+                                                                 const int32_t* __restrict__ write_slot) {
+  extern __shared__ __align__(16) bf16_t v_lds[];        // [16][hkv * d + 8]
+  const int t0 = blockIdx.x * 16;
+  const int nt = min(16, tokens - t0);
+  const int half = d >> 1;
+  const int width = (hq + 2 * hkv) * d;
+  const int64_t page_elems = 2LL * hkv * kPage * d;
+  const int chunks_per_head = half >> 3;                 // groups of 8 pairs
+  const int chunks_per_token = (hq + hkv) * chunks_per_head;
+  // blockIdx.y takes its share of the rotation work and of the value columns.
+  const int rot_total = nt * chunks_per_token;
+  const int rot_lo = static_cast<int>(static_cast<int64_t>(rot_total) * blockIdx.y / gridDim.y);
+  const int rot_hi = static_cast<int>(static_cast<int64_t>(rot_total) * (blockIdx.y + 1) / gridDim.y);
+  for (int idx = rot_lo + threadIdx.x; idx < rot_hi; idx += blockDim.x) {
+    const int j = idx / chunks_per_token, c = idx - j * chunks_per_token;
+    const int h = c / chunks_per_head, i = (c - h * chunks_per_head) << 3;
+    const int64_t t = t0 + j;
+    bf16_t* x = qkv + t * width + h * d + i;
+    uint4 lo = *reinterpret_cast<const uint4*>(x), hi = *reinterpret_cast<const uint4*>(x + half);
+    if (table != nullptr) {
+      const float2* cs = table + static_cast<int64_t>(positions[t]) * half + i;
+      const uint32_t* lw = reinterpret_cast<const uint32_t*>(&lo);
+      const uint32_t* hw = reinterpret_cast<const uint32_t*>(&hi);
+      uint32_t lo_out[4], hi_out[4];
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const float a0 = bf16_to_float(static_cast<bf16_t>(lw[w] & 0xffffu)), a1 = bf16_to_float(static_cast<bf16_t>(lw[w] >> 16));
+        const float b0 = bf16_to_float(static_cast<bf16_t>(hw[w] & 0xffffu)), b1 = bf16_to_float(static_cast<bf16_t>(hw[w] >> 16));
+        const float2 c0 = cs[2 * w], c1 = cs[2 * w + 1];
+        lo_out[w] = static_cast<uint32_t>(float_to_bf16(a0 * c0.x - b0 * c0.y)) |
+                    (static_cast<uint32_t>(float_to_bf16(a1 * c1.x - b1 * c1.y)) << 16);
+        hi_out[w] = static_cast<uint32_t>(float_to_bf16(b0 * c0.x + a0 * c0.y)) |
+                    (static_cast<uint32_t>(float_to_bf16(b1 * c1.x + a1 * c1.y)) << 16);
+      }
+      lo = make_uint4(lo_out[0], lo_out[1], lo_out[2], lo_out[3]);
+      hi = make_uint4(hi_out[0], hi_out[1], hi_out[2], hi_out[3]);
+      *reinterpret_cast<uint4*>(x) = lo;
+      *reinterpret_cast<uint4*>(x + half) = hi;
+    }
+    if (kv != nullptr && h >= hq) {
+      const int slot = write_slot[t];
+      bf16_t* dst = kv + static_cast<int64_t>(slot / kPage) * page_elems +
+                    (static_cast<int64_t>(h - hq) * kPage + slot % kPage) * d + i;
+      *reinterpret_cast<uint4*>(dst) = lo;
+      *reinterpret_cast<uint4*>(dst + half) = hi;
+    }
+  }
+  if (kv == nullptr) return;
+  const int vw = hkv * d;
+  const int c_lo = static_cast<int>(static_cast<int64_t>(vw >> 3) * blockIdx.y / gridDim.y);      // 8-element columns
+  const int c_hi = static_cast<int>(static_cast<int64_t>(vw >> 3) * (blockIdx.y + 1) / gridDim.y);
+  const int nc = c_hi - c_lo, vs = 8 * nc + 8;
+  for (int idx = threadIdx.x; idx < nt * nc; idx += blockDim.x) {
+    const int j = idx / nc, c = idx - j * nc;
+    *reinterpret_cast<uint4*>(v_lds + j * vs + 8 * c) =
+        *reinterpret_cast<const uint4*>(qkv + static_cast<int64_t>(t0 + j) * width + (hq + hkv) * d + 8 * (c_lo + c));
+  }
+  __syncthreads();
+  const int j = threadIdx.x & 15;
+  if (j < nt) {
+    const int slot = write_slot[t0 + j];
+    bf16_t* vpage = kv + static_cast<int64_t>(slot / kPage) * page_elems + static_cast<int64_t>(hkv) * kPage * d + slot % kPage;
+    for (int e = threadIdx.x >> 4; e < 8 * nc; e += blockDim.x >> 4)
+      vpage[static_cast<int64_t>(8 * c_lo + e) * kPage] = v_lds[j * vs + e];
+  }
+}
+
 }  // namespace psamd
 
 using namespace psamd;
@@ -370,7 +448,16 @@ int psamd_rope_kv_append(void* stream, void* qkv, int act_dtype, int64_t tokens,
   if (tokens == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const float2* tab = reinterpret_cast<const float2*>(table);
-  if (act_dtype == kBF16) {
+  if (act_dtype == kBF16 && head_dim % 16 == 0 && static_cast<size_t>(16) * (hkv * head_dim + 8) * sizeof(bf16_t) <= 64 * 1024) {
+    const size_t smem = static_cast<size_t>(16) * (hkv * head_dim + 8) * sizeof(bf16_t);
+    // Enough blocks for every compute unit, each with at least a round of work for its threads.
+    const int64_t groups = ceil_div(tokens, 16);
+    const int64_t rot_rounds = ceil_div(static_cast<int64_t>(16) * (hq + hkv) * (head_dim / 16), 256);
+    const unsigned split = static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>({rot_rounds, 16, ceil_div(1024, groups)})));
+    rope_kv_append_vec_kernel<<<dim3(static_cast<unsigned>(groups), split), dim3(256), smem, s>>>(
+        static_cast<bf16_t*>(qkv), static_cast<int>(tokens), hq, hkv, head_dim, positions, tab, static_cast<bf16_t*>(kv),
+        write_slot);
+  } else if (act_dtype == kBF16) {
     rope_kv_append_kernel<bf16_t><<<dim3(tokens), dim3(256), 0, s>>>(static_cast<bf16_t*>(qkv), hq, hkv, head_dim,
                                                                     positions, tab, static_cast<bf16_t*>(kv), write_slot);
   } else if (act_dtype == kF32) {
