@@ -10,7 +10,6 @@ every 32-bit product and every product with at most 64 rows is a kernel of this 
 
 from __future__ import annotations
 
-import os
 import ctypes
 from typing import Any
 
