@@ -200,14 +200,25 @@ def _random_config(rng):
     return cfg
 
 
-@pytest.mark.parametrize("seed", [0, 1, 2, 3, 4, 5, 6, 7])
+AWKWARD = dict(architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=131, hidden_size=100,
+               intermediate_size=150, num_hidden_layers=2, num_attention_heads=5, num_key_value_heads=1, head_dim=48,
+               rms_norm_eps=1e-5, rope_theta=10000.0, max_position_embeddings=512, tie_word_embeddings=False)
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2, 3, 4, 5, 6, 7, "awkward"])
 def test_random_configurations_in_both_dtypes(seed, tmp_path):
+    """``awkward``: a width and an inner width that are no multiples of 8 (no 16-byte rows: the
+    vectorized kernels and the small-step products must refuse and the general ones run), a
+    head size without a matrix-core kernel, an odd vocabulary."""
     from configs import INIT_STD
     from plain.llama_plain import PlainLlama
     from prefixserve_amd.weights import write_random_model
 
-    rng = np.random.default_rng(1000 + seed)
-    cfg = _random_config(rng)
+    if seed == "awkward":
+        rng, cfg, seed = np.random.default_rng(999), dict(AWKWARD), 99
+    else:
+        rng = np.random.default_rng(1000 + seed)
+        cfg = _random_config(rng)
     write_random_model(tmp_path, cfg, seed=seed, std=INIT_STD)
     plain = PlainLlama(tmp_path)
     reqs = [rng.integers(0, cfg["vocab_size"], n).tolist() for n in (75, 40, 97, 18, 66)]
