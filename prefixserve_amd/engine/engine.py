@@ -50,9 +50,9 @@ class Engine:
         self.sampler = Sampler(self.runner.ops, self.runner.device, max(cfg.max_num_seqs, 1))
         self.capture_logits = False
         self.last_logits: dict[str, torch.Tensor] = {}
-        # req_id -> (preemption count, [(array, filled)] per group): block tables as arrays,
+        # req_id -> (request, preemption count, [(array, filled)] per group): block tables as arrays,
         # extended as the lists grow, so a step does not convert whole lists again.
-        self._tables: dict[str, tuple[int, list[list]]] = {}
+        self._tables: dict[str, tuple[Any, int, list[list]]] = {}
 
     @property
     def num_blocks(self) -> int:
@@ -80,15 +80,17 @@ class Engine:
 
     def _table_arrays(self, req) -> list:
         """The request's block tables as int64 arrays. A request's tables only grow while it
-        runs; after a preemption it gets new ones, which the preemption count tells."""
+        runs; after a preemption it gets new ones, which the preemption count tells. An entry
+        belongs to one request object: an id may come back with another request."""
         entry = self._tables.get(req.req_id)
-        if entry is None or entry[0] != req.num_preemptions or len(entry[1]) != len(req.block_tables):
-            entry = (req.num_preemptions, [[np.empty(64, dtype=np.int64), 0] for _ in req.block_tables])
+        if (entry is None or entry[0] is not req or entry[1] != req.num_preemptions
+                or len(entry[2]) != len(req.block_tables)):
+            entry = (req, req.num_preemptions, [[np.empty(64, dtype=np.int64), 0] for _ in req.block_tables])
             if len(self._tables) > 8 * self.cfg.max_num_seqs:
                 self._tables.clear()           # finished requests leave entries behind
             self._tables[req.req_id] = entry
         out = []
-        for slot, table in zip(entry[1], req.block_tables):
+        for slot, table in zip(entry[2], req.block_tables):
             arr, filled = slot
             n = len(table)
             if n > arr.size:

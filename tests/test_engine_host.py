@@ -180,3 +180,25 @@ def test_several_decode_steps_give_the_same_tokens(temperature, model_dirs, plai
             cut = next((i for i, t in enumerate(full.tokens) if t in sched._stop), None)
             assert o.tokens == (full.tokens if cut is None else full.tokens[:cut + 1])
     assert eng.make_cache().num_free(0) == 32
+
+
+def test_a_request_id_that_comes_back_gets_its_own_block_tables(model_dirs, plain_models):
+    """Runs on one engine and one scheduler reuse the ids req-0, req-1, ...: the second run's
+    requests are longer and get other pages than the first run's, whose prompts stay in the
+    prefix cache. Were anything of the first run's tables to survive in the engine, the second
+    run would write into those cached pages, and the third run, which finds the first prompt
+    in the cache again, would read them."""
+    eng = Engine(EngineConfig(model_path=model_dirs["A"], dtype="float32", device="cpu", max_num_seqs=4,
+                              max_prefill_tokens=64, max_seq_len=256, num_blocks=40, use_graphs=False), ops=EmulatedOps())
+    rng = np.random.default_rng(31)
+    sched = eng.make_scheduler()
+    first = [rng.integers(3, 256, n).tolist() for n in (40, 20)]
+    generate(eng, first, 6, ignore_eos=True, scheduler=sched)
+    second = [rng.integers(3, 256, n).tolist() for n in (90, 70, 33)]
+    outs, _ = generate(eng, second, 9, ignore_eos=True, scheduler=sched)
+    for p, o in zip(second, outs):
+        assert o.tokens == plain_models["A"].greedy(p, 9)[0]
+    again, stats = generate(eng, first, 6, ignore_eos=True, scheduler=sched)
+    assert again[0].cached_tokens >= 32                                     # the first prompt came from the cache
+    for p, o in zip(first, again):
+        assert o.tokens == plain_models["A"].greedy(p, 6)[0]
