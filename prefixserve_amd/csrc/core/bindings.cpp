@@ -143,7 +143,10 @@ py::tuple pack_step(py::array_t<int32_t, py::array::c_style> buffer, const py::s
   its.reserve(n_items);
   keep.arrays.reserve(n_items * (2 + gs.size()));
   // Attribute names as Python strings made once: this runs for every item of every step.
-  static const py::str k_tokens("tokens"), k_start("start"), k_slot("slot"), k_tables("block_tables"), k_want("want");
+  // They are never released: a static object's destructor would run after the interpreter.
+  static const py::handle k_tokens = py::str("tokens").release(), k_start = py::str("start").release(),
+                          k_slot = py::str("slot").release(), k_tables = py::str("block_tables").release(),
+                          k_want = py::str("want").release();
   for (const py::handle& obj : items) {
     PackItem it;
     it.tokens = keep.of(obj.attr(k_tokens), "tokens");
