@@ -142,8 +142,9 @@ def test_rope_kv_append(ops, act, hq, hkv, d):
     assert torch.equal(q2.float(), src.to(act).float())
 
 
-@pytest.mark.parametrize("m", [1, 8, 17, 64])
-@pytest.mark.parametrize("hq,hkv,d,k", [(6, 3, 48, 72), (4, 2, 16, 64), (32, 8, 64, 2048), (3, 1, 32, 96), (2, 2, 128, 200)])
+@pytest.mark.parametrize("m", [1, 8, 17, 40, 64])
+@pytest.mark.parametrize("hq,hkv,d,k", [(6, 3, 48, 72), (4, 2, 16, 64), (32, 8, 64, 2048), (3, 1, 32, 96), (2, 2, 128, 200),
+                                        (32, 8, 128, 264), (50, 1, 128, 72)])   # enough tiles for two per workgroup
 def test_fused_qkv_rope_append_equals_the_separate_kernels(ops, m, hq, hkv, d, k):
     """One kernel for projection + rotation + cache write (small steps) against the product
     followed by rope_kv_append, and against float64."""
