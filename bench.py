@@ -123,13 +123,13 @@ def main() -> int:
             sched.add_request(f"d{batch}-{b}", rng.integers(0, vocab, args.prompt_len), args.context - args.prompt_len - 1,
                               ignore_eos=True)
         # prompts, untimed: one request's prompt per step
-        while any(r.num_computed < len(r.prompt) for r in sched._requests.values()) or sched.stats().num_waiting:
+        while any(r.num_computed < len(r.prompt) for r in sched.requests()):
             bt = sched.schedule_step(args.prompt_len, batch)
             sched.commit(bt, engine.step(bt))
         for _ in range(warmup):
             bt = sched.schedule_step(args.prompt_len, batch)
             sched.commit(bt, engine.step(bt))
-        kv_start = sum(r.num_computed for r in sched._requests.values())
+        kv_start = sum(r.num_computed for r in sched.requests())
         sync()
         t0 = time.perf_counter()
         done = 0
@@ -140,8 +140,8 @@ def main() -> int:
             done += bt.decode_steps
         sync()
         dt = time.perf_counter() - t0
-        kv_end = sum(r.num_computed for r in sched._requests.values())
-        for rid in list(sched._requests):
+        kv_end = sum(r.num_computed for r in sched.requests())
+        for rid in [r.req_id for r in sched.requests()]:
             sched.free_request(rid)
         mean_kv_tokens = 0.5 * (kv_start + kv_end) + 0.5 * batch       # keys read per step, summed over requests
         bytes_per_step = weight_bytes + mean_kv_tokens * kv_bytes_per_token

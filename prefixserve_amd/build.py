@@ -30,7 +30,7 @@ PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
 GPU_ARCH = "gfx950"
 
-CORE_SOURCES = ["core/block_pool.cpp", "core/prefix_tree.cpp", "core/step_pack.cpp", "core/bindings.cpp"]
+CORE_SOURCES = ["core/page_pool.cpp", "core/prefix_tree.cpp", "core/step_pack.cpp", "core/bindings.cpp"]
 KERNEL_LIB = "libpsamd_kernels.so"
 
 HIPCC_FLAGS = [

@@ -1,149 +1,173 @@
-"""Typed Llama configuration read from the architecture's own ``config.json`` keys.
+"""The Llama architecture's configuration, typed, from its own ``config.json`` keys.
 
-Key names, defaults and refusals follow prefixserve/model/config.py:54-120 of the
-reference: both the transformers-4 layout (top-level ``rope_theta`` + ``rope_scaling``)
-and the transformers-5 layout (one ``rope_parameters`` dict); stop ids from
-``generation_config.json`` first; anything not understood raises instead of being
-ignored, because a silently dropped ``rope_scaling`` loads fine and writes garbage at
-long positions.
+Which keys are read, their defaults and what is refused are those of the reference's
+parser (prefixserve/model/config.py:54-120): the rope base and scaling may stand at the
+top level (``rope_theta``, ``rope_scaling``) or together in one ``rope_parameters`` dict
+(the newer layout of the same checkpoints); stop ids come from ``generation_config.json``
+when it has them. A key that changes the arithmetic and is not understood raises: a
+scaling rule dropped without a word would load and then write nonsense at long positions.
 """
 
 from __future__ import annotations
 
 import json
-from dataclasses import dataclass
+from dataclasses import dataclass, fields
 from pathlib import Path
 from typing import Any, Mapping
 
+ARCHITECTURE = "LlamaForCausalLM"
+MODEL_TYPE = "llama"
+DEFAULT_ROPE_THETA = 10000.0
+
+# dataclass field -> config.json key, for the sizes that must be there and are plain integers
+_INT_KEYS = {
+    "vocab_size": "vocab_size",
+    "hidden_size": "hidden_size",
+    "intermediate_size": "intermediate_size",
+    "num_layers": "num_hidden_layers",
+    "num_heads": "num_attention_heads",
+    "max_position_embeddings": "max_position_embeddings",
+}
+_SCALING_KEYS = ("factor", "low_freq_factor", "high_freq_factor", "original_max_position_embeddings")
+
 
 class UnsupportedModelError(ValueError):
-    """The folder describes a model this engine cannot run."""
+    """config.json describes something this engine does not run."""
 
 
 @dataclass(frozen=True)
 class Llama3RopeScaling:
-    """The "llama3" three-band frequency scaling (prefixserve/model/config.py:20-27)."""
+    """The "llama3" rule: long waves are slowed by ``factor``, short ones kept, those between
+    blended; the bands are set by the two frequency factors and the original context length."""
 
     factor: float
     low_freq_factor: float
     high_freq_factor: float
     original_max_position_embeddings: int
 
+    @classmethod
+    def from_json(cls, entry: Mapping[str, Any] | None) -> "Llama3RopeScaling | None":
+        """None for no entry and for the kind "default"; any other kind but "llama3" is refused."""
+        if not entry:
+            return None
+        kind = entry["rope_type"] if "rope_type" in entry else entry.get("type")
+        if kind is None or kind == "default":
+            return None
+        if kind != "llama3":
+            raise UnsupportedModelError(f"rope scaling of kind {kind!r}: only 'llama3' is implemented")
+        values = [entry[k] for k in _SCALING_KEYS]          # KeyError names what is missing
+        return cls(float(values[0]), float(values[1]), float(values[2]), int(values[3]))
+
+    def to_json(self) -> dict[str, Any]:
+        return {"rope_type": "llama3", **{k: getattr(self, k) for k in _SCALING_KEYS}}
+
 
 @dataclass(frozen=True)
 class LlamaConfig:
+    # sizes
     vocab_size: int
     hidden_size: int
     intermediate_size: int
     num_layers: int
+    max_position_embeddings: int
+    # attention
     num_heads: int
     num_kv_heads: int
     head_dim: int
+    # constants
     rms_norm_eps: float
     rope_theta: float
     rope_scaling: Llama3RopeScaling | None
-    max_position_embeddings: int
     tie_word_embeddings: bool
     stop_token_ids: frozenset[int]
 
     @property
     def q_size(self) -> int:
-        return self.num_heads * self.head_dim
+        """Columns of the query projection."""
+        return self.head_dim * self.num_heads
 
     @property
     def kv_size(self) -> int:
-        return self.num_kv_heads * self.head_dim
+        """Columns of the key projection, and of the value projection."""
+        return self.head_dim * self.num_kv_heads
+
+    # ------------------------------------------------------------------ reading
 
     @classmethod
-    def from_dir(cls, path: str | Path) -> "LlamaConfig":
-        path = Path(path)
-        raw = json.loads((path / "config.json").read_text())
-        gen_path = path / "generation_config.json"
-        gen = json.loads(gen_path.read_text()) if gen_path.exists() else {}
-        return cls.from_dicts(raw, gen)
+    def from_dir(cls, model_dir: str | Path) -> "LlamaConfig":
+        folder = Path(model_dir)
+        generation = folder / "generation_config.json"
+        return cls.from_dicts(json.loads((folder / "config.json").read_text()),
+                              json.loads(generation.read_text()) if generation.exists() else None)
 
     @classmethod
     def from_dicts(cls, raw: Mapping[str, Any], gen: Mapping[str, Any] | None = None) -> "LlamaConfig":
-        if raw.get("model_type") != "llama":
-            raise UnsupportedModelError(f"model_type {raw.get('model_type')!r} is not 'llama'")
-        heads = int(raw["num_attention_heads"])
-        kv_heads = int(raw.get("num_key_value_heads", heads))
-        if kv_heads < 1 or heads % kv_heads:
-            raise UnsupportedModelError(f"{heads} query heads not divisible by {kv_heads} KV heads")
-        hidden = int(raw["hidden_size"])
-        head_dim = int(raw.get("head_dim") or hidden // heads)
-        rope_params = raw.get("rope_parameters") or {}
-        rope = raw.get("rope_parameters") or raw.get("rope_scaling")
-        theta_raw = rope_params.get("rope_theta", raw.get("rope_theta"))
-        theta = float(theta_raw) if theta_raw is not None else 10000.0
-        if raw.get("attention_bias") or raw.get("mlp_bias"):
-            raise UnsupportedModelError("biases in attention/MLP are not supported")
-        eos = (gen or {}).get("eos_token_id", raw.get("eos_token_id"))
-        stop = frozenset(int(t) for t in (eos if isinstance(eos, list) else [eos]) if t is not None)
+        """``raw`` = config.json, ``gen`` = generation_config.json or None."""
+        _refuse_what_is_not_llama(raw)
+        sizes = {name: int(raw[key]) for name, key in _INT_KEYS.items()}
+        heads = sizes["num_heads"]
+        kv_heads = int(raw["num_key_value_heads"]) if "num_key_value_heads" in raw else heads
+        if kv_heads < 1 or heads % kv_heads != 0:
+            raise UnsupportedModelError(f"{heads} attention heads cannot share {kv_heads} key/value heads")
+        theta, scaling = _rope_of(raw)
         return cls(
-            vocab_size=int(raw["vocab_size"]),
-            hidden_size=hidden,
-            intermediate_size=int(raw["intermediate_size"]),
-            num_layers=int(raw["num_hidden_layers"]),
-            num_heads=heads,
+            **sizes,
             num_kv_heads=kv_heads,
-            head_dim=head_dim,
+            # 3.2-1B states its head size; older checkpoints leave it to hidden / heads.
+            head_dim=int(raw.get("head_dim") or sizes["hidden_size"] // heads),
             rms_norm_eps=float(raw["rms_norm_eps"]),
             rope_theta=theta,
-            rope_scaling=_parse_rope_scaling(rope),
-            max_position_embeddings=int(raw["max_position_embeddings"]),
+            rope_scaling=scaling,
             tie_word_embeddings=bool(raw.get("tie_word_embeddings", False)),
-            stop_token_ids=stop,
+            stop_token_ids=_stop_ids(raw, gen),
         )
 
+    # ------------------------------------------------------------------ writing
+
     def to_config_json(self) -> dict[str, Any]:
-        """The ``config.json`` this configuration is read back from (used by the
-        random-weights mode to write a model folder)."""
-        raw: dict[str, Any] = {
-            "architectures": ["LlamaForCausalLM"],
-            "model_type": "llama",
-            "vocab_size": self.vocab_size,
-            "hidden_size": self.hidden_size,
-            "intermediate_size": self.intermediate_size,
-            "num_hidden_layers": self.num_layers,
-            "num_attention_heads": self.num_heads,
-            "num_key_value_heads": self.num_kv_heads,
-            "head_dim": self.head_dim,
-            "rms_norm_eps": self.rms_norm_eps,
-            "rope_theta": self.rope_theta,
-            "rope_scaling": None,
-            "max_position_embeddings": self.max_position_embeddings,
-            "tie_word_embeddings": self.tie_word_embeddings,
-            "hidden_act": "silu",
-            "attention_bias": False,
-            "mlp_bias": False,
-        }
-        if self.rope_scaling is not None:
-            rs = self.rope_scaling
-            raw["rope_scaling"] = {
-                "rope_type": "llama3",
-                "factor": rs.factor,
-                "low_freq_factor": rs.low_freq_factor,
-                "high_freq_factor": rs.high_freq_factor,
-                "original_max_position_embeddings": rs.original_max_position_embeddings,
-            }
-        if self.stop_token_ids:
-            ids = sorted(self.stop_token_ids)
-            raw["eos_token_id"] = ids[0] if len(ids) == 1 else ids
-        return raw
+        """A config.json that reads back as this configuration: what the random-weights mode
+        writes next to its model.safetensors."""
+        out: dict[str, Any] = {"architectures": [ARCHITECTURE], "model_type": MODEL_TYPE}
+        out.update({key: getattr(self, name) for name, key in _INT_KEYS.items()})
+        out.update(num_key_value_heads=self.num_kv_heads, head_dim=self.head_dim, rms_norm_eps=self.rms_norm_eps,
+                   rope_theta=self.rope_theta, tie_word_embeddings=self.tie_word_embeddings, hidden_act="silu",
+                   attention_bias=False, mlp_bias=False,
+                   rope_scaling=self.rope_scaling.to_json() if self.rope_scaling is not None else None)
+        stops = sorted(self.stop_token_ids)
+        if stops:
+            out["eos_token_id"] = stops if len(stops) > 1 else stops[0]
+        return out
 
 
-def _parse_rope_scaling(rs: Mapping[str, Any] | None) -> Llama3RopeScaling | None:
-    if rs is None:
-        return None
-    kind = rs.get("rope_type", rs.get("type"))
-    if kind in (None, "default"):
-        return None
-    if kind != "llama3":
-        raise UnsupportedModelError(f"rope_scaling type {kind!r} is not supported")
-    return Llama3RopeScaling(
-        factor=float(rs["factor"]),
-        low_freq_factor=float(rs["low_freq_factor"]),
-        high_freq_factor=float(rs["high_freq_factor"]),
-        original_max_position_embeddings=int(rs["original_max_position_embeddings"]),
-    )
+assert {f.name for f in fields(LlamaConfig)} >= set(_INT_KEYS)
+
+
+def _refuse_what_is_not_llama(raw: Mapping[str, Any]) -> None:
+    kind = raw.get("model_type")
+    if kind != MODEL_TYPE:
+        raise UnsupportedModelError(f"model_type is {kind!r}, expected {MODEL_TYPE!r}")
+    for key in ("attention_bias", "mlp_bias"):
+        if raw.get(key):
+            raise UnsupportedModelError(f"{key} is set: projections with a bias are not implemented")
+
+
+def _rope_of(raw: Mapping[str, Any]) -> tuple[float, Llama3RopeScaling | None]:
+    """(theta, scaling) from ``rope_parameters`` if the file has that dict, else from the
+    top-level ``rope_theta`` and ``rope_scaling``."""
+    joint = raw.get("rope_parameters")
+    if joint:
+        theta = joint.get("rope_theta", raw.get("rope_theta"))
+        entry = joint
+    else:
+        theta = raw.get("rope_theta")
+        entry = raw.get("rope_scaling")
+    return (DEFAULT_ROPE_THETA if theta is None else float(theta)), Llama3RopeScaling.from_json(entry)
+
+
+def _stop_ids(raw: Mapping[str, Any], gen: Mapping[str, Any] | None) -> frozenset[int]:
+    """eos_token_id, an integer or a list of them, from the generation config first."""
+    found = gen.get("eos_token_id") if gen and "eos_token_id" in gen else raw.get("eos_token_id")
+    if found is None:
+        return frozenset()
+    many = found if isinstance(found, (list, tuple)) else [found]
+    return frozenset(int(t) for t in many if t is not None)

@@ -1,21 +1,21 @@
-// Python module prefixserve_amd._core: the host-side cache bookkeeping.
+// The Python module prefixserve_amd._core: the host side of the cache (page pool, prefix
+// index, state slots) and the packing of a step's integers.
 //
-// The Python names and meanings are the reference's (prefixserve/_core.pyi:9-36,
-// csrc/bindings.cpp:96-171): BLOCK_SIZE, CoreError, BlockManager, RadixTree; StateSlots is
-// new. Inputs are borrowed for the length of a call; outputs are fresh Python lists, never
-// views of memory the next call reuses.
+// Python sees the reference's names with the reference's meanings (prefixserve/_core.pyi:9-36,
+// csrc/bindings.cpp:96-171): BLOCK_SIZE, CoreError, BlockManager, RadixTree. StateSlots and
+// pack_step are additions. Arguments are only read during the call; results are new Python
+// lists, never views of memory that a later call writes again.
 
 #include <pybind11/numpy.h>
 #include <pybind11/pybind11.h>
 #include <pybind11/stl.h>
 
 #include <deque>
-#include <memory>
 #include <stdexcept>
 #include <string>
 #include <vector>
 
-#include "block_pool.hpp"
+#include "page_pool.hpp"
 #include "prefix_tree.hpp"
 #include "step_pack.hpp"
 
@@ -24,63 +24,108 @@ using namespace psamd;
 
 namespace {
 
+// Misuse of the counts (a double free, an id out of range, ...) as a Python exception.
 struct CoreError : std::runtime_error {
   using std::runtime_error::runtime_error;
 };
 
-void expect_ok(Status s, const std::string& what) {
-  if (s != Status::kOk) throw CoreError(what + ": " + status_name(s));
+[[noreturn]] void raise_fault(const std::string& where, Fault f) { throw CoreError(where + ": " + describe(f)); }
+
+void require(const std::string& where, Fault f) {
+  if (f != Fault::kNone) raise_fault(where, f);
 }
 
-using Ints = py::array_t<int32_t, py::array::c_style | py::array::forcecast>;
+using IntArray = py::array_t<int32_t, py::array::c_style | py::array::forcecast>;
 
-const Ints& one_dim(const Ints& a, const char* name) {
-  if (a.ndim() != 1) throw py::value_error(std::string(name) + " must be 1-D");
-  return a;
+void require_flat(const IntArray& a, const char* what) {
+  if (a.ndim() != 1) throw py::value_error(std::string(what) + " must be one-dimensional");
 }
 
-py::list as_list(const BlockId* v, size_t n) {
-  py::list out(n);
-  for (size_t i = 0; i < n; ++i) out[i] = py::int_(v[i]);
-  return out;
+py::list python_list(const std::vector<BlockId>& ids, size_t count) {
+  py::list result(count);
+  for (size_t i = 0; i < count; ++i) result[i] = ids[i];
+  return result;
 }
 
-// The tree plus a result buffer sized once, so a match allocates nothing on this side.
-class TreeHandle {
- public:
-  TreeHandle(BlockPool& pool, py::object seed)
-      : tree_(pool, seed.is_none() ? PrefixTree::random_seed() : seed.cast<uint64_t>()),
-        found_(static_cast<size_t>(pool.num_blocks())) {}
+// ---- BlockManager
 
-  py::tuple match_prefix(const Ints& tokens) {
-    one_dim(tokens, "tokens");
-    // At most one page per pool page can match, whatever the prompt's length.
-    const int64_t n = std::min<int64_t>(tokens.size(), static_cast<int64_t>(found_.size()) * kBlockSize);
-    const int64_t matched = tree_.match_prefix(tokens.data(), n, found_.data());
-    return py::make_tuple(matched, as_list(found_.data(), static_cast<size_t>(matched / kBlockSize)));
+py::object pool_allocate(PagePool& pool) {
+  const BlockId id = pool.take();
+  if (id == kNoBlock) return py::none();
+  return py::int_(id);
+}
+
+py::object pool_allocate_many(PagePool& pool, int32_t n) {
+  if (n < 0) throw py::value_error("cannot allocate a negative number of blocks");
+  std::vector<BlockId> ids(static_cast<size_t>(n));
+  if (!pool.take_many(n, ids.data())) return py::none();       // fewer than n free: nothing was taken
+  return python_list(ids, ids.size());
+}
+
+void pool_decref_many(PagePool& pool, const IntArray& ids) {
+  require_flat(ids, "block_ids");
+  for (py::ssize_t i = 0; i < ids.size(); ++i) {
+    const Fault f = pool.drop(ids.at(i));
+    if (f != Fault::kNone)
+      raise_fault("decref_many, block " + std::to_string(ids.at(i)) + " at index " + std::to_string(i), f);
   }
-  int32_t insert(const Ints& tokens, const Ints& blocks) {
-    one_dim(tokens, "tokens");
-    one_dim(blocks, "block_ids");
+}
+
+int32_t pool_ref_count(const PagePool& pool, BlockId id) {
+  const int32_t owners = pool.owners(id);
+  if (owners < 0) raise_fault("ref_count", Fault::kBadPage);
+  return owners;
+}
+
+void pool_check(const PagePool& pool) {
+  std::string why;
+  if (!pool.check_invariants(&why)) throw CoreError("the block manager is inconsistent: " + why);
+}
+
+// ---- RadixTree: the index and a result buffer made once, so that a lookup allocates nothing
+// but its Python result.
+
+class Index {
+ public:
+  Index(PagePool& pool, const py::object& seed)
+      : tree_(pool, seed.is_none() ? PrefixIndex::random_seed() : seed.cast<uint64_t>()),
+        scratch_(static_cast<size_t>(pool.num_blocks())) {}
+
+  py::tuple lookup(const IntArray& tokens) {
+    require_flat(tokens, "tokens");
+    // However long the prompt, no more pages can match than the pool has.
+    const int64_t usable = std::min<int64_t>(tokens.size(), static_cast<int64_t>(scratch_.size()) * kBlockSize);
+    const int64_t matched = tree_.lookup(tokens.data(), usable, scratch_.data());
+    return py::make_tuple(matched, python_list(scratch_, static_cast<size_t>(matched / kBlockSize)));
+  }
+
+  int32_t insert(const IntArray& tokens, const IntArray& pages) {
+    require_flat(tokens, "tokens");
+    require_flat(pages, "block_ids");
     int32_t added = 0;
-    expect_ok(tree_.insert(tokens.data(), tokens.size(), blocks.data(), blocks.size(), &added), "insert");
+    require("insert", tree_.hold(tokens.data(), tokens.size(), pages.data(), pages.size(), &added));
     return added;
   }
-  int32_t evict(int32_t n) {
-    if (n < 0) throw py::value_error("num_blocks must be >= 0");
-    return tree_.evict(n);
+
+  int32_t evict(int32_t count) {
+    if (count < 0) throw py::value_error("cannot evict a negative number of blocks");
+    return tree_.release_oldest(count);
   }
-  int32_t cached() const { return tree_.num_cached_blocks(); }
-  bool is_cached(BlockId id) const { return tree_.is_cached(id); }
+
+  bool is_cached(BlockId id) const { return tree_.holds(id); }
+  int32_t num_cached_blocks() const { return tree_.size(); }
+
   void check() const {
     std::string why;
-    if (!tree_.check_invariants(&why)) throw CoreError("RadixTree invariant broken: " + why);
+    if (!tree_.consistent(&why)) throw CoreError("the prefix tree is inconsistent: " + why);
   }
 
  private:
-  PrefixTree tree_;
-  std::vector<BlockId> found_;
+  PrefixIndex tree_;
+  std::vector<BlockId> scratch_;
 };
+
+// ---- pack_step
 
 using Longs = py::array_t<int64_t, py::array::c_style | py::array::forcecast>;
 
@@ -178,84 +223,49 @@ py::tuple pack_step(py::array_t<int32_t, py::array::c_style> buffer, const py::s
 }  // namespace
 
 PYBIND11_MODULE(_core, m) {
-  m.doc() = "Paged KV block manager, block-granular radix prefix cache and per-request state slots.";
+  m.doc() = "Host side of the paged KV cache: page pool, prefix index, state slots, step packing.";
   m.attr("BLOCK_SIZE") = kBlockSize;
   py::register_exception<CoreError>(m, "CoreError", PyExc_RuntimeError);
 
-  py::class_<BlockPool>(m, "BlockManager")
-      .def(py::init<int32_t>(), py::arg("num_blocks"))
-      .def("allocate",
-           [](BlockPool& p) -> py::object {
-             const BlockId id = p.allocate();
-             return id == kNoBlock ? py::object(py::none()) : py::object(py::int_(id));
-           },
-           "One block with ref_count 1, or None when the pool is empty.")
-      .def("allocate_many",
-           [](BlockPool& p, int32_t n) -> py::object {
-             if (n < 0) throw py::value_error("n must be >= 0");
-             if (p.num_free() < n) return py::none();  // all-or-nothing
-             std::vector<BlockId> ids(static_cast<size_t>(n));
-             (void)p.allocate_many(n, ids.data());
-             return as_list(ids.data(), ids.size());
-           },
-           py::arg("n"), "n blocks, or None (nothing allocated) if fewer than n are free.")
-      .def("incref", [](BlockPool& p, BlockId id) { expect_ok(p.incref(id), "incref"); }, py::arg("block_id"))
-      .def("decref", [](BlockPool& p, BlockId id) { expect_ok(p.decref(id), "decref"); }, py::arg("block_id"))
-      .def("decref_many",
-           [](BlockPool& p, const Ints& ids) {
-             one_dim(ids, "block_ids");
-             const int32_t* v = ids.data();
-             for (py::ssize_t i = 0; i < ids.size(); ++i) {
-               const Status s = p.decref(v[i]);
-               if (s != Status::kOk) {
-                 throw CoreError("decref_many: block " + std::to_string(v[i]) + " at index " + std::to_string(i) +
-                                 ": " + status_name(s));
-               }
-             }
-           },
-           py::arg("block_ids"))
-      .def("ref_count",
-           [](const BlockPool& p, BlockId id) {
-             if (!p.valid(id)) expect_ok(Status::kInvalidBlockId, "ref_count");
-             return p.ref_count(id);
-           },
-           py::arg("block_id"))
-      .def_property_readonly("num_free", &BlockPool::num_free)
-      .def_property_readonly("num_blocks", &BlockPool::num_blocks)
-      .def("check_invariants", [](const BlockPool& p) {
-        std::string why;
-        if (!p.check_invariants(&why)) throw CoreError("BlockManager invariant broken: " + why);
-      });
+  py::class_<PagePool> pool(m, "BlockManager");
+  pool.def(py::init<int32_t>(), py::arg("num_blocks"));
+  pool.def("allocate", &pool_allocate, "A block with one reference, or None if none is free.");
+  pool.def("allocate_many", &pool_allocate_many, py::arg("n"), "n blocks, or None and nothing taken.");
+  pool.def("incref", [](PagePool& p, BlockId id) { require("incref", p.share(id)); }, py::arg("block_id"));
+  pool.def("decref", [](PagePool& p, BlockId id) { require("decref", p.drop(id)); }, py::arg("block_id"));
+  pool.def("decref_many", &pool_decref_many, py::arg("block_ids"));
+  pool.def("ref_count", &pool_ref_count, py::arg("block_id"));
+  pool.def_property_readonly("num_free", &PagePool::num_free);
+  pool.def_property_readonly("num_blocks", &PagePool::num_blocks);
+  pool.def("check_invariants", &pool_check);
 
-  py::class_<TreeHandle>(m, "RadixTree")
-      // keep_alive: the tree points into the pool, so it keeps the pool's Python object alive.
-      .def(py::init<BlockPool&, py::object>(), py::arg("block_manager"), py::arg("hash_seed") = py::none(),
-           py::keep_alive<1, 2>())
-      .def("match_prefix", &TreeHandle::match_prefix, py::arg("tokens"),
-           "(matched_tokens, block_ids). Takes 1 ref per block for the caller.")
-      .def("insert", &TreeHandle::insert, py::arg("tokens"), py::arg("block_ids"),
-           "Caches full blocks. Returns how many new blocks the tree now holds.")
-      .def("evict", &TreeHandle::evict, py::arg("num_blocks"),
-           "Frees up to num_blocks unused blocks, LRU first. Returns how many were freed.")
-      .def("is_cached", &TreeHandle::is_cached, py::arg("block_id"))
-      .def_property_readonly("num_cached_blocks", &TreeHandle::cached)
-      .def("check_invariants", &TreeHandle::check);
+  py::class_<Index> index(m, "RadixTree");
+  // The index points into the pool: it keeps the pool's Python object alive.
+  index.def(py::init<PagePool&, const py::object&>(), py::arg("block_manager"), py::arg("hash_seed") = py::none(),
+            py::keep_alive<1, 2>());
+  index.def("match_prefix", &Index::lookup, py::arg("tokens"),
+            "(matched tokens, block ids); the caller holds one reference on each block.");
+  index.def("insert", &Index::insert, py::arg("tokens"), py::arg("block_ids"),
+            "Holds the full blocks of tokens; returns how many it took.");
+  index.def("evict", &Index::evict, py::arg("num_blocks"), "Frees up to num_blocks blocks nobody uses, oldest first.");
+  index.def("is_cached", &Index::is_cached, py::arg("block_id"));
+  index.def_property_readonly("num_cached_blocks", &Index::num_cached_blocks);
+  index.def("check_invariants", &Index::check);
+
+  py::class_<StateSlots> slots(m, "StateSlots");
+  slots.def(py::init<int32_t, int64_t>(), py::arg("num_slots"), py::arg("bytes_per_slot") = 0);
+  slots.def("acquire", [](StateSlots& s) -> py::object {
+    const int32_t id = s.acquire();
+    if (id < 0) return py::none();
+    return py::int_(id);
+  }, "A free slot, or None if all are taken.");
+  slots.def("release", [](StateSlots& s, int32_t slot) { require("release", s.release(slot)); }, py::arg("slot"));
+  slots.def("in_use", &StateSlots::in_use, py::arg("slot"));
+  slots.def_property_readonly("num_slots", &StateSlots::num_slots);
+  slots.def_property_readonly("num_free", &StateSlots::num_free);
+  slots.def_property_readonly("bytes_per_slot", &StateSlots::bytes_per_slot);
 
   m.def("pack_step", &pack_step, py::arg("buffer"), py::arg("items"), py::arg("groups"), py::arg("vocab_size"),
         py::arg("max_position"), py::arg("num_slots"), py::arg("prefill_tile"), py::arg("static_pages") = py::none(),
         "Checks a step's items and lays their integer arrays out in one buffer.");
-
-  py::class_<StateSlots>(m, "StateSlots")
-      .def(py::init<int32_t, int64_t>(), py::arg("num_slots"), py::arg("bytes_per_slot") = 0)
-      .def("acquire",
-           [](StateSlots& s) -> py::object {
-             const int32_t id = s.acquire();
-             return id < 0 ? py::object(py::none()) : py::object(py::int_(id));
-           },
-           "A free slot id, or None when every slot is taken.")
-      .def("release", [](StateSlots& s, int32_t id) { expect_ok(s.release(id), "release"); }, py::arg("slot"))
-      .def("in_use", &StateSlots::in_use, py::arg("slot"))
-      .def_property_readonly("num_slots", &StateSlots::num_slots)
-      .def_property_readonly("num_free", &StateSlots::num_free)
-      .def_property_readonly("bytes_per_slot", &StateSlots::bytes_per_slot);
 }

@@ -7,327 +7,218 @@ namespace psamd {
 
 namespace {
 
-inline uint64_t finalize64(uint64_t z) noexcept {
-  z += 0x9E3779B97F4A7C15ull;
-  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
-  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
-  return z ^ (z >> 31);
+size_t buckets_for(int32_t entries) {
+  size_t n = 16;
+  while (n < 2 * static_cast<size_t>(entries)) n <<= 1;
+  return n;
 }
-
-inline size_t sz(int64_t v) noexcept { return static_cast<size_t>(v); }
 
 }  // namespace
 
-uint64_t PrefixTree::random_seed() {
-  std::random_device rd;
-  return (static_cast<uint64_t>(rd()) << 32) ^ rd();
+PrefixIndex::PrefixIndex(PagePool& pool, uint64_t seed) : pool_(pool), seed_(seed) {
+  const int32_t pages = pool.num_blocks();
+  entry_.resize(static_cast<size_t>(pages) + 1);
+  text_.assign((static_cast<size_t>(pages) + 1) * kBlockSize, 0);
+  bucket_.assign(buckets_for(pages + 1), kNil);
+  shared_.assign(static_cast<size_t>(pages), 0);
+  seen_in_call_.assign(static_cast<size_t>(pages), 0);
+  unused_.reserve(static_cast<size_t>(pages));
+  for (Ref e = pages; e >= 1; --e) unused_.push_back(e);      // entry 1 is used first
 }
 
-PrefixTree::PrefixTree(BlockPool& pool, uint64_t hash_seed)
-    : pool_(pool), capacity_(pool.num_blocks() + 1) {
-  uint64_t s = hash_seed;
-  for (int32_t i = 0; i < kBlockSize; ++i) {
-    s = finalize64(s);
-    key_[i] = static_cast<uint32_t>(s >> 32);
+PrefixIndex::~PrefixIndex() {
+  for (Ref e = oldest_; e != kNil; e = entry_[static_cast<size_t>(e)].younger)
+    pool_.drop(entry_[static_cast<size_t>(e)].page);
+}
+
+uint64_t PrefixIndex::random_seed() {
+  std::random_device device;
+  return (static_cast<uint64_t>(device()) << 32) ^ device();
+}
+
+// Two tokens at a time through a multiply-and-fold; the prefix enters through the start value.
+// Quality only matters for speed: a hit is confirmed by comparing the tokens.
+uint64_t PrefixIndex::hash_of(Ref parent, const int32_t* t) const noexcept {
+  uint64_t h = seed_ + 0x9E3779B97F4A7C15ull * (static_cast<uint64_t>(parent) + 1);
+  for (int i = 0; i < kBlockSize; i += 2) {
+    const uint64_t two = static_cast<uint32_t>(t[i]) | (static_cast<uint64_t>(static_cast<uint32_t>(t[i + 1])) << 32);
+    h = (h ^ two) * 0xD6E8FEB86659FD93ull;
+    h ^= h >> 32;
   }
-  const size_t cap = sz(capacity_);
-  parent_.assign(cap, kNone);
-  block_.assign(cap, kNoBlock);
-  children_.assign(cap, 0);
-  heap_pos_.assign(cap, -1);
-  used_at_.assign(cap, 0);
-  page_tokens_.assign(cap * kBlockSize, 0);
-  spare_.reserve(cap);
-  for (Node n = capacity_ - 1; n >= 1; --n) spare_.push_back(n);
-
-  size_t slots = 16;
-  while (slots < 2 * cap) slots <<= 1;
-  slot_hash_.assign(slots, 0);
-  slot_node_.assign(slots, kNone);
-  mask_ = slots - 1;
-
-  heap_.assign(cap, kNone);
-  held_back_.reserve(cap);
-  owned_.assign(sz(pool.num_blocks()), 0);
+  return h;
 }
 
-PrefixTree::~PrefixTree() {
-  for (Node n = 1; n < capacity_; ++n) {
-    if (block_[sz(n)] != kNoBlock) (void)pool_.decref(block_[sz(n)]);
+PrefixIndex::Ref PrefixIndex::find(Ref parent, const int32_t* t, uint64_t h) const noexcept {
+  for (Ref e = bucket_[h & (bucket_.size() - 1)]; e != kNil; e = entry_[static_cast<size_t>(e)].same_bucket) {
+    const Entry& x = entry_[static_cast<size_t>(e)];
+    if (x.hash == h && x.parent == parent && std::memcmp(text(e), t, sizeof(int32_t) * kBlockSize) == 0) return e;
+  }
+  return kNil;
+}
+
+void PrefixIndex::unlink_recency(Ref e) noexcept {
+  Entry& x = entry_[static_cast<size_t>(e)];
+  if (x.older != kNil) entry_[static_cast<size_t>(x.older)].younger = x.younger; else oldest_ = x.younger;
+  if (x.younger != kNil) entry_[static_cast<size_t>(x.younger)].older = x.older; else youngest_ = x.older;
+  x.older = x.younger = kNil;
+}
+
+void PrefixIndex::make_youngest(Ref e) noexcept {
+  Entry& x = entry_[static_cast<size_t>(e)];
+  x.older = youngest_;
+  x.younger = kNil;
+  if (youngest_ != kNil) entry_[static_cast<size_t>(youngest_)].younger = e; else oldest_ = e;
+  youngest_ = e;
+}
+
+void PrefixIndex::used(Ref deepest) noexcept {
+  for (Ref e = deepest; e != kTop; e = entry_[static_cast<size_t>(e)].parent) {
+    unlink_recency(e);
+    make_youngest(e);
   }
 }
 
-// NH-style hash over the page: sum of (t[2i]+k[2i]) * (t[2i+1]+k[2i+1]) with 32-bit
-// wrapping adds and a 64-bit product, mixed with the parent id and finalized
-// (csrc/radix_tree.cpp:65-87 of the reference describes the same family).
-uint64_t PrefixTree::edge_hash(Node parent, const int32_t* t) const noexcept {
-  uint64_t acc = 0;
-  for (int32_t i = 0; i < kBlockSize; i += 2) {
-    const uint32_t a = static_cast<uint32_t>(t[i]) + key_[i];
-    const uint32_t b = static_cast<uint32_t>(t[i + 1]) + key_[i + 1];
-    acc += static_cast<uint64_t>(a) * static_cast<uint64_t>(b);
-  }
-  return finalize64(acc ^ (static_cast<uint64_t>(static_cast<uint32_t>(parent)) << 32));
-}
-
-int64_t PrefixTree::find_edge(Node parent, const int32_t* t, uint64_t h) const noexcept {
-  for (size_t s = h & mask_;; s = (s + 1) & mask_) {
-    const Node n = slot_node_[s];
-    if (n == kNone) return -1;
-    // A hash hit alone never returns a page: parent and all tokens must agree.
-    if (slot_hash_[s] == h && parent_[sz(n)] == parent &&
-        std::memcmp(tokens_of(n), t, sizeof(int32_t) * kBlockSize) == 0) {
-      return static_cast<int64_t>(s);
-    }
-  }
-}
-
-void PrefixTree::table_put(uint64_t h, Node node) noexcept {
-  size_t s = h & mask_;
-  while (slot_node_[s] != kNone) s = (s + 1) & mask_;
-  slot_hash_[s] = h;
-  slot_node_[s] = node;
-}
-
-// Linear-probing deletion by shifting later entries back, so no tombstones pile up.
-void PrefixTree::table_remove(size_t hole) noexcept {
-  size_t s = hole;
-  for (;;) {
-    s = (s + 1) & mask_;
-    if (slot_node_[s] == kNone) break;
-    const size_t home = slot_hash_[s] & mask_;
-    // Move the entry at s into the hole unless its home lies cyclically in (hole, s].
-    const bool stays = (hole <= s) ? (home > hole && home <= s) : (home > hole || home <= s);
-    if (!stays) {
-      slot_hash_[hole] = slot_hash_[s];
-      slot_node_[hole] = slot_node_[s];
-      hole = s;
-    }
-  }
-  slot_node_[hole] = kNone;
-  slot_hash_[hole] = 0;
-}
-
-int64_t PrefixTree::match_prefix(const int32_t* tokens, int64_t n, BlockId* out) noexcept {
-  if (n <= 0 || tokens == nullptr) return 0;
-  const uint64_t now = ++clock_;
-  used_at_[kRoot] = now;
-  Node cur = kRoot;
-  int64_t pages = 0;
-  for (int64_t b = 0; b < n / kBlockSize; ++b) {
-    const int32_t* t = tokens + b * kBlockSize;
-    const int64_t s = find_edge(cur, t, edge_hash(cur, t));
-    if (s < 0) break;
-    const Node child = slot_node_[sz(s)];
-    if (pool_.incref(block_[sz(child)]) != Status::kOk) break;  // cannot fail while the tree owns it
-    out[pages++] = block_[sz(child)];
-    used_at_[sz(child)] = now;
-    cur = child;
-  }
-  // Only leaves sit in the heap; the last node's key just grew.
-  if (heap_pos_[sz(cur)] >= 0) heap_down(sz(heap_pos_[sz(cur)]));
-  return pages * kBlockSize;
-}
-
-Status PrefixTree::insert(const int32_t* tokens, int64_t n, const BlockId* blocks, int64_t num_blocks,
-                          int32_t* added) noexcept {
-  if (added != nullptr) *added = 0;
-  if (n < 0 || num_blocks < 0 || (n > 0 && tokens == nullptr) || (num_blocks > 0 && blocks == nullptr)) {
-    return Status::kInvalidArgument;
-  }
+int64_t PrefixIndex::lookup(const int32_t* tokens, int64_t n, BlockId* out) noexcept {
   const int64_t full = n / kBlockSize;
-  if (num_blocks < full) return Status::kInvalidArgument;
-
-  // 1. Walk what is cached already (read only).
-  Node cur = kRoot;
-  int64_t depth = 0;
-  for (; depth < full; ++depth) {
-    const int32_t* t = tokens + depth * kBlockSize;
-    const int64_t s = find_edge(cur, t, edge_hash(cur, t));
-    if (s < 0) break;
-    cur = slot_node_[sz(s)];
+  Ref at = kTop;
+  int64_t matched = 0;
+  for (; matched < full; ++matched) {
+    const int32_t* t = tokens + matched * kBlockSize;
+    const Ref next = find(at, t, hash_of(at, t));
+    if (next == kNil) break;
+    const BlockId page = entry_[static_cast<size_t>(next)].page;
+    if (pool_.share(page) != Fault::kNone) break;          // owner count at its limit: stop here
+    out[matched] = page;
+    at = next;
   }
-  const int64_t fresh = full - depth;
-  if (fresh > static_cast<int64_t>(spare_.size())) return Status::kOutOfNodes;
-
-  // 2. Check every new page before anything changes; marking as we go also catches the
-  //    same id given twice in one call. Marks are rolled back on refusal.
-  for (int64_t i = depth; i < full; ++i) {
-    const BlockId id = blocks[i];
-    Status bad = Status::kOk;
-    if (!pool_.valid(id)) bad = Status::kInvalidBlockId;
-    else if (pool_.ref_count(id) == 0) bad = Status::kBlockNotAllocated;
-    else if (pool_.ref_count(id) == INT32_MAX) bad = Status::kRefCountOverflow;
-    else if (owned_[sz(id)]) bad = Status::kBlockAlreadyCached;
-    if (bad != Status::kOk) {
-      for (int64_t j = depth; j < i; ++j) owned_[sz(blocks[j])] = 0;
-      return bad;
-    }
-    owned_[sz(id)] = 1;
-  }
-
-  // 3. Commit; nothing below can fail.
-  const uint64_t now = ++clock_;
-  if (fresh > 0 && heap_pos_[sz(cur)] >= 0) heap_drop(cur);  // gains a child: no longer a leaf
-  for (Node x = cur; x != kNone; x = parent_[sz(x)]) used_at_[sz(x)] = now;
-  if (fresh == 0) {
-    if (heap_pos_[sz(cur)] >= 0) heap_down(sz(heap_pos_[sz(cur)]));
-    return Status::kOk;
-  }
-  for (int64_t i = depth; i < full; ++i) {
-    const Node child = spare_.back();
-    spare_.pop_back();
-    const int32_t* t = tokens + i * kBlockSize;
-    parent_[sz(child)] = cur;
-    block_[sz(child)] = blocks[i];
-    children_[sz(child)] = 0;
-    heap_pos_[sz(child)] = -1;
-    used_at_[sz(child)] = now;
-    std::memcpy(&page_tokens_[sz(child) * kBlockSize], t, sizeof(int32_t) * kBlockSize);
-    table_put(edge_hash(cur, t), child);
-    ++children_[sz(cur)];
-    (void)pool_.incref(blocks[i]);
-    cur = child;
-  }
-  heap_add(cur);  // only the deepest new node is a leaf
-  if (added != nullptr) *added = static_cast<int32_t>(fresh);
-  return Status::kOk;
+  used(at);
+  return matched * kBlockSize;
 }
 
-int32_t PrefixTree::evict(int32_t want) noexcept {
-  int32_t freed = 0;
-  held_back_.clear();
-  while (freed < want && heap_size_ > 0) {
-    const Node leaf = heap_[0];
-    heap_drop(leaf);
-    if (pool_.ref_count(block_[sz(leaf)]) > 1) {  // a request still reads it
-      held_back_.push_back(leaf);
-      continue;
-    }
-    drop_leaf(leaf);
-    ++freed;
+Fault PrefixIndex::hold(const int32_t* tokens, int64_t n, const BlockId* pages, int64_t num_pages,
+                         int32_t* added) noexcept {
+  if (added != nullptr) *added = 0;
+  const int64_t full = n / kBlockSize;
+  if (n < 0 || num_pages < full) return Fault::kBadArgument;
+  // What is held already.
+  Ref at = kTop;
+  int64_t known = 0;
+  for (; known < full; ++known) {
+    const int32_t* t = tokens + known * kBlockSize;
+    const Ref next = find(at, t, hash_of(at, t));
+    if (next == kNil) break;
+    at = next;
   }
-  for (const Node n : held_back_) heap_add(n);
-  held_back_.clear();
+  // Every new page is looked at before anything changes.
+  if (static_cast<int64_t>(unused_.size()) < full - known) return Fault::kIndexFull;
+  if (++call_ == 0) {                                        // the counter wrapped: old marks mean nothing now
+    std::fill(seen_in_call_.begin(), seen_in_call_.end(), 0u);
+    call_ = 1;
+  }
+  for (int64_t i = known; i < full; ++i) {
+    const BlockId page = pages[i];
+    const int32_t owners = pool_.owners(page);
+    if (owners < 0) return Fault::kBadPage;
+    if (owners == 0) return Fault::kNotInUse;
+    if (owners == INT32_MAX) return Fault::kTooManyOwners;
+    if (shared_[static_cast<size_t>(page)] || seen_in_call_[static_cast<size_t>(page)] == call_)
+      return Fault::kAlreadyShared;                          // held elsewhere, or given twice in this call
+    seen_in_call_[static_cast<size_t>(page)] = call_;
+  }
+  for (int64_t i = known; i < full; ++i) {
+    const int32_t* t = tokens + i * kBlockSize;
+    const Ref e = unused_.back();
+    unused_.pop_back();
+    Entry& x = entry_[static_cast<size_t>(e)];
+    x.parent = at;
+    x.page = pages[i];
+    x.continuations = 0;
+    x.hash = hash_of(at, t);
+    std::memcpy(&text_[static_cast<size_t>(e) * kBlockSize], t, sizeof(int32_t) * kBlockSize);
+    Ref& head = bucket_[x.hash & (bucket_.size() - 1)];
+    x.same_bucket = head;
+    head = e;
+    entry_[static_cast<size_t>(at)].continuations += 1;
+    pool_.share(x.page);
+    shared_[static_cast<size_t>(x.page)] = 1;
+    make_youngest(e);
+    at = e;
+  }
+  held_ += static_cast<int32_t>(full - known);
+  if (added != nullptr) *added = static_cast<int32_t>(full - known);
+  used(at);                                                  // new pages, then their prefix, youngest last
+  return Fault::kNone;
+}
+
+void PrefixIndex::forget(Ref leaf) noexcept {
+  Entry& x = entry_[static_cast<size_t>(leaf)];
+  unlink_recency(leaf);
+  Ref* link = &bucket_[x.hash & (bucket_.size() - 1)];
+  while (*link != leaf) link = &entry_[static_cast<size_t>(*link)].same_bucket;
+  *link = x.same_bucket;
+  entry_[static_cast<size_t>(x.parent)].continuations -= 1;
+  shared_[static_cast<size_t>(x.page)] = 0;
+  pool_.drop(x.page);
+  x = Entry{};
+  unused_.push_back(leaf);
+  --held_;
+}
+
+int32_t PrefixIndex::release_oldest(int32_t want) noexcept {
+  int32_t freed = 0;
+  // From the old end. An entry stands before its ancestors, so a prefix whose last
+  // continuation goes is met later in the same walk.
+  for (Ref e = oldest_; e != kNil && freed < want;) {
+    const Ref next = entry_[static_cast<size_t>(e)].younger;
+    const Entry& x = entry_[static_cast<size_t>(e)];
+    if (x.continuations == 0 && pool_.owners(x.page) == 1) {
+      forget(e);
+      ++freed;
+    }
+    e = next;
+  }
   return freed;
 }
 
-void PrefixTree::drop_leaf(Node leaf) noexcept {
-  const Node parent = parent_[sz(leaf)];
-  const int32_t* t = tokens_of(leaf);
-  const int64_t s = find_edge(parent, t, edge_hash(parent, t));
-  if (s >= 0) table_remove(sz(s));
-  owned_[sz(block_[sz(leaf)])] = 0;
-  (void)pool_.decref(block_[sz(leaf)]);  // count was 1: the page returns to the pool
-  parent_[sz(leaf)] = kNone;
-  block_[sz(leaf)] = kNoBlock;
-  children_[sz(leaf)] = 0;
-  heap_pos_[sz(leaf)] = -1;
-  used_at_[sz(leaf)] = 0;
-  spare_.push_back(leaf);
-  if (--children_[sz(parent)] == 0 && parent != kRoot) heap_add(parent);
-}
-
-bool PrefixTree::older(Node a, Node b) const noexcept {
-  const uint64_t ta = used_at_[sz(a)], tb = used_at_[sz(b)];
-  return ta < tb || (ta == tb && a < b);  // ties by id: eviction order is deterministic
-}
-
-void PrefixTree::heap_set(size_t pos, Node n) noexcept {
-  heap_[pos] = n;
-  heap_pos_[sz(n)] = static_cast<int32_t>(pos);
-}
-
-void PrefixTree::heap_up(size_t pos) noexcept {
-  const Node n = heap_[pos];
-  while (pos > 0) {
-    const size_t up = (pos - 1) / 2;
-    if (!older(n, heap_[up])) break;
-    heap_set(pos, heap_[up]);
-    pos = up;
-  }
-  heap_set(pos, n);
-}
-
-void PrefixTree::heap_down(size_t pos) noexcept {
-  const Node n = heap_[pos];
-  for (;;) {
-    size_t kid = 2 * pos + 1;
-    if (kid >= heap_size_) break;
-    if (kid + 1 < heap_size_ && older(heap_[kid + 1], heap_[kid])) ++kid;
-    if (!older(heap_[kid], n)) break;
-    heap_set(pos, heap_[kid]);
-    pos = kid;
-  }
-  heap_set(pos, n);
-}
-
-void PrefixTree::heap_add(Node n) noexcept {
-  heap_[heap_size_] = n;
-  heap_pos_[sz(n)] = static_cast<int32_t>(heap_size_);
-  ++heap_size_;
-  heap_up(heap_size_ - 1);
-}
-
-void PrefixTree::heap_drop(Node n) noexcept {
-  const size_t pos = sz(heap_pos_[sz(n)]);
-  heap_pos_[sz(n)] = -1;
-  --heap_size_;
-  if (pos == heap_size_) return;
-  const Node moved = heap_[heap_size_];
-  heap_set(pos, moved);
-  heap_up(pos);
-  heap_down(sz(heap_pos_[sz(moved)]));
-}
-
-bool PrefixTree::check_invariants(std::string* why) const {
-  auto fail = [&](const std::string& m) {
-    if (why != nullptr) *why = m;
+bool PrefixIndex::consistent(std::string* why) const {
+  auto broken = [why](std::string what) {
+    if (why != nullptr) *why = std::move(what);
     return false;
   };
-  std::vector<uint8_t> seen_block(sz(pool_.num_blocks()), 0);
-  std::vector<int32_t> kids(sz(capacity_), 0);
-  int32_t live = 0;
-  for (Node n = 1; n < capacity_; ++n) {
-    const BlockId b = block_[sz(n)];
-    if (b == kNoBlock) {
-      if (heap_pos_[sz(n)] != -1) return fail("spare node in heap");
-      continue;
-    }
-    ++live;
-    if (!pool_.valid(b)) return fail("node holds invalid block");
-    if (seen_block[sz(b)]) return fail("block in two nodes");
-    seen_block[sz(b)] = 1;
-    if (!owned_[sz(b)]) return fail("node's block not marked cached");
-    if (pool_.ref_count(b) < 1) return fail("cached block has no reference");
-    const Node p = parent_[sz(n)];
-    if (p < 0 || p >= capacity_ || (p != kRoot && block_[sz(p)] == kNoBlock)) return fail("dangling parent");
-    ++kids[sz(p)];
-    if (used_at_[sz(p)] < used_at_[sz(n)]) return fail("parent used before child");
-    const int64_t s = find_edge(p, tokens_of(n), edge_hash(p, tokens_of(n)));
-    if (s < 0 || slot_node_[sz(s)] != n) return fail("node not reachable through the table");
+  const size_t n = entry_.size();
+  std::vector<int32_t> place(n, -1), kids(n, 0);
+  int32_t count = 0;
+  Ref before = kNil;
+  for (Ref e = oldest_; e != kNil; e = entry_[static_cast<size_t>(e)].younger) {
+    if (e <= kTop || static_cast<size_t>(e) >= n) return broken("the recency list leaves the entries");
+    if (place[static_cast<size_t>(e)] >= 0) return broken("an entry is in the recency list twice");
+    if (entry_[static_cast<size_t>(e)].older != before) return broken("recency links disagree");
+    place[static_cast<size_t>(e)] = count++;
+    before = e;
   }
-  if (live != num_cached_blocks()) return fail("live nodes != cached count");
-  for (int32_t b = 0; b < pool_.num_blocks(); ++b) {
-    if (owned_[sz(b)] && !seen_block[sz(b)]) return fail("cached mark without a node");
+  if (before != youngest_) return broken("the young end of the recency list is wrong");
+  if (count != held_) return broken("held count and recency list disagree");
+  if (static_cast<size_t>(held_) + unused_.size() + 1 != n) return broken("entries in use + unused != all");
+  int32_t marks = 0;
+  for (uint8_t m : shared_) marks += m;
+  if (marks != held_) return broken("page marks and entries disagree");
+  for (size_t e = 1; e < n; ++e) {
+    if (place[e] < 0) continue;
+    const Entry& x = entry_[e];
+    if (x.parent != kTop && (x.parent < 0 || place[static_cast<size_t>(x.parent)] < 0))
+      return broken("an entry continues a prefix that is not held");
+    if (x.parent != kTop && place[static_cast<size_t>(x.parent)] < place[e])
+      return broken("an entry stands after its prefix in the recency list");
+    kids[static_cast<size_t>(x.parent)] += 1;
+    if (!pool_.valid(x.page) || !shared_[static_cast<size_t>(x.page)]) return broken("an entry's page is not marked");
+    if (pool_.owners(x.page) < 1) return broken("the index holds a page that has no owner");
+    if (x.hash != hash_of(x.parent, text(static_cast<Ref>(e)))) return broken("a stored hash is stale");
+    if (find(x.parent, text(static_cast<Ref>(e)), x.hash) != static_cast<Ref>(e))
+      return broken("an entry cannot be found through its bucket");
   }
-  size_t in_heap = 0;
-  for (Node n = 0; n < capacity_; ++n) {
-    if (kids[sz(n)] != children_[sz(n)]) return fail("child count wrong");
-    const bool leaf = n != kRoot && block_[sz(n)] != kNoBlock && children_[sz(n)] == 0;
-    if (leaf != (heap_pos_[sz(n)] >= 0)) return fail("heap membership != leaf");
-    if (heap_pos_[sz(n)] >= 0) {
-      ++in_heap;
-      if (sz(heap_pos_[sz(n)]) >= heap_size_ || heap_[sz(heap_pos_[sz(n)])] != n) return fail("heap position stale");
-    }
+  for (size_t e = 0; e < n; ++e) {
+    if ((e == 0 || place[e] >= 0) && entry_[e].continuations != kids[e]) return broken("a continuation count is wrong");
   }
-  if (in_heap != heap_size_) return fail("heap size wrong");
-  for (size_t i = 1; i < heap_size_; ++i) {
-    if (older(heap_[i], heap_[(i - 1) / 2])) return fail("heap order broken");
-  }
-  size_t filled = 0;
-  for (size_t s = 0; s <= mask_; ++s) filled += slot_node_[s] != kNone;
-  if (filled != static_cast<size_t>(live)) return fail("table entries != live nodes");
   return true;
 }
 

@@ -1,102 +1,97 @@
-// Prefix cache over KV pages: a tree with one node per full 16-token page. A path from
-// the root spells a cached prompt prefix page by page, so a new request whose tokens
-// start the same way can reuse those pages instead of recomputing them.
+// The prefix cache: an index from token prefixes, one full page (16 tokens) at a time, to the
+// KV pages that hold them, so that a request whose tokens start like an earlier one's reuses
+// those pages instead of computing them again.
 //
-// Behaviour follows the reference's RadixTree (csrc/radix_tree.hpp:36-144,
+// What a caller can observe is the reference's RadixTree (csrc/radix_tree.hpp:36-144,
 // csrc/radix_tree.cpp:130-297):
-//   * a child is found by hashing ALL tokens of its page together with the parent id and
-//     is accepted only after comparing the tokens: two siblings may start with the same
-//     token, and the same tokens at another depth are another node;
-//   * the tree owns one reference on every cached page; a request using the page owns
-//     one more, so "count == 1" means only the tree holds it and it may be evicted;
-//   * match_prefix takes one reference per matched page for the caller;
-//   * insert is all-or-nothing, never replaces a page that is already cached for the
-//     same tokens, and ignores a trailing partial page;
-//   * evict removes least-recently-used leaves nobody else holds; a parent that loses
-//     its last child becomes a leaf and may go in the same call;
+//   * a page is found by ALL its 16 tokens and its place in the prefix, and only after the
+//     tokens were compared: two pages after the same prefix may start with the same token,
+//     and the same 16 tokens after another prefix are another entry;
+//   * the index is one owner of every page it holds and a request using the page is another,
+//     so a page with a single owner is held by the index alone and may be evicted;
+//   * match_prefix makes the caller an owner of every page it returns;
+//   * insert takes all of its new pages or none, never replaces a page that is already held
+//     for the same tokens, and ignores a trailing partial page;
+//   * evict gives up the pages used longest ago that nobody else owns, leaves first; a page
+//     whose last continuation went can go in the same call;
 //   * nothing allocates after the constructor.
-// Single-threaded by design, like its owner, the scheduler.
+//
+// How it is built here: entries live in one array; children are found through a hash table
+// with chaining (bucket heads plus a link per entry, so removal is a list unlink and there
+// are no tombstones and nothing to shift); recency is a doubly linked list through all
+// entries, oldest first, with no clock: whenever an entry is used, it and then each of its
+// ancestors move to the young end, so an entry always stands before its ancestors and a walk
+// from the old end meets the leaves of a stale prefix before the prefix itself.
+// One thread at a time, like the scheduler that owns it.
 #pragma once
 
 #include <cstdint>
 #include <string>
 #include <vector>
 
-#include "block_pool.hpp"
+#include "page_pool.hpp"
 
 namespace psamd {
 
-class PrefixTree {
+class PrefixIndex {
  public:
-  // `pool` must outlive the tree. The destructor gives the tree's references back.
-  PrefixTree(BlockPool& pool, uint64_t hash_seed);
-  ~PrefixTree();
-  PrefixTree(const PrefixTree&) = delete;
-  PrefixTree& operator=(const PrefixTree&) = delete;
+  // `pool` must outlive the index. The destructor returns the pages the index owns.
+  PrefixIndex(PagePool& pool, uint64_t seed);
+  ~PrefixIndex();
+  PrefixIndex(const PrefixIndex&) = delete;
+  PrefixIndex& operator=(const PrefixIndex&) = delete;
 
   static uint64_t random_seed();
 
-  // Longest cached prefix of tokens[0, n) in whole pages. Writes the page ids to
-  // out[0 .. matched/16) (out must hold n/16 entries), takes one reference on each for
-  // the caller, marks the path as used now. Returns the matched token count.
-  int64_t match_prefix(const int32_t* tokens, int64_t n, BlockId* out) noexcept;
+  // Longest held prefix of tokens[0, n), in whole pages: page ids into out[0 .. result / 16)
+  // (room for n / 16 entries), the caller becomes an owner of each, and the prefix counts as
+  // used now. Returns the number of tokens matched.
+  int64_t lookup(const int32_t* tokens, int64_t n, BlockId* out) noexcept;
 
-  // Caches the full pages of tokens[0, n); blocks[i] holds tokens [16i, 16i+16).
-  Status insert(const int32_t* tokens, int64_t n, const BlockId* blocks, int64_t num_blocks,
-                int32_t* added) noexcept;
+  // Holds the full pages of tokens[0, n); pages[i] has tokens [16 i, 16 i + 16). *added = how
+  // many pages the index took (those not held before).
+  Fault hold(const int32_t* tokens, int64_t n, const BlockId* pages, int64_t num_pages, int32_t* added) noexcept;
 
-  // Frees up to `want` pages, least recently used first. Returns how many were freed.
-  int32_t evict(int32_t want) noexcept;
+  // Gives up to `want` pages back to the pool; returns how many.
+  int32_t release_oldest(int32_t want) noexcept;
 
-  int32_t num_cached_blocks() const noexcept { return capacity_ - 1 - static_cast<int32_t>(spare_.size()); }
-  int32_t max_blocks() const noexcept { return pool_.num_blocks(); }
-  bool is_cached(BlockId id) const noexcept { return pool_.valid(id) && owned_[static_cast<size_t>(id)] != 0; }
+  int32_t size() const noexcept { return held_; }
+  bool holds(BlockId id) const noexcept { return pool_.valid(id) && shared_[static_cast<size_t>(id)] != 0; }
 
-  bool check_invariants(std::string* why) const;
+  bool consistent(std::string* why) const;
 
  private:
-  using Node = int32_t;
-  static constexpr Node kRoot = 0;
-  static constexpr Node kNone = -1;
+  using Ref = int32_t;                       // index of an entry; 0 is the empty prefix
+  static constexpr Ref kTop = 0, kNil = -1;
 
-  uint64_t edge_hash(Node parent, const int32_t* page_tokens) const noexcept;
-  // Slot of the child of `parent` spelling `page_tokens`, or -1.
-  int64_t find_edge(Node parent, const int32_t* page_tokens, uint64_t h) const noexcept;
-  void table_put(uint64_t h, Node node) noexcept;
-  void table_remove(size_t slot) noexcept;
-  const int32_t* tokens_of(Node n) const noexcept { return &page_tokens_[static_cast<size_t>(n) * kBlockSize]; }
+  struct Entry {
+    Ref parent = kNil;                       // the prefix this page continues
+    BlockId page = kNoBlock;
+    int32_t continuations = 0;               // entries whose parent this is
+    Ref same_bucket = kNil;                  // next entry of the hash bucket
+    Ref older = kNil, younger = kNil;        // recency list
+    uint64_t hash = 0;
+  };
 
-  // Indexed min-heap of leaves by (last use, node id); each node knows its position.
-  bool older(Node a, Node b) const noexcept;
-  void heap_set(size_t pos, Node n) noexcept;
-  void heap_up(size_t pos) noexcept;
-  void heap_down(size_t pos) noexcept;
-  void heap_add(Node n) noexcept;
-  void heap_drop(Node n) noexcept;
+  uint64_t hash_of(Ref parent, const int32_t* page_tokens) const noexcept;
+  Ref find(Ref parent, const int32_t* page_tokens, uint64_t h) const noexcept;
+  const int32_t* text(Ref e) const noexcept { return &text_[static_cast<size_t>(e) * kBlockSize]; }
+  void unlink_recency(Ref e) noexcept;
+  void make_youngest(Ref e) noexcept;
+  void used(Ref deepest) noexcept;           // the entry and its ancestors, in that order
+  void forget(Ref leaf) noexcept;
 
-  void drop_leaf(Node leaf) noexcept;
-
-  BlockPool& pool_;
-  int32_t capacity_;                 // nodes including the root: num_blocks + 1
-  uint32_t key_[kBlockSize];         // random per-position hash keys
-  uint64_t clock_ = 0;               // logical time of the last match/insert
-
-  std::vector<Node> parent_;
-  std::vector<BlockId> block_;       // kNoBlock for the root and for spare nodes
-  std::vector<int32_t> children_;
-  std::vector<int32_t> heap_pos_;    // -1 when not in the heap
-  std::vector<uint64_t> used_at_;
-  std::vector<int32_t> page_tokens_; // [capacity_][kBlockSize]
-  std::vector<Node> spare_;
-
-  std::vector<uint64_t> slot_hash_;  // open addressing, power-of-two size, <= 50 % load
-  std::vector<Node> slot_node_;      // kNone = empty
-  size_t mask_ = 0;
-
-  std::vector<Node> heap_;
-  size_t heap_size_ = 0;
-  std::vector<Node> held_back_;      // evict(): leaves somebody still uses, re-added after
-  std::vector<uint8_t> owned_;       // owned_[page] = the tree holds a reference on it
+  PagePool& pool_;
+  uint64_t seed_;
+  std::vector<Entry> entry_;                 // pages + 1
+  std::vector<int32_t> text_;                // 16 tokens per entry
+  std::vector<Ref> bucket_;                  // power of two many heads
+  std::vector<Ref> unused_;                  // entries not in use
+  std::vector<uint8_t> shared_;              // per page: the index owns it
+  std::vector<uint32_t> seen_in_call_;       // per page: the insert call that last looked at it
+  uint32_t call_ = 0;
+  Ref oldest_ = kNil, youngest_ = kNil;
+  int32_t held_ = 0;
 };
 
 }  // namespace psamd

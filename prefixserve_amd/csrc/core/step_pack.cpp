@@ -2,7 +2,7 @@
 
 #include <algorithm>
 
-#include "block_pool.hpp"
+#include "page_pool.hpp"
 
 namespace psamd {
 

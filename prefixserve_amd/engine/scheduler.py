@@ -1,162 +1,79 @@
-"""Continuous-batching scheduler over the cache manager.
+"""Continuous batching over the cache manager.
 
-Every request is a token list ``seq = prompt + output`` and a counter ``num_computed``
-(tokens whose keys and values are in the cache). A step runs some of
-``seq[num_computed:]`` for each scheduled request; a request that reaches the end of its
-``seq`` gets one new token sampled. Decode is "one token left", prefill "more than one
-left", recomputation after preemption is prefill again: one code path for all three.
+A request is a token sequence ``prompt + output`` and a count of how much of it is in the
+cache. Every step runs the next stretch of that sequence for each scheduled request; when
+the stretch reaches the end of the sequence one more token is sampled. A decode step is the
+case "one token left", a prompt portion is "several left", and recomputing after a
+preemption is a prompt portion again, so there is a single path through this file.
 
-The rules are the reference's (prefixserve/scheduler.py:143-451): running requests first
-and oldest first; decodes never use the prefill budget; prompts are cut into portions of
-at most ``chunk_size`` under a shared per-step token budget; admission is FIFO, matches the
-prefix cache on ``seq[:-1]`` and never preempts; a running request that needs pages evicts
-cached prefixes and then preempts the NEWEST running request (recompute, not swap), which
-returns to the front of the queue; aborting a request of the batch in flight waits for
-``commit``. Added here: a state slot per running request, block tables per layer group,
-release of pages a window has passed, and per-request sampling options.
+The policy is the reference's (prefixserve/scheduler.py:143-451), restated:
 
-Not thread-safe, on purpose: one owner drives schedule_step -> engine.step -> commit.
+* who runs: every running request, oldest arrival first, then newcomers in arrival order
+  while there is room for them among the running;
+* how much: a decode takes its one token and costs nothing of the step's token budget; a
+  prompt is cut into portions of at most ``chunk_size`` and of what the budget still holds;
+* a newcomer first looks its sequence up in the prefix cache (all but the last token, so
+  something is always left to run), then needs a state slot and pages for its first
+  portion; if it cannot have them it waits, and so does everyone behind it: starting a
+  request never takes anything from a running one;
+* a running request that needs a page it cannot get first has unused cached prefixes
+  evicted (inside the cache manager), then sends the newest running request back to the
+  head of the queue, as often as it takes; that request's finished pages go into the
+  prefix cache, so it usually finds them again. The oldest request can take from everyone
+  and nothing was admitted that does not fit the pool alone, so everything ends;
+* a request that is aborted while its batch is on the device keeps its pages until commit.
+
+Beyond the reference: block tables per layer group, pages a window has passed are given
+back at commit, a state slot per running request, temperature and seed per request, and
+batches of several decode steps (``schedule_step(..., decode_steps=k)``).
+
+One owner calls schedule_step -> engine.step -> commit in turn; nothing here is thread-safe.
 """
 
 from __future__ import annotations
 
-import bisect
+import itertools
 import logging
 import time
 from collections import deque
 from dataclasses import dataclass, field
-from enum import Enum
 from typing import Iterable, Mapping, Sequence
 
 import numpy as np
 
 from prefixserve_amd.cache.manager import BLOCK_SIZE, CacheManager, blocks_for
+from prefixserve_amd.engine.request import (AddResult, Batch, FinishReason, ReqState, Request, SchedulerError,
+                                            SchedulerStats, StepResult, WorkItem, as_token_list)
 
-logger = logging.getLogger(__name__)
+__all__ = ["AddResult", "Batch", "FinishReason", "ReqState", "Request", "Scheduler", "SchedulerError",
+           "SchedulerStats", "StepResult", "WorkItem", "DEFAULT_CHUNK_SIZE"]
+
+log = logging.getLogger(__name__)
 
 DEFAULT_CHUNK_SIZE = 512
-SLOW_STEP_SECONDS = 1e-3
+_SLOW_PLAN_MS = 1.0
 
 
-class SchedulerError(RuntimeError):
-    """The caller broke the schedule -> commit protocol."""
+@dataclass
+class _Plan:
+    """What schedule_step has decided so far."""
+
+    tokens_left: int                                   # of the step's prompt-token budget
+    items: list[WorkItem] = field(default_factory=list)
+    sent_back: list[str] = field(default_factory=list)
+
+    def take(self, req: Request, count: int, *, costs_budget: bool) -> None:
+        self.items.append(WorkItem(req, req.num_computed, req.num_computed + count))
+        if costs_budget:
+            self.tokens_left -= count
 
 
-class ReqState(Enum):
-    WAITING = "waiting"
-    RUNNING = "running"
-    FINISHED = "finished"
-
-
-class FinishReason(str, Enum):
-    LENGTH = "length"
-    STOP = "stop"
-    ABORT = "abort"
-
-
-class AddResult(Enum):
-    ACCEPTED = "accepted"
-    QUEUE_FULL = "queue_full"
-    TOO_LONG = "too_long"          # cannot fit even with the whole pool to itself
-    DUPLICATE_ID = "duplicate_id"
-    INVALID = "invalid"
-
-
-@dataclass(eq=False)
-class Request:
-    req_id: str
-    prompt: np.ndarray
-    max_tokens: int
-    arrival: int                    # fixed for life, so priority survives preemption
-    ignore_eos: bool = False
-    temperature: float = 0.0
-    seed: int = 0
-    state: ReqState = ReqState.WAITING
-    output: list[int] = field(default_factory=list)
-    block_tables: list[list[int]] = field(default_factory=list)   # one per layer group; 1 ref held on each entry
-    slot: int = -1
-    num_computed: int = 0
-    cached_tokens: int = 0          # tokens reused from the prefix cache, summed over admissions
-    num_preemptions: int = 0
-    abort_pending: bool = False
-    prompt_cached: bool = False
-
-    @property
-    def seq_len(self) -> int:
-        return len(self.prompt) + len(self.output)
-
-    @property
-    def block_table(self) -> list[int]:
-        """The table of the first layer group (the only one for a single-group model)."""
-        return self.block_tables[0] if self.block_tables else []
-
-    def seq(self) -> np.ndarray:
-        if not self.output:
-            return self.prompt
-        return np.concatenate((self.prompt, np.asarray(self.output, dtype=np.int32)))
-
-    def tokens(self, start: int, end: int) -> np.ndarray | list[int]:
-        """seq[start:end] without building the whole sequence: an array, or a list when all
-        of it is output (every decode step asks for that; a slice of a list costs least)."""
-        n = len(self.prompt)
-        if end <= n:
-            return self.prompt[start:end]
-        if start >= n:
-            return self.output[start - n:end - n]
-        return np.concatenate((self.prompt[start:], np.asarray(self.output[:end - n], dtype=np.int32)))
-
-
-@dataclass(frozen=True)
-class WorkItem:
-    req: Request
-    start: int      # run seq[start:end]
-    end: int
-
-    @property
-    def samples(self) -> bool:
-        """The item reaches the end of seq, so a token must be sampled for it."""
-        return self.end == self.req.seq_len
-
-
-@dataclass(frozen=True)
-class Batch:
-    """``decode_steps`` > 1: every item is a decoding request and the engine runs that many
-    steps in a row for them (item j of a request starts at ``start + j``), feeding each step's
-    token to the next on the device; ``commit`` then takes a list of tokens per request."""
-
-    work: list[WorkItem]
-    preempted: list[str]
-    decode_steps: int = 1
-
-    @property
-    def num_tokens(self) -> int:
-        return sum(w.end - w.start for w in self.work)
-
-
-@dataclass(frozen=True)
-class StepResult:
-    """``new_tokens``: the last token each request got in this commit; ``tokens``: all of
-    them in order (more than one after a batch of several decode steps)."""
-
-    new_tokens: dict[str, int]
-    finished: dict[str, FinishReason]
-    tokens: dict[str, list[int]] = field(default_factory=dict)
-
-
-@dataclass(frozen=True)
-class SchedulerStats:
-    num_waiting: int
-    num_running: int
-    free_blocks: int
-    cached_blocks: int
-    prompt_tokens: int
-    cached_prompt_tokens: int
-    preemptions: int
-    rejected: int
-
-    @property
-    def prefix_hit_rate(self) -> float:
-        return self.cached_prompt_tokens / self.prompt_tokens if self.prompt_tokens else 0.0
+@dataclass
+class _Tally:
+    prompt_tokens: int = 0
+    cached_prompt_tokens: int = 0
+    preemptions: int = 0
+    rejected: int = 0
 
 
 class Scheduler:
@@ -164,292 +81,291 @@ class Scheduler:
                  chunk_size: int = DEFAULT_CHUNK_SIZE, stop_token_ids: Iterable[int] = (),
                  enable_prefix_cache: bool = True, cache: CacheManager | None = None,
                  num_slots: int = 1024) -> None:
-        if max_waiting < 1 or chunk_size < 1:
-            raise ValueError("max_waiting and chunk_size must be >= 1")
+        if chunk_size < 1 or max_waiting < 1:
+            raise ValueError("chunk_size and max_waiting must be at least 1")
         if cache is None:
             if num_blocks is None:
-                raise ValueError("give num_blocks or a CacheManager")
-            sizes = [num_blocks] if isinstance(num_blocks, int) else list(num_blocks)
-            cache = CacheManager(sizes, num_slots=num_slots, enable_prefix_cache=enable_prefix_cache)
+                raise ValueError("a Scheduler needs num_blocks or a CacheManager")
+            pools = list(num_blocks) if not isinstance(num_blocks, int) else [num_blocks]
+            cache = CacheManager(pools, num_slots=num_slots, enable_prefix_cache=enable_prefix_cache)
         self.cache = cache
+        # The first group's pool and tree under the reference's names.
         self.block_manager = cache.pools[0]
         self.tree = cache.trees[0] if cache.trees else None
-        self._max_waiting = max_waiting
-        self._chunk_size = chunk_size
-        self._stop = frozenset(int(t) for t in stop_token_ids)
+        self.chunk_size = int(chunk_size)
+        self.max_waiting = int(max_waiting)
+        self.stop_token_ids = frozenset(int(t) for t in stop_token_ids)
 
-        self._requests: dict[str, Request] = {}
-        self._waiting: deque[Request] = deque()
-        self._running: list[Request] = []     # by arrival, newest last
-        self._inflight: Batch | None = None
-        self._pending_aborts: list[Request] = []
-        self._next_arrival = 0
-        self._prompt_tokens = 0
-        self._cached_prompt_tokens = 0
-        self._preemptions = 0
-        self._rejected = 0
+        self._live: dict[str, Request] = {}            # everything not finished, by id
+        self._queue: deque[Request] = deque()          # waiting, next to start first
+        self._active: list[Request] = []               # running, oldest arrival first
+        self._open: Batch | None = None                # scheduled, not yet committed
+        self._abort_at_commit: list[Request] = []
+        self._arrivals = itertools.count()
+        self._tally = _Tally()
 
-    # ---------------------------------------------------------------- API
+    # ------------------------------------------------------------------ requests in and out
 
     def add_request(self, req_id: str, prompt: Iterable[int] | np.ndarray, max_tokens: int, *,
                     ignore_eos: bool = False, temperature: float = 0.0, seed: int = 0) -> AddResult:
-        checked = self._validate(req_id, prompt, max_tokens, temperature)
-        if isinstance(checked, AddResult):
-            self._rejected += 1
-            return checked
-        req = Request(req_id=req_id, prompt=checked, max_tokens=max_tokens, arrival=self._next_arrival,
-                      ignore_eos=ignore_eos, temperature=float(temperature), seed=int(seed))
-        self._next_arrival += 1
-        self._requests[req_id] = req
-        self._waiting.append(req)
-        self._prompt_tokens += len(checked)
+        verdict, ids = self._screen(req_id, prompt, max_tokens, temperature)
+        if ids is None:
+            self._tally.rejected += 1
+            return verdict
+        req = Request(req_id, ids, max_tokens, next(self._arrivals), ignore_eos=ignore_eos,
+                      temperature=float(temperature), seed=int(seed))
+        self._live[req_id] = req
+        self._queue.append(req)
+        self._tally.prompt_tokens += int(ids.shape[0])
         return AddResult.ACCEPTED
 
-    def schedule_step(self, max_prefill_tokens: int, max_decode_seqs: int, decode_steps: int = 1) -> Batch:
-        """Chooses this step's work. ``commit`` must follow before the next call.
-
-        ``decode_steps`` > 1 lets a batch that holds nothing but decoding requests, with nobody
-        waiting, run up to that many steps before the host looks at the tokens (fewer if a
-        request would pass its ``max_tokens`` or the free pages do not reach). A request that
-        meets a stop token in between finishes there; what was computed for it after that is
-        dropped. Nothing else changes: the pages for those positions are taken now."""
-        if self._inflight is not None:
-            raise SchedulerError("commit() the previous batch before scheduling another")
-        if max_prefill_tokens < 1 or max_decode_seqs < 1:
-            raise ValueError("max_prefill_tokens and max_decode_seqs must be >= 1")
-        started = time.perf_counter()
-        work: list[WorkItem] = []
-        preempted: list[str] = []
-        budget = max_prefill_tokens
-
-        # Running requests, oldest first. A victim of _reserve is always newer than the
-        # asker, hence later in this loop and never in `work` already.
-        i = 0
-        while i < len(self._running):
-            req = self._running[i]
-            remaining = req.seq_len - req.num_computed
-            n = 1 if remaining == 1 else min(self._chunk_size, remaining, budget)
-            if n == 0:           # budget used up: this prefill waits a step
-                i += 1
-                continue
-            need = [max(blocks_for(req.num_computed + n) - len(t), 0) for t in req.block_tables]
-            if any(need) and not self._reserve(req, need, preempted):
-                continue         # req preempted itself; the same index now holds the next request
-            if remaining > 1:
-                budget -= n
-            work.append(WorkItem(req, req.num_computed, req.num_computed + n))
-            i += 1
-
-        # Waiting requests, first come first served; the head that cannot start blocks the rest.
-        while self._waiting and len(self._running) < max_decode_seqs:
-            item = self._admit(self._waiting[0], budget)
-            if item is None:
-                break
-            self._waiting.popleft()
-            if item.end - item.start > 1:
-                budget -= item.end - item.start
-            work.append(item)
-
-        steps = 1
-        if (decode_steps > 1 and work and not self._waiting and not preempted
-                and all(w.end - w.start == 1 and w.samples for w in work)):
-            steps = min(decode_steps, min(w.req.max_tokens - len(w.req.output) for w in work))
-            for w in work:
-                if steps == 1:
-                    break
-                need = [max(blocks_for(w.start + steps) - len(t), 0) for t in w.req.block_tables]
-                if any(need):
-                    fresh = self.cache.allocate(need)
-                    if fresh is None:
-                        steps = 1        # pages already taken for others stay theirs: they will be used
-                    else:
-                        for table, new in zip(w.req.block_tables, fresh):
-                            table.extend(new)
-        batch = Batch(work=work, preempted=preempted, decode_steps=steps)
-        self._inflight = batch
-        elapsed = time.perf_counter() - started
-        if elapsed > SLOW_STEP_SECONDS:
-            logger.debug("schedule_step took %.2f ms", elapsed * 1e3)
-        return batch
-
-    def commit(self, batch: Batch, sampled: Mapping[str, int]) -> StepResult:
-        """Applies the engine's results; ``sampled`` has a token for every item that samples."""
-        if batch is not self._inflight:
-            raise SchedulerError("commit() got a batch that isn't the one in flight")
-        self._inflight = None
-        new_tokens: dict[str, int] = {}
-        all_tokens: dict[str, list[int]] = {}
-        finished: dict[str, FinishReason] = {}
-        for w in batch.work:
-            req = w.req
-            if req.num_computed != w.start:
-                raise SchedulerError(f"{req.req_id}: batch is stale")
-            if not w.samples:
-                req.num_computed = w.end
-                self.cache.trim_windows(req.block_tables, req.num_computed)
-                continue
-            if req.req_id not in sampled:
-                raise SchedulerError(f"engine returned no token for {req.req_id}")
-            got = sampled[req.req_id]
-            tokens = [int(got)] if isinstance(got, (int, np.integer)) else [int(t) for t in got]
-            if len(tokens) != batch.decode_steps:
-                raise SchedulerError(f"{req.req_id}: {len(tokens)} tokens for {batch.decode_steps} decode steps")
-            for j, token in enumerate(tokens):
-                req.num_computed = w.end + j
-                self.cache.trim_windows(req.block_tables, req.num_computed)
-                if not req.prompt_cached:      # prompt complete for the first time: share it now
-                    self._cache(req)
-                    req.prompt_cached = True
-                req.output.append(token)
-                new_tokens[req.req_id] = token
-                all_tokens.setdefault(req.req_id, []).append(token)
-                if req.abort_pending:
-                    break
-                if token in self._stop and not req.ignore_eos:
-                    self._finish(req, FinishReason.STOP)
-                    finished[req.req_id] = FinishReason.STOP
-                    break
-                if len(req.output) >= req.max_tokens:
-                    self._finish(req, FinishReason.LENGTH)
-                    finished[req.req_id] = FinishReason.LENGTH
-                    break
-        for req in self._pending_aborts:   # safe now: the batch that wrote their pages is done
-            if req.state is ReqState.RUNNING:
-                self._finish(req, FinishReason.ABORT)
-                finished[req.req_id] = FinishReason.ABORT
-        self._pending_aborts.clear()
-        return StepResult(new_tokens=new_tokens, finished=finished, tokens=all_tokens)
+    def _screen(self, req_id: str, prompt: Iterable[int] | np.ndarray, max_tokens: int,
+                temperature: float) -> tuple[AddResult, np.ndarray | None]:
+        """(verdict, the prompt as our own int32 copy or None)."""
+        bad = AddResult.INVALID, None
+        if not req_id or isinstance(max_tokens, bool) or not isinstance(max_tokens, int) or max_tokens < 1:
+            return bad
+        try:
+            ids = np.asarray(prompt)
+            temperature_ok = float(temperature) >= 0.0
+        except (TypeError, ValueError, OverflowError):
+            return bad
+        # Integers only: a float prompt would be truncated without a word.
+        if not temperature_ok or ids.ndim != 1 or ids.size == 0 or ids.dtype.kind not in "iu":
+            return bad
+        if ids.min() < 0 or ids.max() > np.iinfo(np.int32).max:
+            return bad
+        if req_id in self._live:
+            return AddResult.DUPLICATE_ID, None
+        longest = int(ids.size) + max_tokens
+        if any(self.cache.pages_needed(g, longest, self.chunk_size) > self.cache.num_blocks(g)
+               for g in range(self.cache.num_groups)):
+            return AddResult.TOO_LONG, None            # would not finish with the pool to itself
+        if len(self._queue) >= self.max_waiting:
+            return AddResult.QUEUE_FULL, None
+        return AddResult.ACCEPTED, ids.astype(np.int32)   # astype copies: the caller's array stays theirs
 
     def free_request(self, req_id: str) -> bool:
-        """Aborts a request. False for an unknown id or a second call."""
-        req = self._requests.get(req_id)
+        """Aborts a request; False if there is none of that id or it is being aborted already."""
+        req = self._live.get(req_id)
         if req is None or req.abort_pending:
             return False
         if req.state is ReqState.WAITING:
-            self._waiting.remove(req)
+            self._queue.remove(req)
             req.state = ReqState.FINISHED
-            del self._requests[req_id]
-            return True
-        if self._inflight is not None:
-            # The device may still be writing this request's pages; give them back at commit.
+            self._live.pop(req_id)
+        elif self._open is None:
+            self._retire(req, FinishReason.ABORT)
+        else:
+            # Its pages may be written by the step on the device: they go back at commit.
             req.abort_pending = True
-            self._pending_aborts.append(req)
-            return True
-        self._finish(req, FinishReason.ABORT)
+            self._abort_at_commit.append(req)
         return True
 
     def get_request(self, req_id: str) -> Request | None:
-        return self._requests.get(req_id)
+        return self._live.get(req_id)
+
+    def requests(self) -> list[Request]:
+        """Every request that has not finished, waiting or running."""
+        return list(self._live.values())
 
     def has_work(self) -> bool:
-        return bool(self._waiting or self._running)
+        return bool(self._active) or bool(self._queue)
 
     def stats(self) -> SchedulerStats:
-        return SchedulerStats(
-            num_waiting=len(self._waiting), num_running=len(self._running),
-            free_blocks=self.cache.num_free(0), cached_blocks=self.cache.num_cached(0),
-            prompt_tokens=self._prompt_tokens, cached_prompt_tokens=self._cached_prompt_tokens,
-            preemptions=self._preemptions, rejected=self._rejected)
+        t = self._tally
+        return SchedulerStats(num_waiting=len(self._queue), num_running=len(self._active),
+                              free_blocks=self.cache.num_free(0), cached_blocks=self.cache.num_cached(0),
+                              prompt_tokens=t.prompt_tokens, cached_prompt_tokens=t.cached_prompt_tokens,
+                              preemptions=t.preemptions, rejected=t.rejected)
 
-    # ---------------------------------------------------------- internals
+    # ------------------------------------------------------------------ planning a step
 
-    def _validate(self, req_id: str, prompt: Iterable[int] | np.ndarray, max_tokens: int,
-                  temperature: float) -> np.ndarray | AddResult:
-        if not req_id or not isinstance(max_tokens, int) or isinstance(max_tokens, bool) or max_tokens < 1:
-            return AddResult.INVALID
-        try:
-            if not float(temperature) >= 0.0:
-                return AddResult.INVALID
-            arr = np.asarray(prompt)
-        except (TypeError, ValueError, OverflowError):
-            return AddResult.INVALID
-        if arr.ndim != 1 or arr.size == 0 or arr.dtype.kind not in "iu":
-            return AddResult.INVALID      # floats would be truncated silently
-        if int(arr.min()) < 0 or int(arr.max()) > np.iinfo(np.int32).max:
-            return AddResult.INVALID
-        if req_id in self._requests:
-            return AddResult.DUPLICATE_ID
-        total = int(arr.size) + max_tokens
-        for g in range(self.cache.num_groups):
-            if self.cache.pages_needed(g, total, self._chunk_size) > self.cache.num_blocks(g):
-                return AddResult.TOO_LONG  # could never finish even alone
-        if len(self._waiting) >= self._max_waiting:
-            return AddResult.QUEUE_FULL
-        return arr.astype(np.int32)       # a copy: later changes by the caller do not reach us
+    def schedule_step(self, max_prefill_tokens: int, max_decode_seqs: int, decode_steps: int = 1) -> Batch:
+        """Decides the next step's work; ``commit`` of this batch must come before the next call.
 
-    def _admit(self, req: Request, budget: int) -> WorkItem | None:
-        seq = req.seq()
-        # At least one token stays to be computed: the model must run something to give logits.
-        matched, cached = self.cache.match_prefix(seq[:-1])
-        remaining = len(seq) - matched
-        n = 1 if remaining == 1 else min(self._chunk_size, remaining, budget)
-        fresh = None
-        slot = None
-        if n > 0:
-            slot = self.cache.acquire_slot()
-            if slot is not None:
-                need = [blocks_for(matched + n) - len(t) for t in cached]
-                fresh = self.cache.allocate(need)
-        if fresh is None:
-            # Admission never preempts: evicting a running request to start a new one only
-            # swaps who waits, and under load both keep redoing work.
-            self.cache.release(cached)
-            if slot is not None:
-                self.cache.release_slot(slot)
-            return None
-        req.block_tables = [c + f for c, f in zip(cached, fresh)]
-        req.slot = slot if slot is not None else -1
-        req.num_computed = matched
-        req.cached_tokens += matched
-        if req.num_preemptions == 0:
-            self._cached_prompt_tokens += min(matched, len(req.prompt))
-        req.state = ReqState.RUNNING
-        bisect.insort(self._running, req, key=lambda r: r.arrival)
-        return WorkItem(req, matched, matched + n)
+        ``decode_steps`` > 1: if the batch holds only decoding requests and nobody waits, it
+        may run up to that many steps before the host sees the tokens (fewer if a request
+        would pass its ``max_tokens`` or the free pages do not reach that far; the pages are
+        taken now). A request that samples a stop token in between ends there and what was
+        computed for it afterwards is dropped."""
+        if self._open is not None:
+            raise SchedulerError("the previous batch has not been committed")
+        if min(max_prefill_tokens, max_decode_seqs) < 1:
+            raise ValueError("max_prefill_tokens and max_decode_seqs must be at least 1")
+        t0 = time.perf_counter()
+        plan = _Plan(tokens_left=max_prefill_tokens)
+        # A request sent back while an older one grows is newer than that one, so its turn in
+        # this loop has not come yet: the state check skips it.
+        for req in tuple(self._active):
+            if req.state is ReqState.RUNNING:
+                self._continue(req, plan)
+        while self._queue and len(self._active) < max_decode_seqs and self._start(self._queue[0], plan):
+            self._queue.popleft()
+        batch = Batch(plan.items, plan.sent_back, self._decode_lookahead(plan, decode_steps))
+        self._open = batch
+        spent_ms = 1e3 * (time.perf_counter() - t0)
+        if spent_ms > _SLOW_PLAN_MS:
+            log.debug("planning a step took %.2f ms", spent_ms)
+        return batch
 
-    def _reserve(self, req: Request, need: list[int], preempted: list[str]) -> bool:
-        """More pages for a running request: evict cached prefixes, then preempt the newest
-        running request, until it fits. False if ``req`` itself had to go. The oldest request
-        can take from everyone newer and nothing admitted exceeds the pool, so it finishes."""
+    def _portion(self, left: int, plan: _Plan) -> int:
+        """Tokens of a sequence with ``left`` uncomputed tokens to run now (0: none this step)."""
+        return 1 if left == 1 else min(left, self.chunk_size, plan.tokens_left)
+
+    def _continue(self, req: Request, plan: _Plan) -> None:
+        left = req.seq_len - req.num_computed
+        count = self._portion(left, plan)
+        if count > 0 and self._grow(req, req.num_computed + count, plan):
+            plan.take(req, count, costs_budget=left > 1)
+
+    def _grow(self, req: Request, upto: int, plan: _Plan) -> bool:
+        """Pages for positions [0, upto) of a running request. False: ``req`` itself had to go."""
         while True:
-            fresh = self.cache.allocate(need)
-            if fresh is not None:
-                for table, new in zip(req.block_tables, fresh):
-                    table.extend(new)
+            short = [max(blocks_for(upto) - len(table), 0) for table in req.block_tables]
+            if not any(short):
                 return True
-            victim = self._running[-1]
-            self._preempt(victim)
-            preempted.append(victim.req_id)
-            if victim is req:
+            fresh = self.cache.allocate(short)
+            if fresh is not None:
+                for table, more in zip(req.block_tables, fresh):
+                    table += more
+                return True
+            newest = self._active[-1]
+            self._send_back(newest)
+            plan.sent_back.append(newest.req_id)
+            if newest is req:
                 return False
 
-    def _release(self, req: Request) -> None:
+    def _start(self, req: Request, plan: _Plan) -> bool:
+        """Tries to make the head of the queue a running request with its first portion planned."""
+        seq = req.seq()
+        hit, shared = self.cache.match_prefix(seq[:-1])      # the last token always runs: it gives the logits
+        count = self._portion(len(seq) - hit, plan)
+        slot = self.cache.acquire_slot() if count > 0 else None
+        own = None
+        if slot is not None:
+            own = self.cache.allocate([blocks_for(hit + count) - len(table) for table in shared])
+        if own is None:
+            self.cache.release(shared)
+            if slot is not None:
+                self.cache.release_slot(slot)
+            return False
+        req.block_tables = [a + b for a, b in zip(shared, own)]
+        req.slot, req.num_computed, req.state = slot, hit, ReqState.RUNNING
+        req.cached_tokens += hit
+        if req.num_preemptions == 0:
+            self._tally.cached_prompt_tokens += min(hit, int(req.prompt.shape[0]))
+        # Oldest arrival first; a request that returns after a preemption goes back to its place.
+        at = next((i for i, other in enumerate(self._active) if other.arrival > req.arrival), len(self._active))
+        self._active.insert(at, req)
+        plan.take(req, count, costs_budget=count > 1)
+        return True
+
+    def _decode_lookahead(self, plan: _Plan, wanted: int) -> int:
+        """How many decode steps the planned batch may run in a row."""
+        if wanted <= 1 or not plan.items or self._queue or plan.sent_back:
+            return 1
+        if any(item.end - item.start != 1 or not item.samples for item in plan.items):
+            return 1
+        steps = min(wanted, min(item.req.max_tokens - len(item.req.output) for item in plan.items))
+        if steps <= 1:
+            return 1
+        for item in plan.items:
+            tables = item.req.block_tables
+            short = [max(blocks_for(item.start + steps) - len(table), 0) for table in tables]
+            if any(short):
+                fresh = self.cache.allocate(short)
+                if fresh is None:
+                    return 1           # pages already taken for others stay theirs and get used later
+                for table, more in zip(tables, fresh):
+                    table += more
+        return steps
+
+    # ------------------------------------------------------------------ after the step
+
+    def commit(self, batch: Batch, sampled: Mapping[str, int | Sequence[int]]) -> StepResult:
+        """Takes the engine's tokens for ``batch``: one per sampling request, or one per decode
+        step each for a batch of several decode steps."""
+        if self._open is None or batch is not self._open:
+            raise SchedulerError("this is not the batch that was scheduled last")
+        self._open = None
+        last: dict[str, int] = {}
+        everything: dict[str, list[int]] = {}
+        ended: dict[str, FinishReason] = {}
+        for item in batch.work:
+            req = item.req
+            if req.num_computed != item.start:
+                raise SchedulerError(f"{req.req_id}: the batch does not continue where the request stands")
+            if not item.samples:
+                self._computed(req, item.end)
+                continue
+            if req.req_id not in sampled:
+                raise SchedulerError(f"the engine gave no token for {req.req_id}")
+            tokens = as_token_list(sampled[req.req_id])
+            if len(tokens) != batch.decode_steps:
+                raise SchedulerError(f"{req.req_id}: {len(tokens)} tokens for {batch.decode_steps} decode steps")
+            for extra, token in enumerate(tokens):
+                self._computed(req, item.end + extra)
+                if not req.prompt_cached:
+                    # The whole prompt is in the cache for the first time: others may share it now.
+                    self._remember(req)
+                    req.prompt_cached = True
+                req.output.append(token)
+                last[req.req_id] = token
+                everything.setdefault(req.req_id, []).append(token)
+                why = self._why_finished(req, token)
+                if why is not None:
+                    self._retire(req, why)
+                    ended[req.req_id] = why
+                if why is not None or req.abort_pending:
+                    break
+        for req in self._abort_at_commit:
+            if req.state is ReqState.RUNNING:
+                self._retire(req, FinishReason.ABORT)
+                ended[req.req_id] = FinishReason.ABORT
+        self._abort_at_commit = []
+        return StepResult(new_tokens=last, finished=ended, tokens=everything)
+
+    def _computed(self, req: Request, upto: int) -> None:
+        req.num_computed = upto
+        self.cache.trim_windows(req.block_tables, upto)
+
+    def _why_finished(self, req: Request, token: int) -> FinishReason | None:
+        if req.abort_pending:
+            return None                                  # the abort below decides
+        if token in self.stop_token_ids and not req.ignore_eos:
+            return FinishReason.STOP
+        if len(req.output) >= req.max_tokens:
+            return FinishReason.LENGTH
+        return None
+
+    # ------------------------------------------------------------------ leaving the running set
+
+    def _remember(self, req: Request) -> None:
+        """Puts the request's full computed pages into the prefix cache."""
+        if req.num_computed >= BLOCK_SIZE:
+            self.cache.cache(req.seq()[:req.num_computed], req.block_tables)
+
+    def _give_back(self, req: Request) -> None:
+        self._remember(req)
         self.cache.release(req.block_tables)
         req.block_tables = []
         if req.slot >= 0:
             self.cache.release_slot(req.slot)
-            req.slot = -1
+        req.slot = -1
+        self._active.remove(req)
 
-    def _preempt(self, req: Request) -> None:
-        # Recompute, not swap; but what it computed is cached first, so coming back is
-        # usually a prefix hit on its own pages.
-        self._cache(req)
-        self._release(req)
+    def _send_back(self, req: Request) -> None:
+        """Preemption: recompute later rather than keep. It goes to the head of the queue."""
+        self._give_back(req)
         req.num_computed = 0
         req.num_preemptions += 1
         req.state = ReqState.WAITING
-        self._running.remove(req)
-        self._waiting.appendleft(req)
-        self._preemptions += 1
+        self._queue.appendleft(req)
+        self._tally.preemptions += 1
 
-    def _finish(self, req: Request, reason: FinishReason) -> None:
-        self._cache(req)
-        self._release(req)
+    def _retire(self, req: Request, why: FinishReason) -> None:
+        self._give_back(req)
         req.state = ReqState.FINISHED
-        self._running.remove(req)
-        del self._requests[req.req_id]
-        logger.debug("finished %s: %s", req.req_id, reason.value)
-
-    def _cache(self, req: Request) -> None:
-        if req.num_computed >= BLOCK_SIZE:
-            self.cache.cache(req.seq()[:req.num_computed], req.block_tables)
+        self._live.pop(req.req_id)
+        log.debug("%s finished: %s", req.req_id, why.value)

@@ -1,4 +1,5 @@
-"""Configuration parsing and the architecture registry. Vectors are the reference's
+"""Reading config.json into the typed configuration, and the registry from architecture names
+to models. The 8B numbers and the four refusals are those of the reference's own test
 (tests/test_llama_config.py:18-64)."""
 
 from __future__ import annotations
@@ -12,65 +13,75 @@ from prefixserve_amd.config import (Llama3RopeScaling, LlamaConfig, UnknownArchi
                                     architecture_of, read_model_dir, registered_architectures)
 from prefixserve_amd.parts import DecoderModel
 
-SCALING = {"factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
-           "original_max_position_embeddings": 8192, "rope_type": "llama3"}
-WANT = Llama3RopeScaling(8.0, 1.0, 4.0, 8192)
+LLAMA3_RULE = dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                   original_max_position_embeddings=8192)
+SCALING = LLAMA3_RULE
 
 
-def base(**kw):
-    cfg = {"model_type": "llama", "vocab_size": 128256, "hidden_size": 4096, "intermediate_size": 14336,
-           "num_hidden_layers": 32, "num_attention_heads": 32, "num_key_value_heads": 8, "rms_norm_eps": 1e-5,
-           "max_position_embeddings": 131072, "eos_token_id": 128001}
-    cfg.update(kw)
-    return cfg
+def base(**changes):
+    """config.json of the 8B model without its rope entries, plus ``changes``."""
+    raw = dict(model_type="llama", vocab_size=128256, hidden_size=4096, intermediate_size=14336, num_hidden_layers=32,
+               num_attention_heads=32, num_key_value_heads=8, rms_norm_eps=1e-5, max_position_embeddings=131072,
+               eos_token_id=128001)
+    raw.update(changes)
+    return raw
 
 
-def test_transformers4_layout():
-    c = LlamaConfig.from_dicts(base(rope_theta=500000.0, rope_scaling=SCALING), {"eos_token_id": [128001, 128008, 128009]})
-    assert c.rope_theta == 500000.0 and c.rope_scaling == WANT
-    assert c.head_dim == 128 and c.q_size == 4096 and c.kv_size == 1024
-    assert c.stop_token_ids == {128001, 128008, 128009}
+def parse(gen=None, **changes):
+    return LlamaConfig.from_dicts(base(**changes), gen)
 
 
-def test_transformers5_layout():
-    c = LlamaConfig.from_dicts(base(rope_parameters={**SCALING, "rope_theta": 500000.0}))
-    assert c.rope_theta == 500000.0 and c.rope_scaling == WANT
+@pytest.mark.parametrize("layout", ["top-level keys", "one rope_parameters dict"])
+def test_rope_entries_in_either_layout(layout):
+    if layout == "top-level keys":
+        cfg = parse(rope_theta=500000.0, rope_scaling=LLAMA3_RULE)
+    else:
+        cfg = parse(rope_parameters=dict(LLAMA3_RULE, rope_theta=500000.0))
+    assert cfg.rope_theta == 500000.0
+    assert cfg.rope_scaling == Llama3RopeScaling(factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                                                 original_max_position_embeddings=8192)
 
 
-def test_no_scaling_and_defaults():
-    for raw in (base(rope_theta=500000.0), base(rope_parameters={"rope_type": "default", "rope_theta": 500000.0})):
-        c = LlamaConfig.from_dicts(raw)
-        assert c.rope_theta == 500000.0 and c.rope_scaling is None
-    c = LlamaConfig.from_dicts(base())
-    assert c.rope_theta == 10000.0 and not c.tie_word_embeddings
-    assert LlamaConfig.from_dicts(base(rope_theta=1.0)).stop_token_ids == {128001}
-    assert LlamaConfig.from_dicts(base(head_dim=64)).head_dim == 64
-    assert LlamaConfig.from_dicts(base(head_dim=None)).head_dim == 128
-    c = LlamaConfig.from_dicts({k: v for k, v in base().items() if k != "num_key_value_heads"})
-    assert c.num_kv_heads == 32
+def test_sizes_that_follow_from_the_keys():
+    cfg = parse()
+    assert (cfg.head_dim, cfg.q_size, cfg.kv_size) == (128, 4096, 1024)
+    assert parse(head_dim=64).head_dim == 64 and parse(head_dim=None).head_dim == 128
+    without_kv = base()
+    without_kv.pop("num_key_value_heads")
+    assert LlamaConfig.from_dicts(without_kv).num_kv_heads == 32
 
 
-@pytest.mark.parametrize("bad", [
-    {"model_type": "mistral"}, {"rope_scaling": {"rope_type": "yarn", "factor": 4.0}},
-    {"attention_bias": True}, {"mlp_bias": True}, {"num_key_value_heads": 5},
-])
-def test_refuses_what_it_cannot_run(bad):
+def test_defaults_and_stop_ids():
+    cfg = parse()
+    assert cfg.rope_theta == 10000.0 and cfg.rope_scaling is None and cfg.tie_word_embeddings is False
+    assert cfg.stop_token_ids == {128001}
+    assert parse(gen={"eos_token_id": [128001, 128008, 128009]}).stop_token_ids == {128001, 128008, 128009}
+    for no_rule in (dict(rope_theta=500000.0), dict(rope_parameters={"rope_type": "default", "rope_theta": 500000.0})):
+        cfg = parse(**no_rule)
+        assert cfg.rope_theta == 500000.0 and cfg.rope_scaling is None
+
+
+@pytest.mark.parametrize("change", [dict(model_type="mistral"), dict(rope_scaling={"rope_type": "yarn", "factor": 4.0}),
+                                    dict(attention_bias=True), dict(mlp_bias=True), dict(num_key_value_heads=5)])
+def test_what_cannot_run_is_refused(change):
     with pytest.raises(UnsupportedModelError):
-        LlamaConfig.from_dicts(base(**bad))
+        parse(**change)
 
 
-def test_missing_required_key_raises():
-    raw = base()
-    del raw["rms_norm_eps"]
-    with pytest.raises(KeyError):
-        LlamaConfig.from_dicts(raw)
-    with pytest.raises(KeyError):
-        LlamaConfig.from_dicts(base(rope_scaling={"rope_type": "llama3", "factor": 8.0}))
+def test_a_key_that_is_needed_and_missing_is_named():
+    incomplete = base()
+    incomplete.pop("rms_norm_eps")
+    with pytest.raises(KeyError, match="rms_norm_eps"):
+        LlamaConfig.from_dicts(incomplete)
+    with pytest.raises(KeyError, match="low_freq_factor"):
+        parse(rope_scaling={"rope_type": "llama3", "factor": 8.0})
 
 
-def test_roundtrip_through_config_json():
-    c = LlamaConfig.from_dicts(base(rope_theta=500000.0, rope_scaling=SCALING, tie_word_embeddings=True))
-    assert LlamaConfig.from_dicts(c.to_config_json()) == c
+def test_what_is_written_reads_back():
+    cfg = parse(rope_theta=500000.0, rope_scaling=LLAMA3_RULE, tie_word_embeddings=True)
+    assert LlamaConfig.from_dicts(cfg.to_config_json()) == cfg
+    plain = parse()
+    assert LlamaConfig.from_dicts(plain.to_config_json()) == plain
 
 
 def test_registry(tmp_path):

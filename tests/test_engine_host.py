@@ -144,7 +144,7 @@ def test_stop_token_ends_generation(model_dirs, plain_models):
     eng = Engine(EngineConfig(model_path=model_dirs["A"], dtype="float32", device="cpu", max_num_seqs=2,
                               max_seq_len=128, num_blocks=16, use_graphs=False), ops=EmulatedOps())
     sched = eng.make_scheduler()
-    sched._stop = frozenset({want[3]})
+    sched.stop_token_ids = frozenset({want[3]})
     outs, _ = generate(eng, [prompt], 6, scheduler=sched)
     stop_at = want.index(want[3])
     assert outs[0].tokens == want[:stop_at + 1] and outs[0].finish_reason.value == "stop"
@@ -174,10 +174,10 @@ def test_several_decode_steps_give_the_same_tokens(temperature, model_dirs, plai
     if temperature == 0.0:
         assert one[0].tokens == plain_models["A"].greedy(prompts[0], 11)[0]
         sched = eng.make_scheduler()
-        sched._stop = frozenset({one[1].tokens[5]})
+        sched.stop_token_ids = frozenset({one[1].tokens[5]})
         stopped, _ = generate(eng, prompts, 11, scheduler=sched, decode_steps=4)
         for o, full in zip(stopped, one):
-            cut = next((i for i, t in enumerate(full.tokens) if t in sched._stop), None)
+            cut = next((i for i, t in enumerate(full.tokens) if t in sched.stop_token_ids), None)
             assert o.tokens == (full.tokens if cut is None else full.tokens[:cut + 1])
     assert eng.make_cache().num_free(0) == 32
 
