@@ -131,22 +131,31 @@ def main() -> int:
             sched.commit(bt, engine.step(bt))
         kv_start = sum(r.num_computed for r in sched.requests())
         sync()
-        t0 = time.perf_counter()
+        clock = time.perf_counter
+        t0 = clock()
         done = 0
+        in_schedule = in_commit = 0.0
         while done < steps:
+            t1 = clock()
             bt = sched.schedule_step(args.prompt_len, batch, min(args.decode_steps, steps - done))
             assert len(bt.work) == batch and bt.num_tokens == batch
-            sched.commit(bt, engine.step(bt))
+            t2 = clock()
+            sampled = engine.step(bt)
+            t3 = clock()
+            sched.commit(bt, sampled)
+            in_schedule += t2 - t1
+            in_commit += clock() - t3
             done += bt.decode_steps
         sync()
-        dt = time.perf_counter() - t0
+        dt = clock() - t0
         kv_end = sum(r.num_computed for r in sched.requests())
         for rid in [r.req_id for r in sched.requests()]:
             sched.free_request(rid)
         mean_kv_tokens = 0.5 * (kv_start + kv_end) + 0.5 * batch       # keys read per step, summed over requests
         bytes_per_step = weight_bytes + mean_kv_tokens * kv_bytes_per_token
         return {"tok_s": batch * steps / dt, "ms_per_step": 1e3 * dt / steps,
-                "gbs": bytes_per_step * steps / dt / 1e9, "kv_len": mean_kv_tokens / batch}
+                "gbs": bytes_per_step * steps / dt / 1e9, "kv_len": mean_kv_tokens / batch,
+                "schedule_us": 1e6 * in_schedule / steps, "commit_us": 1e6 * in_commit / steps}
 
     def prefill_run(reps: int = 5, warm: int = 2) -> dict:
         from prefixserve_amd.engine.batch import StepItem
@@ -212,6 +221,9 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": main_run["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": main_run["gbs"] / HBM_PEAK_GBS},
         "points": points,
+        # host time per decode step inside ms_per_step: the scheduler's two calls (the rest is
+        # engine.step: packing, the device's work, the wait for the tokens)
+        "host_us_per_step": {"schedule": main_run["schedule_us"], "commit": main_run["commit_us"]},
         "measured_peaks": peaks,
     }
     print(json.dumps(line), flush=True)

@@ -14,7 +14,7 @@ from prefixserve_amd.engine.scheduler import (AddResult, Batch, FinishReason, Re
 
 __all__ = [
     "BLOCK_SIZE", "AddResult", "Batch", "BlockManager", "CacheManager", "CoreError", "Engine", "EngineConfig",
-    "EngineError", "FinishReason", "LlamaEngine", "RadixTree", "ReqState", "Request", "Scheduler", "SchedulerError",
+    "EngineError", "FinishReason", "LlamaEngine", "LoopTimes", "RadixTree", "ReqState", "Request", "Scheduler", "SchedulerError",
     "SchedulerStats", "StateSlots", "StepItem", "StepResult", "WorkItem", "generate",
 ]
 
@@ -25,8 +25,8 @@ def __getattr__(name: str):
         from prefixserve_amd.engine import engine as _engine
 
         return getattr(_engine, name)
-    if name == "generate":
-        from prefixserve_amd.generation import generate as _generate
+    if name in ("generate", "LoopTimes"):
+        from prefixserve_amd import generation as _generation
 
-        return _generate
+        return getattr(_generation, name)
     raise AttributeError(f"module 'prefixserve_amd' has no attribute {name!r}")

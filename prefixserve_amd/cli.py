@@ -38,7 +38,7 @@ def _generate(args: argparse.Namespace) -> int:
     import numpy as np
 
     from prefixserve_amd.engine.engine import Engine, EngineConfig
-    from prefixserve_amd.generation import generate
+    from prefixserve_amd.generation import LoopTimes, generate
 
     cfg = EngineConfig(model_path=Path(args.model), dtype=args.dtype, max_num_seqs=args.max_running_requests,
                        max_prefill_tokens=args.chunked_prefill_size, max_seq_len=args.max_seq_len,
@@ -58,10 +58,12 @@ def _generate(args: argparse.Namespace) -> int:
         return 2
     sched = engine.make_scheduler(max_waiting=args.max_waiting, chunk_size=args.chunked_prefill_size,
                                   enable_prefix_cache=not args.disable_prefix_cache)
+    times = LoopTimes()
     t0 = time.perf_counter()
     outs, stats = generate(engine, prompts, args.max_tokens, temperature=args.temperature, seed=args.sample_seed,
                            ignore_eos=args.ignore_eos, scheduler=sched,
-                           max_prefill_tokens=args.chunked_prefill_size, max_running_requests=args.max_running_requests)
+                           max_prefill_tokens=args.chunked_prefill_size, max_running_requests=args.max_running_requests,
+                           times=times)
     dt = time.perf_counter() - t0
     new = sum(len(o.tokens) for o in outs)
     print(json.dumps({
@@ -70,7 +72,8 @@ def _generate(args: argparse.Namespace) -> int:
                      "cached_tokens": o.cached_tokens, "preemptions": o.preemptions} for o in outs],
         "stats": {"seconds": dt, "new_tokens": new, "tokens_per_second": new / dt if dt > 0 else None,
                   "prompt_tokens": stats.prompt_tokens, "cached_prompt_tokens": stats.cached_prompt_tokens,
-                  "prefix_hit_rate": stats.prefix_hit_rate, "preemptions": stats.preemptions},
+                  "prefix_hit_rate": stats.prefix_hit_rate, "preemptions": stats.preemptions,
+                  "loop": times.as_dict()},
     }))
     return 0
 

@@ -7,6 +7,7 @@ commit(batch, sampled)``.
 
 from __future__ import annotations
 
+import time
 from dataclasses import dataclass, field
 from typing import Iterable, Sequence
 
@@ -24,13 +25,38 @@ class Generation:
     preemptions: int = 0
 
 
+@dataclass
+class LoopTimes:
+    """Where the loop's time goes, summed over its steps: the same three intervals the
+    reference's serving loop keeps (prefixserve/server.py:104-115, 221-237). ``engine_s`` is
+    the whole of ``engine.step``: packing the step's arrays, the device's work and the wait
+    for the sampled tokens."""
+
+    steps: int = 0
+    schedule_s: float = 0.0
+    engine_s: float = 0.0
+    commit_s: float = 0.0
+
+    @property
+    def scheduler_overhead(self) -> float:
+        """schedule / (schedule + engine), the reference's "scheduler overhead" figure."""
+        both = self.schedule_s + self.engine_s
+        return self.schedule_s / both if both > 0 else 0.0
+
+    def as_dict(self) -> dict[str, float]:
+        return {"steps": self.steps, "schedule_s": self.schedule_s, "engine_s": self.engine_s,
+                "commit_s": self.commit_s, "scheduler_overhead": self.scheduler_overhead}
+
+
 def generate(engine: Engine, prompts: Sequence[Iterable[int]], max_tokens: int, *, temperature: float = 0.0,
              seed: int = 0, ignore_eos: bool = False, scheduler: Scheduler | None = None,
              max_prefill_tokens: int | None = None, max_running_requests: int | None = None,
-             enable_prefix_cache: bool = True, decode_steps: int | None = None) -> tuple[list[Generation], SchedulerStats]:
+             enable_prefix_cache: bool = True, decode_steps: int | None = None,
+             times: LoopTimes | None = None) -> tuple[list[Generation], SchedulerStats]:
     """Generates up to ``max_tokens`` tokens for every prompt (token ids in, token ids out).
     ``decode_steps``: how many decode steps a batch of decoding requests may run before the
-    host looks at the tokens (default: the engine configuration's)."""
+    host looks at the tokens (default: the engine configuration's). ``times``, if given, is
+    added to step by step."""
     steps = decode_steps if decode_steps is not None else engine.cfg.decode_steps
     budget = max_prefill_tokens if max_prefill_tokens is not None else engine.cfg.max_prefill_tokens
     running = max_running_requests if max_running_requests is not None else engine.cfg.max_num_seqs
@@ -46,13 +72,22 @@ def generate(engine: Engine, prompts: Sequence[Iterable[int]], max_tokens: int, 
         if res is not AddResult.ACCEPTED:
             raise ValueError(f"{rid} rejected: {res.value}")
         results[rid] = Generation(rid, ids)
+    clock = time.perf_counter
     while sched.has_work():
+        t0 = clock()
         batch = sched.schedule_step(budget, running, steps)
         if not batch.work:
             raise RuntimeError("the scheduler has work but could schedule none of it (pool too small?)")
         tracked = {w.req.req_id: w.req for w in batch.work}
+        t1 = clock()
         sampled = engine.step(batch)
+        t2 = clock()
         step = sched.commit(batch, sampled)
+        if times is not None:
+            times.steps += 1
+            times.schedule_s += t1 - t0
+            times.engine_s += t2 - t1
+            times.commit_s += clock() - t2
         for rid, toks in step.tokens.items():
             results[rid].tokens.extend(toks)
         for rid, why in step.finished.items():

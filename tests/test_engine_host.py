@@ -15,7 +15,7 @@ from prefixserve_amd.engine.batch import EngineError, GroupMeta, StepItem, StepP
 from prefixserve_amd.engine.engine import Engine, EngineConfig
 from prefixserve_amd.engine.replay import TraceReplayer
 from prefixserve_amd.engine.runner import ModelRunner
-from prefixserve_amd.generation import generate
+from prefixserve_amd.generation import LoopTimes, generate
 from prefixserve_amd.sampling import request_key, uniform_for
 
 
@@ -114,11 +114,14 @@ def test_scheduler_driven_greedy_generation_equals_plain(name, model_dirs, plain
     eng = Engine(EngineConfig(model_path=model_dirs[name], dtype="float32", device="cpu", max_num_seqs=4,
                               max_prefill_tokens=24, max_seq_len=256, num_blocks=11, use_graphs=False), ops=EmulatedOps())
     eng.capture_logits = True
-    outs, stats = generate(eng, prompts, new, ignore_eos=True)
+    times = LoopTimes()
+    outs, stats = generate(eng, prompts, new, ignore_eos=True, times=times)
     for p, o in zip(prompts, outs):
         want, _ = plain_models[name].greedy(p, new)
         assert o.tokens == want, f"prompt of {len(p)}: {o.tokens} != {want}"
     assert stats.preemptions > 0 and stats.cached_prompt_tokens > 0
+    assert times.steps >= new and min(times.schedule_s, times.engine_s, times.commit_s) > 0
+    assert 0 < times.scheduler_overhead < 1
     sched_cache = eng.make_cache()
     assert sched_cache.num_free(0) == 11
 
