@@ -4,6 +4,7 @@
 //   float everywhere it is the true 32-bit product of the exact path (plain v_fma_f32: no
 //   reduced-precision matrix mode is involved); it is also the fallback for shapes the
 //   bfloat16 kernels below refuse.
+// * rows_f32: the 32-bit product for up to 8 tokens (a wave per row of w), for decode steps.
 // * skinny_mfma: bfloat16 product for M <= 64 rows (decode steps and small portions). It is
 //   bound by reading w once from HBM, so each wave streams 16 rows of w through the
 //   16x16x32 matrix-core instruction with the M tokens as the other operand. Optional
@@ -73,6 +74,54 @@ static int launch_tiled(hipStream_t s, const void* x, const void* w, void* out, 
   dim3 grid(static_cast<unsigned>(ceil_div(N, 64)), static_cast<unsigned>(ceil_div(M, 64)));
   gemm_tiled_kernel<TX, TW, TO><<<grid, dim3(256), 0, s>>>(static_cast<const TX*>(x), static_cast<const TW*>(w),
                                                            static_cast<TO*>(out), M, N, K);
+  return check_launch("psamd_linear");
+}
+
+// ------------------------------------------------------------------ float32, a few tokens
+
+// The 32-bit product for up to MB tokens (decode steps): one wave per row of w, which it reads
+// once in 16-byte pieces; the tokens' rows come from the caches. Plain fused multiply-adds,
+// 4 partial sums per lane and token, summed over the lanes at the end. K % 4 == 0.
+template <int MB>
+__global__ __launch_bounds__(256) void rows_f32_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                       float* __restrict__ out, int M, int N, int K) {
+  const int lane = threadIdx.x & 63;
+  const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (n >= N) return;
+  const float* wr = w + static_cast<int64_t>(n) * K;
+  float4 acc[MB];
+#pragma unroll
+  for (int m = 0; m < MB; ++m) acc[m] = float4{0.f, 0.f, 0.f, 0.f};
+  for (int k = 4 * lane; k < K; k += 4 * kWave) {
+    const float4 wv = *reinterpret_cast<const float4*>(wr + k);
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+      if (m < M) {
+        const float4 xv = *reinterpret_cast<const float4*>(x + static_cast<int64_t>(m) * K + k);
+        acc[m].x = fmaf(xv.x, wv.x, acc[m].x);
+        acc[m].y = fmaf(xv.y, wv.y, acc[m].y);
+        acc[m].z = fmaf(xv.z, wv.z, acc[m].z);
+        acc[m].w = fmaf(xv.w, wv.w, acc[m].w);
+      }
+    }
+  }
+#pragma unroll
+  for (int m = 0; m < MB; ++m) {
+    const float sum = wave_sum((acc[m].x + acc[m].y) + (acc[m].z + acc[m].w));
+    if (lane == 0 && m < M) out[static_cast<int64_t>(m) * N + n] = sum;
+  }
+}
+
+static int launch_rows_f32(hipStream_t s, const void* x, const void* w, void* out, int M, int N, int K) {
+  const dim3 grid(static_cast<unsigned>(ceil_div(N, 4)));
+  const float* xf = static_cast<const float*>(x);
+  const float* wf = static_cast<const float*>(w);
+  float* of = static_cast<float*>(out);
+  if (M <= 2) {
+    rows_f32_kernel<2><<<grid, dim3(256), 0, s>>>(xf, wf, of, M, N, K);
+  } else {
+    rows_f32_kernel<8><<<grid, dim3(256), 0, s>>>(xf, wf, of, M, N, K);
+  }
   return check_launch("psamd_linear");
 }
 
@@ -446,7 +495,10 @@ int psamd_linear(void* stream, const void* x, int x_dtype, const void* w, int w_
   PSAMD_REQUIRE(ceil_div(M, 64) <= 65535, "too many rows for one launch");
   if (M == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (x_dtype == kF32 && w_dtype == kF32 && out_dtype == kF32) return launch_tiled<float, float, float>(s, x, w, out, M, N, K);
+  if (x_dtype == kF32 && w_dtype == kF32 && out_dtype == kF32) {
+    if (M <= 8 && K % 4 == 0) return launch_rows_f32(s, x, w, out, static_cast<int>(M), N, K);
+    return launch_tiled<float, float, float>(s, x, w, out, M, N, K);
+  }
   if (x_dtype == kBF16 && w_dtype == kBF16 && out_dtype == kBF16) return launch_tiled<bf16_t, bf16_t, bf16_t>(s, x, w, out, M, N, K);
   if (x_dtype == kBF16 && w_dtype == kBF16 && out_dtype == kF32) return launch_tiled<bf16_t, bf16_t, float>(s, x, w, out, M, N, K);
   return fail("psamd_linear: supported types are (f32,f32)->f32, (bf16,bf16)->bf16 and (bf16,bf16)->f32");

@@ -186,7 +186,8 @@ def test_fused_qkv_rope_append_equals_the_separate_kernels(ops, m, hq, hkv, d, k
 
 # --------------------------------------------------------------------- products
 
-@pytest.mark.parametrize("m,n,k", [(1, 100, 72), (3, 64, 16), (17, 257, 96), (130, 70, 200), (64, 128, 64)])
+@pytest.mark.parametrize("m,n,k", [(1, 100, 72), (3, 64, 16), (17, 257, 96), (130, 70, 200), (64, 128, 64),
+                                   (2, 7, 2048), (8, 1001, 1000), (9, 1001, 1000), (5, 33, 70), (8, 3, 4)])
 def test_linear_float32_is_exact_fp32(ops, m, n, k):
     x, w = rnd(m, k, seed=1), rnd(n, k, seed=2)
     out = torch.empty(m, n, device=DEV)
