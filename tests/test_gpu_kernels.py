@@ -207,6 +207,19 @@ def test_linear_bf16_small_m(ops, m, n, k, out_dtype):
     assert rel(out, want) < (1e-5 if out_dtype == torch.float32 else 5e-3)
 
 
+@pytest.mark.parametrize("m", [8, 9, 16, 31, 48, 64])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+def test_linear_bf16_very_many_columns(ops, m, out_dtype):
+    """The forms the output matrix takes from 9 tokens on (more row tiles per wave); a row count
+    that is no multiple of the largest group of tiles, a K with a partial last step."""
+    n, k = 65536 + 40, 72
+    x, w = rnd(m, k, dtype=torch.bfloat16, seed=1), rnd(n, k, dtype=torch.bfloat16, seed=2, scale=0.1)
+    out = torch.full((m + 1, n), 7.0, dtype=out_dtype, device=DEV)
+    ops.linear(x, w, out[:m])
+    assert rel(out[:m], x.double() @ w.double().T) < (1e-5 if out_dtype == torch.float32 else 5e-3)
+    assert torch.all(out[m] == 7.0)
+
+
 @pytest.mark.parametrize("m", [1, 8, 33, 64])
 @pytest.mark.parametrize("n,k", [(2048, 2048), (200, 8192), (72, 520), (256, 688)])
 def test_linear_to_residual_splits_k(ops, m, n, k):
