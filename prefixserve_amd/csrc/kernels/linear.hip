@@ -4,7 +4,7 @@
 //   float everywhere it is the true 32-bit product of the exact path (plain v_fma_f32: no
 //   reduced-precision matrix mode is involved); it is also the fallback for shapes the
 //   bfloat16 kernels below refuse.
-// * rows_f32: the 32-bit product for up to 8 tokens (a wave per row of w), for decode steps.
+// * rows_f32: the 32-bit product for up to 16 tokens (decode steps), in the tiled kernel's order of summation.
 // * skinny_mfma: bfloat16 product for M <= 64 rows (decode steps and small portions). It is
 //   bound by reading w once from HBM, so each wave streams 16 rows of w through the
 //   16x16x32 matrix-core instruction with the M tokens as the other operand. Optional
@@ -79,49 +79,53 @@ static int launch_tiled(hipStream_t s, const void* x, const void* w, void* out, 
 
 // ------------------------------------------------------------------ float32, a few tokens
 
-// The 32-bit product for up to MB tokens (decode steps): one wave per row of w, which it reads
-// once in 16-byte pieces; the tokens' rows come from the caches. Plain fused multiply-adds,
-// 4 partial sums per lane and token, summed over the lanes at the end. K % 4 == 0.
-template <int MB>
+// The 32-bit product for up to 16 tokens (decode steps), where the tiled kernel above would
+// leave most of its 64-token tile and most of the chip idle. A workgroup owns 16 rows of w;
+// thread (row, token) sums its products over k in ascending order with one fused multiply-add
+// each, exactly the order of the tiled kernel: a position's 32-bit result is the same bit for
+// bit whether its step had 1 token or 1,000, which is what lets tests of the 32-bit path
+// demand equality between different ways of cutting a sequence. The next 64-wide piece of
+// w and x is on its way from memory while the current one is summed from LDS. K % 4 == 0.
 __global__ __launch_bounds__(256) void rows_f32_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                        float* __restrict__ out, int M, int N, int K) {
-  const int lane = threadIdx.x & 63;
-  const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (n >= N) return;
-  const float* wr = w + static_cast<int64_t>(n) * K;
-  float4 acc[MB];
+  constexpr int BK = 64, LD = BK + 4;
+  __shared__ __align__(16) float ws[16][LD];
+  __shared__ __align__(16) float xs[16][LD];
+  const int tid = threadIdx.x;
+  const int r = tid & 15, m = tid >> 4;            // the output this thread sums
+  const int lr = tid >> 4, lc = (tid & 15) * 4;    // the 16-byte piece this thread brings in
+  const int n0 = blockIdx.x * 16;
+  const float4 zero = float4{0.f, 0.f, 0.f, 0.f};
+  const float* wsrc = w + static_cast<int64_t>(min(n0 + lr, N - 1)) * K + lc;
+  const float* xsrc = x + static_cast<int64_t>(min(lr, M - 1)) * K + lc;
+  float4 wv = lc < K ? *reinterpret_cast<const float4*>(wsrc) : zero;
+  float4 xv = lc < K ? *reinterpret_cast<const float4*>(xsrc) : zero;
+  float acc = 0.f;
+  for (int k0 = 0; k0 < K; k0 += BK) {
+    __syncthreads();                               // the previous piece has been summed
+    *reinterpret_cast<float4*>(&ws[lr][lc]) = wv;
+    *reinterpret_cast<float4*>(&xs[lr][lc]) = xv;
+    __syncthreads();
+    const int kn = k0 + BK + lc;
+    wv = kn < K ? *reinterpret_cast<const float4*>(wsrc + k0 + BK) : zero;
+    xv = kn < K ? *reinterpret_cast<const float4*>(xsrc + k0 + BK) : zero;
 #pragma unroll
-  for (int m = 0; m < MB; ++m) acc[m] = float4{0.f, 0.f, 0.f, 0.f};
-  for (int k = 4 * lane; k < K; k += 4 * kWave) {
-    const float4 wv = *reinterpret_cast<const float4*>(wr + k);
-#pragma unroll
-    for (int m = 0; m < MB; ++m) {
-      if (m < M) {
-        const float4 xv = *reinterpret_cast<const float4*>(x + static_cast<int64_t>(m) * K + k);
-        acc[m].x = fmaf(xv.x, wv.x, acc[m].x);
-        acc[m].y = fmaf(xv.y, wv.y, acc[m].y);
-        acc[m].z = fmaf(xv.z, wv.z, acc[m].z);
-        acc[m].w = fmaf(xv.w, wv.w, acc[m].w);
-      }
+    for (int kk = 0; kk < BK; kk += 4) {
+      const float4 a = *reinterpret_cast<const float4*>(&ws[r][kk]);
+      const float4 b = *reinterpret_cast<const float4*>(&xs[m][kk]);
+      acc = fmaf(b.x, a.x, acc);
+      acc = fmaf(b.y, a.y, acc);
+      acc = fmaf(b.z, a.z, acc);
+      acc = fmaf(b.w, a.w, acc);
     }
   }
-#pragma unroll
-  for (int m = 0; m < MB; ++m) {
-    const float sum = wave_sum((acc[m].x + acc[m].y) + (acc[m].z + acc[m].w));
-    if (lane == 0 && m < M) out[static_cast<int64_t>(m) * N + n] = sum;
-  }
+  if (m < M && n0 + r < N) out[static_cast<int64_t>(m) * N + n0 + r] = acc;
 }
 
 static int launch_rows_f32(hipStream_t s, const void* x, const void* w, void* out, int M, int N, int K) {
-  const dim3 grid(static_cast<unsigned>(ceil_div(N, 4)));
-  const float* xf = static_cast<const float*>(x);
-  const float* wf = static_cast<const float*>(w);
-  float* of = static_cast<float*>(out);
-  if (M <= 2) {
-    rows_f32_kernel<2><<<grid, dim3(256), 0, s>>>(xf, wf, of, M, N, K);
-  } else {
-    rows_f32_kernel<8><<<grid, dim3(256), 0, s>>>(xf, wf, of, M, N, K);
-  }
+  const dim3 grid(static_cast<unsigned>(ceil_div(N, 16)));
+  rows_f32_kernel<<<grid, dim3(256), 0, s>>>(static_cast<const float*>(x), static_cast<const float*>(w),
+                                             static_cast<float*>(out), M, N, K);
   return check_launch("psamd_linear");
 }
 
@@ -519,7 +523,8 @@ int psamd_linear(void* stream, const void* x, int x_dtype, const void* w, int w_
   if (M == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (x_dtype == kF32 && w_dtype == kF32 && out_dtype == kF32) {
-    if (M <= 8 && K % 4 == 0) return launch_rows_f32(s, x, w, out, static_cast<int>(M), N, K);
+    const bool aligned = (reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) % 16 == 0;
+    if (M <= 16 && K % 4 == 0 && aligned) return launch_rows_f32(s, x, w, out, static_cast<int>(M), N, K);
     return launch_tiled<float, float, float>(s, x, w, out, M, N, K);
   }
   if (x_dtype == kBF16 && w_dtype == kBF16 && out_dtype == kBF16) return launch_tiled<bf16_t, bf16_t, bf16_t>(s, x, w, out, M, N, K);

@@ -193,7 +193,21 @@ def test_linear_float32_is_exact_fp32(ops, m, n, k):
     out = torch.empty(m, n, device=DEV)
     ops.linear(x, w, out)
     want = (x.double() @ w.double().T)
-    assert rel(out, want) < 2e-6                                    # a reduced-precision mode would give ~1e-3
+    # One rounding per term, summed in order: the error grows like sqrt(k) * 2^-24. A
+    # reduced-precision mode would give ~1e-3.
+    assert rel(out, want) < max(2e-6, 1.2e-7 * k ** 0.5)
+
+
+@pytest.mark.parametrize("n,k", [(100, 72), (257, 2048), (33, 4), (3072, 200)])
+def test_linear_float32_does_not_depend_on_the_row_count(ops, n, k):
+    """The kernel for a few rows and the tiled kernel sum in one order: bit for bit the same."""
+    x, w = rnd(40, k, seed=1), rnd(n, k, seed=2)
+    big = torch.empty(40, n, device=DEV)
+    ops.linear(x, w, big)
+    for m in (1, 3, 16, 17):
+        small = torch.full((m + 1, n), 7.0, device=DEV)
+        ops.linear(x[:m], w, small[:m])
+        assert torch.equal(small[:m], big[:m]) and torch.all(small[m] == 7.0), f"{m} rows"
 
 
 @pytest.mark.parametrize("m", [1, 2, 7, 16, 17, 33, 64])
