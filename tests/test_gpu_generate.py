@@ -162,3 +162,48 @@ def test_several_decode_steps_before_the_host_reads(model_dirs, plain_models):
     many_t, _ = generate(eng, prompts, 23, temperature=0.7, ignore_eos=True)
     assert [o.tokens for o in one_t] == [o.tokens for o in many_t]
     assert [o.tokens for o in one_t] != [o.tokens for o in many]
+
+
+@pytest.mark.parametrize("seed", [0, 1])
+def test_random_workloads_through_the_scheduler(seed, model_dirs, plain_models):
+    """Random prompts, pools, budgets, running limits and decode steps per round, on a scheduler
+    that has served other requests with the same ids before: greedy tokens equal the plain
+    model's; sampled tokens equal those of a roomy engine that is never short of pages (in
+    32-bit a position's logits are the same bits however the work was cut, so the draws are)."""
+    from prefixserve_amd import Engine, EngineConfig, generate
+
+    rng = np.random.default_rng(100 + seed)
+    roomy = {}
+    preemptions = cached = 0
+    for _ in range(20):
+        name = str(rng.choice(list(TINY)))
+        vocab = TINY[name]["vocab_size"]
+        shared = rng.integers(3, vocab, int(rng.integers(0, 50))).tolist()
+        prompts = [(shared if rng.integers(0, 2) else []) + rng.integers(3, vocab, int(rng.integers(1, 60))).tolist()
+                   for _ in range(int(rng.integers(1, 7)))]
+        new = int(rng.integers(1, 30))
+        pages = -(-(max(len(p) for p in prompts) + new) // 16)
+        eng = Engine(EngineConfig(model_path=model_dirs[name], dtype="float32", max_num_seqs=int(rng.integers(1, 7)),
+                                  max_prefill_tokens=int(rng.choice([3, 8, 24, 64, 200])), max_seq_len=160,
+                                  num_blocks=int(rng.integers(pages + 1, 4 * pages + 4)),
+                                  decode_steps=int(rng.choice([1, 2, 4, 8])), sample_seed=int(rng.integers(0, 100))))
+        sched = eng.make_scheduler(chunk_size=eng.cfg.max_prefill_tokens, enable_prefix_cache=bool(rng.integers(0, 2)))
+        earlier = [rng.integers(3, vocab, int(rng.integers(1, 16 * pages - 3))).tolist() for _ in range(int(rng.integers(1, 5)))]
+        generate(eng, earlier, 3, ignore_eos=True, scheduler=sched)
+        temperature = float(rng.choice([0.0, 0.0, 0.9]))
+        outs, stats = generate(eng, prompts, new, temperature=temperature, ignore_eos=True, scheduler=sched)
+        preemptions += stats.preemptions
+        cached += stats.cached_prompt_tokens
+        if temperature == 0.0:
+            for p, o in zip(prompts, outs):
+                assert o.tokens == plain_models[name].greedy(p, new)[0], f"{name}, prompt of {len(p)}, {eng.cfg}"
+        else:
+            key = (name, eng.cfg.sample_seed)
+            if key not in roomy:
+                roomy[key] = Engine(EngineConfig(model_path=model_dirs[name], dtype="float32", max_num_seqs=8,
+                                                 max_prefill_tokens=256, max_seq_len=160, num_blocks=64,
+                                                 sample_seed=eng.cfg.sample_seed))
+            want, _ = generate(roomy[key], prompts, new, temperature=temperature, ignore_eos=True)
+            assert [o.tokens for o in outs] == [o.tokens for o in want], f"{name}, sampled, {eng.cfg}"
+        assert sched.cache.num_free(0) + sched.stats().cached_blocks == eng.cfg.num_blocks
+    assert preemptions > 0 and cached > 0
