@@ -37,6 +37,12 @@ int psamd_rope_kv_append(void* stream, void* qkv, int act_dtype, int64_t tokens,
 int psamd_linear(void* stream, const void* x, int x_dtype, const void* w, int w_dtype, void* out, int out_dtype,
                  int64_t M, int N, int K);
 
+// Library product (hipBLASLt, looked up at run time) for large bfloat16 steps, with the
+// descriptors and the chosen algorithm kept per shape. psamd_gemm_lt_available(): 1 if the
+// library is ready on the current device; its first call per device allocates the workspace.
+int psamd_gemm_lt_available();
+int psamd_gemm_lt(void* stream, const void* x, const void* w, void* out, int64_t M, int N, int K);
+
 // bfloat16 product for M <= 64 on the matrix cores. epilogue 1: w = [gate; up], out = silu(gate) * up.
 // ksplit > 1: out receives ksplit float32 partial sums [ksplit][M, n_out] (plain epilogue only).
 int psamd_linear_skinny_ksplit(int M, int n_out, int K);

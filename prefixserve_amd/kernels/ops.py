@@ -10,6 +10,7 @@ every 32-bit product and every product with at most 64 rows is a kernel of this 
 
 from __future__ import annotations
 
+import contextlib
 import ctypes
 from typing import Any
 
@@ -43,6 +44,7 @@ _SIGNATURES = {
     "psamd_swiglu": [_vp, _vp, _vp, _i32, _i64, _i32],
     "psamd_rope_kv_append": [_vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp, _vp, _vp, _vp],
     "psamd_linear": [_vp, _vp, _i32, _vp, _i32, _vp, _i32, _i64, _i32, _i32],
+    "psamd_gemm_lt": [_vp, _vp, _vp, _vp, _i64, _i32, _i32],
     "psamd_linear_skinny": [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32],
     "psamd_linear_skinny_ksplit": [_i32, _i32, _i32],
     "psamd_qkv_rope_append": [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp],
@@ -76,12 +78,31 @@ class HipOps:
         self.lib.psamd_sample_scratch_floats.restype = ctypes.c_int64
         self.ws = workspace
         self._sample_scratch: torch.Tensor | None = None
+        self._step_stream: int | None = None
+        # The library for large bfloat16 products, called directly if it can be (it sets itself up
+        # here, outside any capture); through torch.mm otherwise.
+        self.lib.psamd_gemm_lt_available.argtypes = []
+        with torch.cuda.device(self.device):
+            self._direct_library = bool(self.lib.psamd_gemm_lt_available())
         self.decode_split_kv_len: int | None = None   # fixed key length to size splits by (graph capture)
 
     # ---------------------------------------------------------------- helpers
 
     def _stream(self) -> int:
+        if self._step_stream is not None:
+            return self._step_stream
         return torch.cuda.current_stream(self.device).cuda_stream
+
+    @contextlib.contextmanager
+    def step_scope(self):
+        """All calls inside go to the stream that is current now: a step runs on one stream,
+        and asking torch for it costs as much as launching a small kernel."""
+        outer = self._step_stream
+        self._step_stream = torch.cuda.current_stream(self.device).cuda_stream
+        try:
+            yield
+        finally:
+            self._step_stream = outer
 
     def _ok(self, rc: int) -> None:
         if rc != 0:
@@ -200,7 +221,11 @@ class HipOps:
                                                           out[r0:r1].data_ptr(), _code(out.dtype), r1 - r0, n, k, 0, 1))
                 return
             if out.dtype == torch.bfloat16:
-                torch.matmul(x, w.t(), out=out)   # library product, as in the reference
+                # Library product, as in the reference.
+                if self._direct_library:
+                    self._ok(self.lib.psamd_gemm_lt(self._stream(), x.data_ptr(), w.data_ptr(), out.data_ptr(), m, n, k))
+                else:
+                    torch.matmul(x, w.t(), out=out)
                 return
         self._ok(self.lib.psamd_linear(self._stream(), x.data_ptr(), _code(x.dtype), w.data_ptr(), _code(w.dtype),
                                        out.data_ptr(), _code(out.dtype), m, n, k))

@@ -57,8 +57,13 @@ class Workspace:
         self.device = device
         self.version = 0
         self._bufs: dict[str, torch.Tensor] = {}
+        self._views: dict[tuple, torch.Tensor] = {}      # (name, shape, dtype) -> view handed out before
 
     def get(self, name: str, shape: tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
+        key = (name, tuple(shape), dtype)
+        view = self._views.get(key)
+        if view is not None:
+            return view
         n = 1
         for s in shape:
             n *= int(s)
@@ -68,7 +73,11 @@ class Workspace:
             buf = torch.empty(grow, dtype=dtype, device=self.device)
             self._bufs[name] = buf
             self.version += 1
-        return buf[:n].view(*shape)
+            self._views.clear()                          # views of the buffer this one replaces
+        if len(self._views) >= 2048:                     # every token count brings shapes of its own
+            self._views.clear()
+        view = self._views[key] = buf[:n].view(*shape)
+        return view
 
     def get_zeroed(self, name: str, shape: tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
         """Like ``get``, but the buffer is zero when first handed out or after it grew. Users

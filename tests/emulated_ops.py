@@ -9,6 +9,8 @@ the compiled kernels and a GPU the engine raises.
 
 from __future__ import annotations
 
+import contextlib
+
 import torch
 
 PAGE = 16
@@ -21,6 +23,9 @@ class EmulatedOps:
     def __init__(self, device: torch.device | str = "cpu", workspace=None) -> None:
         self.device = torch.device(device)
         self.ws = workspace
+
+    def step_scope(self):
+        return contextlib.nullcontext()
 
     def prepare_matrix(self, w: torch.Tensor, rt) -> torch.Tensor:
         return w.to(device=rt.device, dtype=rt.dtype).contiguous()

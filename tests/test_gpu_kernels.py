@@ -259,6 +259,26 @@ def test_linear_bf16_other_paths(ops, m, n, k):
         assert rel(out, x.double() @ w.double().T) < (2e-5 if out_dtype == torch.float32 else 5e-3)
 
 
+def test_library_product_called_directly_and_through_torch(ops):
+    """Large bfloat16 products go to hipBLASLt through the kernel library's own call (plans kept
+    per shape); torch.mm is what remains if the library cannot be found. Both against float64,
+    and a shape seen twice (the second call takes the kept plan)."""
+    assert ops._direct_library, "hipBLASLt was not found in the process"
+    for m, n, k in [(65, 300, 96), (512, 2048, 2048), (200, 64, 2048), (65, 300, 96)]:
+        x, w = rnd(m, k, dtype=torch.bfloat16, seed=1), rnd(n, k, dtype=torch.bfloat16, seed=2, scale=0.1)
+        want = x.double() @ w.double().T
+        direct = torch.full((m + 1, n), 7.0, dtype=torch.bfloat16, device=DEV)
+        ops.linear(x, w, direct[:m])
+        assert rel(direct[:m], want) < 5e-3 and torch.all(direct[m] == 7.0)
+        ops._direct_library = False
+        try:
+            through_torch = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+            ops.linear(x, w, through_torch)
+        finally:
+            ops._direct_library = True
+        assert rel(through_torch, want) < 5e-3
+
+
 @pytest.mark.parametrize("m", [1, 5, 64, 100])
 @pytest.mark.parametrize("act", [torch.float32, torch.bfloat16])
 def test_linear_swiglu(ops, m, act):
