@@ -5,6 +5,10 @@
 // which makes a step of a few hundred tokens host-bound. Here the descriptors and the chosen
 // algorithm are kept per (M, N, K), so that a call is one hipblasLtMatmul.
 //
+// use_workspace = 0 asks for an algorithm that needs no workspace: what a caller under stream
+// capture wants, since algorithms with a workspace may clear it with a memset, and memset nodes
+// of a captured graph are not to be relied on when the graph is replayed.
+//
 // The library is looked up at run time (the copy already in the process, which is torch's, else
 // the system's): nothing links against it, and if it or one of its entry points is missing
 // psamd_gemm_lt_available() says so and the caller keeps using torch.mm.
@@ -80,7 +84,7 @@ struct Plan {
 struct Device {
   hipblasLtHandle_t handle = nullptr;
   void* workspace = nullptr;
-  std::map<std::tuple<int64_t, int, int>, Plan> plans;
+  std::map<std::tuple<int64_t, int, int, bool>, Plan> plans;
 };
 
 std::mutex g_lock;
@@ -96,7 +100,7 @@ void drop(const Api& a, Plan& p) {
 
 // Row-major out[M, N] = x[M, K] * w[N, K]^T is, in the library's column-major terms,
 // C[N x M] = A^T * B with A = w seen as [K x N] (leading dimension K) and B = x seen as [K x M].
-int make_plan(const Api& a, Device& dev, int64_t M, int N, int K, Plan& p) {
+int make_plan(const Api& a, Device& dev, int64_t M, int N, int K, bool use_workspace, Plan& p) {
   const hipblasOperation_t trans = HIPBLAS_OP_T, none = HIPBLAS_OP_N;
   bool ok = a.desc_create(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F) == HIPBLAS_STATUS_SUCCESS &&
             a.desc_set(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &trans, sizeof(trans)) == HIPBLAS_STATUS_SUCCESS &&
@@ -106,12 +110,12 @@ int make_plan(const Api& a, Device& dev, int64_t M, int N, int K, Plan& p) {
             a.layout_create(&p.out, HIP_R_16BF, N, M, N) == HIPBLAS_STATUS_SUCCESS;
   hipblasLtMatmulPreference_t pref = nullptr;
   ok = ok && a.pref_create(&pref) == HIPBLAS_STATUS_SUCCESS;
-  const uint64_t room = kWorkspaceBytes;
+  const uint64_t room = use_workspace ? kWorkspaceBytes : 0;
   ok = ok && a.pref_set(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &room, sizeof(room)) == HIPBLAS_STATUS_SUCCESS;
   hipblasLtMatmulHeuristicResult_t found;
   int count = 0;
   ok = ok && a.heuristic(dev.handle, p.desc, p.w, p.x, p.out, p.out, pref, 1, &found, &count) == HIPBLAS_STATUS_SUCCESS &&
-       count > 0 && found.state == HIPBLAS_STATUS_SUCCESS && found.workspaceSize <= kWorkspaceBytes;
+       count > 0 && found.state == HIPBLAS_STATUS_SUCCESS && found.workspaceSize <= room;
   if (pref) a.pref_destroy(pref);
   if (!ok) {
     drop(a, p);
@@ -148,7 +152,7 @@ int psamd_gemm_lt_available() {
   return 1;
 }
 
-int psamd_gemm_lt(void* stream, const void* x, const void* w, void* out, int64_t M, int N, int K) {
+int psamd_gemm_lt(void* stream, const void* x, const void* w, void* out, int64_t M, int N, int K, int use_workspace) {
   PSAMD_REQUIRE(M > 0 && N > 0 && K > 0 && M <= INT32_MAX, "bad sizes");
   const Api& a = api();
   int id = 0;
@@ -156,7 +160,8 @@ int psamd_gemm_lt(void* stream, const void* x, const void* w, void* out, int64_t
   std::lock_guard<std::mutex> guard(g_lock);
   Device& dev = g_devices[id];
   PSAMD_REQUIRE(dev.handle != nullptr, "call psamd_gemm_lt_available() on this device first");
-  const auto key = std::make_tuple(M, N, K);
+  const bool roomy = use_workspace != 0;
+  const auto key = std::make_tuple(M, N, K, roomy);
   auto it = dev.plans.find(key);
   if (it == dev.plans.end()) {
     if (dev.plans.size() >= kMaxPlans) {
@@ -164,13 +169,14 @@ int psamd_gemm_lt(void* stream, const void* x, const void* w, void* out, int64_t
       dev.plans.clear();
     }
     Plan p;
-    if (const int rc = make_plan(a, dev, M, N, K, p)) return rc;
+    if (const int rc = make_plan(a, dev, M, N, K, roomy, p)) return rc;
     it = dev.plans.emplace(key, p).first;
   }
   const Plan& p = it->second;
   const float one = 1.f, zero = 0.f;
   const hipblasStatus_t st = a.matmul(dev.handle, p.desc, &one, w, p.w, x, p.x, &zero, out, p.out, out, p.out, &p.algo,
-                                      dev.workspace, kWorkspaceBytes, static_cast<hipStream_t>(stream));
+                                      roomy ? dev.workspace : nullptr, roomy ? kWorkspaceBytes : 0,
+                                      static_cast<hipStream_t>(stream));
   if (st != HIPBLAS_STATUS_SUCCESS) return fail("psamd_gemm_lt: hipblasLtMatmul returned " + std::to_string(st));
   return 0;
 }

@@ -6,7 +6,13 @@ the whole launch sequence is captured once per (batch size, wanted rows) and rep
 the step's integers are copied into the same device buffer at the same offsets (block
 tables padded to a fixed width), and the kernels read lengths and tables from there, so
 one graph serves every step of that shape. The number of key splits of the decode
-attention is fixed from ``max_seq_len`` so the grid does not depend on the step.
+attention is fixed from ``max_seq_len`` so the grid does not depend on the step, and a
+library product (a batch of more than 64 requests) is asked for an algorithm without a
+workspace, which has nothing to clear with a memset node.
+
+Steps with portions of prompts in them were captured by shape as well, as an experiment: the
+step times did not move (such steps are bound by their kernels, not by launches), so they run
+eagerly.
 
 The graph holds addresses of the packer's device buffer and of workspace buffers; if
 either is reallocated (their ``version`` changes) the graph is dropped and captured again.
@@ -37,8 +43,8 @@ def graphed_decode_step(runner: "ModelRunner", items: Sequence[StepItem], token_
         entry[0].replay()
         return entry[1]
 
-    previous = ops.decode_split_kv_len
-    ops.decode_split_kv_len = runner.max_seq_len
+    previous = ops.fixed_kv_len
+    ops.fixed_kv_len = runner.max_seq_len
     try:
         # An eager run first: it sizes every workspace buffer (and is this step's result if
         # capture is not possible). Then capture the same sequence and replay it.
@@ -54,4 +60,4 @@ def graphed_decode_step(runner: "ModelRunner", items: Sequence[StepItem], token_
         graph.replay()         # idempotent: same inputs, same cache writes as the eager run
         return captured
     finally:
-        ops.decode_split_kv_len = previous
+        ops.fixed_kv_len = previous

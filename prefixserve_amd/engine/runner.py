@@ -84,7 +84,10 @@ class ModelRunner:
         self.packer = StepPacker(
             self.device, [GroupMeta(nb, g.need.window) for g, nb in zip(self.layer_groups, blocks)],
             self.spec.vocab_size, self.max_seq_len, self.max_num_seqs, self.ops.PREFILL_TILE_Q)
-        self.use_graphs = bool(use_graphs) and self.device.type == "cuda"
+        # A model whose mixers keep state of their own runs eagerly: capturing a step runs it
+        # once before and once after the capture, which pages of keys and values do not mind
+        # and a state that is added to does.
+        self.use_graphs = bool(use_graphs) and self.device.type == "cuda" and not self.model.state_needs()
         self._graphs: dict[Any, Any] = {}
         logger.info("KV pools: %s blocks (%.2f GB)", blocks, self.pools.nbytes() / 1e9)
 

@@ -44,7 +44,7 @@ _SIGNATURES = {
     "psamd_swiglu": [_vp, _vp, _vp, _i32, _i64, _i32],
     "psamd_rope_kv_append": [_vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp, _vp, _vp, _vp],
     "psamd_linear": [_vp, _vp, _i32, _vp, _i32, _vp, _i32, _i64, _i32, _i32],
-    "psamd_gemm_lt": [_vp, _vp, _vp, _vp, _i64, _i32, _i32],
+    "psamd_gemm_lt": [_vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32],
     "psamd_linear_skinny": [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32],
     "psamd_linear_skinny_ksplit": [_i32, _i32, _i32],
     "psamd_qkv_rope_append": [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp],
@@ -84,7 +84,9 @@ class HipOps:
         self.lib.psamd_gemm_lt_available.argtypes = []
         with torch.cuda.device(self.device):
             self._direct_library = bool(self.lib.psamd_gemm_lt_available())
-        self.decode_split_kv_len: int | None = None   # fixed key length to size splits by (graph capture)
+        # Set while a step is run for, or under, graph capture: the key length that grids and
+        # LDS tables are sized by instead of the step's own, and no product with a workspace.
+        self.fixed_kv_len: int | None = None
 
     # ---------------------------------------------------------------- helpers
 
@@ -223,7 +225,8 @@ class HipOps:
             if out.dtype == torch.bfloat16:
                 # Library product, as in the reference.
                 if self._direct_library:
-                    self._ok(self.lib.psamd_gemm_lt(self._stream(), x.data_ptr(), w.data_ptr(), out.data_ptr(), m, n, k))
+                    self._ok(self.lib.psamd_gemm_lt(self._stream(), x.data_ptr(), w.data_ptr(), out.data_ptr(), m, n, k,
+                                                    0 if self.fixed_kv_len else 1))
                 else:
                     torch.matmul(x, w.t(), out=out)
                 return
@@ -283,10 +286,11 @@ class HipOps:
             if ctx.num_prefill_tiles:
                 self._ok(self.lib.psamd_attention_prefill(
                     s, qkv.data_ptr(), stride, out.data_ptr(), kv.data_ptr(), ctx.pf_tiles.data_ptr(),
-                    ctx.num_prefill_tiles, ctx.max_kv_len, ctx.item_start.data_ptr(), ctx.item_pos0.data_ptr(),
+                    ctx.num_prefill_tiles, self.fixed_kv_len or ctx.max_kv_len, ctx.item_start.data_ptr(),
+                    ctx.item_pos0.data_ptr(),
                     g.table_off.data_ptr(), g.block_ids.data_ptr(), hq, hkv, d, scale, win))
             if ctx.num_decode:
-                kv_len = self.decode_split_kv_len or ctx.max_kv_len
+                kv_len = self.fixed_kv_len or ctx.max_kv_len
                 if win:
                     kv_len = min(kv_len, win)
                 nsplit = max(1, min(64, 512 // (ctx.num_decode * hkv), -(-kv_len // 128)))
