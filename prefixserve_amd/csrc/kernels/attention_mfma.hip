@@ -281,7 +281,8 @@ __global__ __launch_bounds__(256 * KP) void attn_prefill_grouped_kernel(
     const bf16_t* __restrict__ qkv, int q_stride, bf16_t* __restrict__ out, const bf16_t* __restrict__ kv,
     const int32_t* __restrict__ pf_tiles, const int32_t* __restrict__ item_start,
     const int32_t* __restrict__ item_pos0, const int32_t* __restrict__ table_off,
-    const int32_t* __restrict__ block_ids, int n_tiles, int hq, int hkv, int table_pages, float scale, int window) {
+    const int32_t* __restrict__ block_ids, int n_tiles, int paired, int hq, int hkv, int table_pages, float scale,
+    int window) {
   constexpr int D = 16 * NS;
   constexpr int DT = (D + 31) / 32;
   constexpr int KS = D + 8;                      // elements per key row in LDS
@@ -304,10 +305,11 @@ __global__ __launch_bounds__(256 * KP) void attn_prefill_grouped_kernel(
   const int head_in_group = (blockIdx.y - kvh * wg_per_kv) * 4 + (wave & 3);
   const bool head_valid = head_in_group < group;       // a spare wave repeats the last head and writes nothing
   const int h = kvh * group + min(head_in_group, group - 1);
-  // A workgroup takes two tiles, one after the other: the b-th from the end and the b-th from
-  // the start. In a causal prompt the first sees the most keys and the second the fewest, so
-  // all workgroups get the same amount of work and none is left running alone at the end.
-  for (int phase = 0; phase < 2; ++phase) {
+  // With `paired`, a workgroup takes two tiles, one after the other: the b-th from the end and
+  // the b-th from the start. In a causal prompt the first sees the most keys and the second the
+  // fewest, so all workgroups get the same amount of work and none is left running alone at the
+  // end. Without, one tile each, the late ones first.
+  for (int phase = 0; phase < (paired ? 2 : 1); ++phase) {
   const int tile = phase == 0 ? n_tiles - 1 - static_cast<int>(blockIdx.x) : static_cast<int>(blockIdx.x);
   if (phase == 1) {
     if (tile >= n_tiles - 1 - static_cast<int>(blockIdx.x)) break;     // the middle tile is taken once
@@ -749,22 +751,47 @@ static bool lds_allowed(Kernel kernel, size_t bytes) {
                              static_cast<int>(bytes)) == hipSuccess;
 }
 
+// Which kernel a step's portions go to, when three or more query heads share a kv head
+// (measured at head sizes 64 and 128 on 256 compute units; us per layer, per-head / grouped
+// with one tile per workgroup / grouped with paired tiles):
+//   128 new tokens on 1,920 cached   16 / 30 / 56      512 on 1,536     29 / 31 / 52
+//   512 from position 0              12 / 12 / 16      1,024 from 0     31 / 19 / 24
+//   2,048 from position 0            87 / 62 / 39      4,096 from 0    255 / 162 / 128
+//  * few tiles: the per-head kernel, whose grid is four times as large, fills the chip best;
+//  * in between: the grouped kernel, one tile per workgroup;
+//  * two workgroups per compute unit or more AND little cached in front of the portions:
+//    paired tiles. Pairing evens out a causal triangle; on top of a long prefix every tile
+//    has much the same work and pairing only halves the number of workgroups.
+enum class PrefillForm { kPerHead, kGrouped, kGroupedPaired };
+
+static PrefillForm prefill_form(int n_tiles, int64_t prefix_tokens, int hq, int hkv) {
+  const int group = hq / hkv;
+  if (group < 3) return PrefillForm::kPerHead;
+  const int64_t workgroups = static_cast<int64_t>(n_tiles) * hkv * ((group + 3) / 4);
+  if (workgroups < 128) return PrefillForm::kPerHead;
+  if (workgroups >= 512 && 4 * prefix_tokens <= 32LL * n_tiles) return PrefillForm::kGroupedPaired;
+  return PrefillForm::kGrouped;
+}
+
 template <int NS>
 static int launch_prefill(hipStream_t s, const void* qkv, int q_stride, void* out, const void* kv,
-                          const int32_t* pf_tiles, int n_tiles, int table_pages, const int32_t* item_start, const int32_t* item_pos0,
+                          const int32_t* pf_tiles, int n_tiles, int64_t prefix_tokens, int table_pages,
+                          const int32_t* item_start, const int32_t* item_pos0,
                           const int32_t* table_off, const int32_t* block_ids, int hq, int hkv, float scale, int window) {
   const int group = hq / hkv;
-  // Three or more query heads per kv head: they share the keys and values through LDS, two
-  // waves per head (each its own run of keys) if the stages fit, else one.
-  if (group >= 3) {
-    const dim3 grid((n_tiles + 1) / 2, hkv * ((group + 3) / 4));
+  const PrefillForm form = prefill_form(n_tiles, prefix_tokens, hq, hkv);
+  // The heads of a kv head share its keys and values through LDS, two waves per head (each its
+  // own run of keys) if the stages fit, else one.
+  if (form != PrefillForm::kPerHead) {
+    const int paired = form == PrefillForm::kGroupedPaired ? 1 : 0;
+    const dim3 grid(paired ? (n_tiles + 1) / 2 : n_tiles, hkv * ((group + 3) / 4));
 #define PSAMD_GROUPED(KP_)                                                                                         \
   {                                                                                                               \
     const size_t smem = grouped_smem(16 * NS, 1, KP_, table_pages);                                               \
     if (lds_allowed(attn_prefill_grouped_kernel<NS, 1, KP_>, smem)) {                                             \
       attn_prefill_grouped_kernel<NS, 1, KP_><<<grid, dim3(256 * KP_), smem, s>>>(                                \
           static_cast<const bf16_t*>(qkv), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(kv),   \
-          pf_tiles, item_start, item_pos0, table_off, block_ids, n_tiles, hq, hkv, table_pages, scale, window);   \
+          pf_tiles, item_start, item_pos0, table_off, block_ids, n_tiles, paired, hq, hkv, table_pages, scale, window); \
       return check_launch("psamd_attention_prefill");                                                             \
     }                                                                                                             \
   }
@@ -827,8 +854,11 @@ int psamd_attention_mfma_supports(int hq, int hkv, int head_dim) {
 }
 
 // max_kv_len: the longest request of the step after it (sizes the block table staged in LDS).
+// prefix_tokens: tokens already cached in front of the portions, summed over them (with the
+// number of tiles it decides which form of the kernel runs).
 int psamd_attention_prefill(void* stream, const void* qkv, int q_stride, void* out, const void* kv,
-                            const int32_t* pf_tiles, int n_tiles, int max_kv_len, const int32_t* item_start,
+                            const int32_t* pf_tiles, int n_tiles, int max_kv_len, int64_t prefix_tokens,
+                            const int32_t* item_start,
                             const int32_t* item_pos0, const int32_t* table_off, const int32_t* block_ids, int hq,
                             int hkv, int head_dim, float scale, int window) {
   PSAMD_REQUIRE(psamd_attention_mfma_supports(hq, hkv, head_dim), "shape not supported by the matrix-core kernels");
@@ -838,8 +868,8 @@ int psamd_attention_prefill(void* stream, const void* qkv, int q_stride, void* o
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int table_pages = static_cast<int>(ceil_div(max_kv_len, kPage));
 #define PSAMD_PF(NS_)                                                                                           \
-  return launch_prefill<NS_>(s, qkv, q_stride, out, kv, pf_tiles, n_tiles, table_pages, item_start, item_pos0, \
-                             table_off, block_ids, hq, hkv, scale, window)
+  return launch_prefill<NS_>(s, qkv, q_stride, out, kv, pf_tiles, n_tiles, prefix_tokens, table_pages, item_start, \
+                             item_pos0, table_off, block_ids, hq, hkv, scale, window)
   switch (head_dim / 16) {
     case 1: PSAMD_PF(1);
     case 2: PSAMD_PF(2);

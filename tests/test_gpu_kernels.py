@@ -353,6 +353,26 @@ def test_paged_attention_mixed_batch(ops, act, hq, hkv, d):
     assert rel(got, want) < (2e-5 if act == torch.float32 else 2e-2)
 
 
+@pytest.mark.parametrize("hq,hkv,d,new,old,window", [
+    (32, 8, 64, [2048], [0], None),              # 512 workgroups, nothing cached: grouped, paired tiles
+    (24, 8, 128, [2100], [0], None),             # three heads per kv head, an odd number of tiles, a last tile of 20
+    (16, 4, 64, [2048, 2100], [0, 0], None),     # two prompts from position 0 in one step, paired
+    (32, 8, 64, [512], [1536], None),            # 128 workgroups on a long prefix: grouped, one tile each
+    (32, 8, 64, [2048, 3], [2048, 7], None),     # 512 workgroups but much cached: one tile each
+    (40, 2, 64, [500, 77], [100, 0], None),      # twenty heads per kv head: five workgroups per kv head
+    (6, 2, 256, [1500, 1000], [0, 200], None),   # head size 256
+    (16, 4, 64, [700, 300], [50, 0], 100),       # one tile each, with a window
+    (32, 8, 64, [2048], [0], 300),               # paired tiles, with a window
+    (32, 8, 64, [100], [1948], None),            # few tiles: the per-head kernel
+])
+def test_prefill_attention_in_each_form(ops, hq, hkv, d, new, old, window):
+    """The portions of a step go to one of three forms of the kernel by their number of tiles and
+    by how much is cached in front of them; each form at sizes that select it."""
+    pages = sum(-(-(n + o) // 16) for n, o in zip(new, old)) + 8
+    got, want = paged_case(ops, torch.bfloat16, hq, hkv, d, new, old, window=window, seed=len(new) + d, num_blocks=pages)
+    assert rel(got, want) < 2e-2
+
+
 @pytest.mark.parametrize("act", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("window", [1, 16, 33, 100])
 def test_paged_attention_window(ops, act, window):
