@@ -76,7 +76,7 @@ class Engine:
                        enable_prefix_cache: bool = True) -> Scheduler:
         return Scheduler(cache=self.make_cache(enable_prefix_cache), max_waiting=max_waiting,
                          chunk_size=chunk_size if chunk_size is not None else self.cfg.max_prefill_tokens,
-                         stop_token_ids=self.stop_token_ids)
+                         stop_token_ids=self.stop_token_ids, max_seq_len=self.cfg.max_seq_len)
 
     def _table_arrays(self, req) -> list:
         """The request's block tables as int64 arrays. A request's tables only grow while it
@@ -105,12 +105,26 @@ class Engine:
             out.append(arr[:n])
         return out
 
+    def _padded(self, work: list) -> list:
+        """A batch of decoding requests filled up to one of a few sizes (1, 2, 4, 8, then
+        multiples of 8) by repeating its last item, when steps are replayed as graphs: a batch
+        that loses one request at a time would otherwise meet a new shape, and a capture, at
+        every step. The repeated item computes what the original computes and writes the same
+        values to the same place; its row of the result is not looked at."""
+        n = len(work)
+        if not self.runner.use_graphs or n == 0:
+            return work
+        size = 1 << (n - 1).bit_length() if n <= 8 else -(-n // 8) * 8
+        size = min(size, self.cfg.max_num_seqs)
+        return work + [work[-1]] * (size - n) if size > n else work
+
     def _decode_steps(self, batch: Batch) -> dict[str, list[int]]:
         """``batch.decode_steps`` steps in a row for a batch of decoding requests. The token a
         step samples stays on the device and is the next step's input there; the host packs
         the next step's integers while the device runs the current one and waits once, at the
         end, for all tokens."""
-        k, reqs = batch.decode_steps, [w.req for w in batch.work]
+        k, work = batch.decode_steps, self._padded(batch.work)
+        reqs = [w.req for w in work]
         for w in batch.work:
             if w.start + k > self.cfg.max_seq_len:
                 raise EngineError(f"{w.req.req_id}: position {w.start + k} > max_seq_len {self.cfg.max_seq_len}")
@@ -119,11 +133,11 @@ class Engine:
                      if r.temperature > 0 else 0.0 for r in reqs] for j in range(k)]
         t_dev, u_dev, out_dev = self.sampler.stage_steps(temps, uniforms)
         tables = [self._table_arrays(r) for r in reqs]
-        first = [r.tokens(w.start, w.end) for r, w in zip(reqs, batch.work)]
+        first = [r.tokens(w.start, w.end) for r, w in zip(reqs, work)]
         for j in range(k):
             items = [StepItem(key=r.req_id, tokens=first[i] if j == 0 else (0,), start=w.start + j,
                               block_tables=tables[i], slot=max(r.slot, 0), want=(0,))
-                     for i, (r, w) in enumerate(zip(reqs, batch.work))]
+                     for i, (r, w) in enumerate(zip(reqs, work))]
             logits = self.runner.step(items, token_feed=out_dev[j - 1] if j else None)
             assert logits is not None
             self.sampler.sample_into(logits, t_dev, u_dev[j], out_dev[j])
@@ -139,8 +153,11 @@ class Engine:
             return self._decode_steps(batch)
         if len(batch.work) > self.cfg.max_num_seqs:
             raise EngineError(f"batch of {len(batch.work)} requests is over max_num_seqs {self.cfg.max_num_seqs}")
+        work = batch.work
+        if all(w.end - w.start == 1 and w.samples for w in work):
+            work = self._padded(work)
         items, sampling = [], []
-        for w in batch.work:
+        for w in work:
             req, n = w.req, w.end - w.start
             if w.end > self.cfg.max_seq_len:
                 raise EngineError(f"{req.req_id}: position {w.end} > max_seq_len {self.cfg.max_seq_len}")

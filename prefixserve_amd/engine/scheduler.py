@@ -80,7 +80,7 @@ class Scheduler:
     def __init__(self, num_blocks: int | Sequence[int] | None = None, *, max_waiting: int = 1024,
                  chunk_size: int = DEFAULT_CHUNK_SIZE, stop_token_ids: Iterable[int] = (),
                  enable_prefix_cache: bool = True, cache: CacheManager | None = None,
-                 num_slots: int = 1024) -> None:
+                 num_slots: int = 1024, max_seq_len: int | None = None) -> None:
         if chunk_size < 1 or max_waiting < 1:
             raise ValueError("chunk_size and max_waiting must be at least 1")
         if cache is None:
@@ -95,6 +95,9 @@ class Scheduler:
         self.chunk_size = int(chunk_size)
         self.max_waiting = int(max_waiting)
         self.stop_token_ids = frozenset(int(t) for t in stop_token_ids)
+        # The engine's limit on positions, if the scheduler is told: a round of several decode
+        # steps may then run past a request's max_tokens (see _decode_lookahead).
+        self.max_seq_len = None if max_seq_len is None else int(max_seq_len)
 
         self._live: dict[str, Request] = {}            # everything not finished, by id
         self._queue: deque[Request] = deque()          # waiting, next to start first
@@ -185,9 +188,9 @@ class Scheduler:
         """Decides the next step's work; ``commit`` of this batch must come before the next call.
 
         ``decode_steps`` > 1: if the batch holds only decoding requests and nobody waits, it
-        may run up to that many steps before the host sees the tokens (fewer if a request
-        would pass its ``max_tokens`` or the free pages do not reach that far; the pages are
-        taken now). A request that samples a stop token in between ends there and what was
+        may run up to that many steps before the host sees the tokens (fewer if no request has
+        that many tokens left or the free pages do not reach that far; the pages are taken
+        now). A request that samples a stop token in between ends there and what was
         computed for it afterwards is dropped."""
         if self._open is not None:
             raise SchedulerError("the previous batch has not been committed")
@@ -267,7 +270,16 @@ class Scheduler:
             return 1
         if any(item.end - item.start != 1 or not item.samples for item in plan.items):
             return 1
-        steps = min(wanted, min(item.req.max_tokens - len(item.req.output) for item in plan.items))
+        left = [item.req.max_tokens - len(item.req.output) for item in plan.items]
+        if self.max_seq_len is None:
+            steps = min(wanted, min(left))
+        else:
+            # Requests end at different times, so in a full batch somebody is always a step or
+            # two from max_tokens; cutting every round short for them would leave few rounds of
+            # full length. The round runs on for the others, and what it computes for a request
+            # past its last token is dropped at commit, as after a stop token. Positions stay
+            # inside what the engine can address.
+            steps = min(wanted, max(left), min(self.max_seq_len - item.start for item in plan.items))
         if steps <= 1:
             return 1
         for item in plan.items:

@@ -313,6 +313,34 @@ def test_several_decode_steps_in_one_batch():
         sched.commit(batch, {"a": [6, 7]})
 
 
+def test_a_round_of_decode_steps_runs_past_a_request_that_ends_in_it():
+    """Told the engine's position limit, the scheduler does not cut a round short for the request
+    nearest its max_tokens: that one ends in the middle and the rest of its tokens are dropped."""
+    sched = Scheduler(num_blocks=16, max_seq_len=64)
+    sched.add_request("a", ids(20), 3, ignore_eos=True)
+    sched.add_request("b", ids(30, 50), 30, ignore_eos=True)
+    first = sched.schedule_step(2048, 8, decode_steps=8)
+    sched.commit(first, {"a": 1, "b": 1})
+    batch = sched.schedule_step(2048, 8, decode_steps=8)
+    assert batch.decode_steps == 8                                   # a has two tokens left, b has 29
+    result = sched.commit(batch, {"a": list(range(10, 18)), "b": list(range(20, 28))})
+    assert result.tokens == {"a": [10, 11], "b": list(range(20, 28))} and result.finished == {"a": FinishReason.LENGTH}
+    assert sched.get_request("b").num_computed == 38
+    batch = sched.schedule_step(2048, 8, decode_steps=40)
+    assert batch.decode_steps == 21                                  # b's 21 tokens left: nobody needs more
+    sched.commit(batch, {"b": list(range(21))})
+    batch = sched.schedule_step(2048, 8, decode_steps=40)
+    assert batch.work == [] and not sched.has_work()
+    assert sched.block_manager.num_free + sched.stats().cached_blocks == 16
+    # positions stay below the limit
+    tight = Scheduler(num_blocks=16, max_seq_len=36)
+    tight.add_request("c", ids(30), 3, ignore_eos=True)
+    tight.add_request("d", ids(10), 20, ignore_eos=True)
+    first = tight.schedule_step(2048, 8, decode_steps=8)
+    tight.commit(first, {"c": 1, "d": 1})
+    assert tight.schedule_step(2048, 8, decode_steps=8).decode_steps == 6      # c stands at 30
+
+
 def test_decode_steps_fall_back_to_one():
     sim = Sim(4)                                                     # 64 positions in all
     sim.add("a", 30, max_tokens=20, ignore_eos=True)
