@@ -32,6 +32,8 @@ def _add_engine_options(p: argparse.ArgumentParser) -> None:
     p.add_argument("--no-graphs", action="store_true", help="do not capture decode steps as HIP graphs")
     p.add_argument("--decode-steps", type=int, default=1,
                    help="decode steps a batch of decoding requests runs before the host looks at the tokens")
+    p.add_argument("--warm-up", action="store_true",
+                   help="size buffers and capture the decode graphs before the first request (not timed)")
 
 
 def _generate(args: argparse.Namespace) -> int:
@@ -45,6 +47,8 @@ def _generate(args: argparse.Namespace) -> int:
                        num_blocks=args.num_blocks, use_graphs=not args.no_graphs, sample_seed=args.sample_seed,
                        decode_steps=args.decode_steps)
     engine = Engine(cfg)
+    if args.warm_up:
+        engine.warm_up()
     prompts: list[list[int]] = [[int(t) for t in s.split(",") if t.strip()] for s in (args.prompt_ids or [])]
     if args.prompt_len:
         rng = np.random.default_rng(args.seed)

@@ -14,7 +14,7 @@ import numpy as np
 import torch
 
 from prefixserve_amd.cache.manager import CacheManager
-from prefixserve_amd.engine.batch import EngineError, StepItem
+from prefixserve_amd.engine.batch import PAGE, EngineError, StepItem
 from prefixserve_amd.engine.runner import ModelRunner
 from prefixserve_amd.engine.scheduler import Batch, Scheduler
 from prefixserve_amd.sampling.sampler import Sampler, request_key, uniform_for
@@ -53,6 +53,7 @@ class Engine:
         # req_id -> (request, preemption count, [(array, filled)] per group): block tables as arrays,
         # extended as the lists grow, so a step does not convert whole lists again.
         self._tables: dict[str, tuple[Any, int, list[list]]] = {}
+        self._sizes = self._batch_sizes()
 
     @property
     def num_blocks(self) -> int:
@@ -105,6 +106,38 @@ class Engine:
             out.append(arr[:n])
         return out
 
+    def _batch_sizes(self) -> list[int]:
+        """The sizes decode batches are filled up to."""
+        top = self.cfg.max_num_seqs
+        sizes = [n for n in (1, 2, 4, 8) if n <= top] + list(range(16, top + 1, 8))
+        return sizes if sizes and sizes[-1] == top else sizes + [top]
+
+    def warm_up(self) -> None:
+        """Does before the first request what the first requests would otherwise pay for: the
+        largest step there can be (it sizes the buffers that steps share; a buffer that grows
+        later drops the captured graphs, which hold its address) and, if steps are replayed as
+        graphs, a capture of the decode step at every size batches are filled up to. The steps run on
+        token 0 and write into the first pages of every pool, which hold nothing anybody reads
+        before writing it. Call it before any request is running."""
+        r = self.runner
+        groups = r.num_blocks_per_group
+        n = min(self.cfg.max_prefill_tokens, self.cfg.max_seq_len, PAGE * min(groups))
+        one_page = [[0] for _ in groups]
+        # The largest step a scheduler can ask for: a portion of the whole budget beside
+        # decoding requests in all other places, every item wanting its logits.
+        items = [StepItem(key="warm-up", tokens=np.zeros(n, dtype=np.int32), start=0,
+                          block_tables=[list(range(-(-n // PAGE))) for _ in groups], slot=0, want=(n - 1,))]
+        items += [StepItem(key=f"warm-up-{i}", tokens=(0,), start=0, block_tables=one_page, slot=0, want=(0,))
+                  for i in range(self.cfg.max_num_seqs - 1)]
+        r.step(items)
+        if r.use_graphs:
+            for size in reversed(self._batch_sizes()):
+                items = [StepItem(key=f"warm-up-{i}", tokens=(0,), start=0, block_tables=one_page, slot=0, want=(0,))
+                         for i in range(size)]
+                r.step(items)
+        if r.device.type == "cuda":
+            torch.cuda.synchronize(r.device)
+
     def _padded(self, work: list) -> list:
         """A batch of decoding requests filled up to one of a few sizes (1, 2, 4, 8, then
         multiples of 8) by repeating its last item, when steps are replayed as graphs: a batch
@@ -114,8 +147,7 @@ class Engine:
         n = len(work)
         if not self.runner.use_graphs or n == 0:
             return work
-        size = 1 << (n - 1).bit_length() if n <= 8 else -(-n // 8) * 8
-        size = min(size, self.cfg.max_num_seqs)
+        size = next((s for s in self._sizes if s >= n), n)
         return work + [work[-1]] * (size - n) if size > n else work
 
     def _decode_steps(self, batch: Batch) -> dict[str, list[int]]:

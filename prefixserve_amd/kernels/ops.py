@@ -79,6 +79,7 @@ class HipOps:
         self.ws = workspace
         self._sample_scratch: torch.Tensor | None = None
         self._step_stream: int | None = None
+        self._slice_views: dict[tuple, tuple] = {}      # (name, slices, rows) -> (buffer, its [slices, rows, N] view)
         # The library for large bfloat16 products, called directly if it can be (it sets itself up
         # here, outside any capture); through torch.mm otherwise.
         self.lib.psamd_gemm_lt_available.argtypes = []
@@ -244,7 +245,13 @@ class HipOps:
             ksplit = self.lib.psamd_linear_skinny_ksplit(m, n, k)
             if ksplit > 1:
                 self._need(w.shape[1] == k and x.is_contiguous() and w.is_contiguous(), "linear_to_residual: operands")
-                out = self.ws.get(name, (ksplit, m, n), torch.float32)
+                # Room for the most slices of the most rows, so that the buffer never grows.
+                self._need(ksplit <= 8, "linear_to_residual: more slices than there is room for")
+                room = self.ws.get(name + ".slices", (8 * self.SKINNY_MAX_ROWS * n,), torch.float32)
+                kept = self._slice_views.get((name, ksplit, m))
+                if kept is None or kept[0] is not room:
+                    kept = self._slice_views[(name, ksplit, m)] = (room, room[:ksplit * m * n].view(ksplit, m, n))
+                out = kept[1]
                 self._ok(self.lib.psamd_linear_skinny(self._stream(), x.data_ptr(), w.data_ptr(), out.data_ptr(),
                                                       _F32, m, n, k, 0, ksplit))
                 return out
@@ -294,8 +301,11 @@ class HipOps:
                 if win:
                     kv_len = min(kv_len, win)
                 nsplit = max(1, min(64, 512 // (ctx.num_decode * hkv), -(-kv_len // 128)))
-                part_o = self.ws.get("attn.part_o", (ctx.num_decode * hq * nsplit * d,), torch.float32)
-                part_ml = self.ws.get("attn.part_ml", (ctx.num_decode * hq * nsplit * 2,), torch.float32)
+                # (requests x splits) is at most 512 / hkv unless there are more requests than
+                # that: asked for at that size, the buffers do not grow from step to step.
+                parts = max(ctx.num_decode * nsplit, 512 // hkv)
+                part_o = self.ws.get("attn.part_o", (parts * hq * d,), torch.float32)
+                part_ml = self.ws.get("attn.part_ml", (parts * hq * 2,), torch.float32)
                 self._ok(self.lib.psamd_attention_decode(
                     s, qkv.data_ptr(), stride, out.data_ptr(), kv.data_ptr(), part_o.data_ptr(), part_ml.data_ptr(),
                     ctx.dec_items.data_ptr(), ctx.num_decode, ctx.item_start.data_ptr(),

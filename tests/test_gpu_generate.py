@@ -207,3 +207,24 @@ def test_random_workloads_through_the_scheduler(seed, model_dirs, plain_models):
             assert [o.tokens for o in outs] == [o.tokens for o in want], f"{name}, sampled, {eng.cfg}"
         assert sched.cache.num_free(0) + sched.stats().cached_blocks == eng.cfg.num_blocks
     assert preemptions > 0 and cached > 0
+
+
+def test_warm_up_then_generation(model_dirs, plain_models):
+    """After warm_up every decode batch size has its graph and the shared buffers their final
+    size: generation captures nothing more, and its tokens are the plain model's (what the
+    warm-up steps wrote into the first pages is never read)."""
+    from prefixserve_amd import Engine, EngineConfig, generate
+
+    name = "B"
+    eng = Engine(EngineConfig(model_path=model_dirs[name], dtype="float32", max_num_seqs=12, max_prefill_tokens=64,
+                              max_seq_len=128, num_blocks=40, decode_steps=3))
+    eng.warm_up()
+    captured = set(eng.runner._graphs)
+    assert {shape[0] for shape in captured} == {1, 2, 4, 8, 12}
+    version = eng.runner.workspace.version
+    rng = np.random.default_rng(8)
+    prompts = [rng.integers(3, 512, n).tolist() for n in (33, 5, 18, 47, 60, 9, 21)]
+    outs, _ = generate(eng, prompts, 14, ignore_eos=True)
+    for p, o in zip(prompts, outs):
+        assert o.tokens == plain_models[name].greedy(p, 14)[0]
+    assert set(eng.runner._graphs) == captured and eng.runner.workspace.version == version
