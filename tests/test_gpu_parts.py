@@ -4,7 +4,6 @@ registered, built into a model and stepped without touching the package's files.
 
 from __future__ import annotations
 
-import math
 
 import numpy as np
 import pytest

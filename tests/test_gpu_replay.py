@@ -14,7 +14,6 @@ from pathlib import Path
 
 import numpy as np
 import pytest
-import torch
 
 import traces
 from configs import TINY, TOL_BF16, TOL_F32

@@ -7,7 +7,6 @@ from __future__ import annotations
 import math
 
 import numpy as np
-import pytest
 import torch
 
 from plain import llama_plain as P
