@@ -347,6 +347,18 @@ static int launch_skinny1(hipStream_t s, const void* x, const void* w, void* out
       return check_launch("psamd_linear_skinny");
     }
   }
+  if constexpr (SWIGLU) {
+    // A wide feed-forward (896 tiles of gate/up pairs at an intermediate size of 14,336) has
+    // workgroups to spare at four pairs of tiles per wave, and the tokens are then read half as
+    // often: 66 -> 56 us at 32 tokens, 78 -> 65 at 64. At 8,192 (512 tiles) it would leave half
+    // the compute units idle, and two pairs stay the best.
+    if (M > 8 && ceil_div(n_out, 16) >= 4 * 200) {
+      const dim3 grid(static_cast<unsigned>(ceil_div(ceil_div(n_out, 16), 4)), 1u), block(64 * 8);
+      skinny_mfma_kernel<MT, 4, 8, true, true, bf16_t, 1><<<grid, block, 0, s>>>(
+          static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), M, n_out, K);
+      return check_launch("psamd_linear_skinny");
+    }
+  }
   constexpr int RT = skinny_rt(MT, SWIGLU), WV = skinny_wv(MT);
   // Enough row groups to fill the chip with one wave each: no need to split K inside a workgroup.
   if (ceil_div(ceil_div(n_out, 16), RT) >= 2048)
@@ -494,18 +506,19 @@ __global__ __launch_bounds__(64 * WV) void qkv_rope_append_kernel(
 }
 
 // One tile per workgroup keeps the most workgroups, and K cannot be split over workgroups
-// here (the rotation needs whole sums); two tiles halve the traffic for the tokens once there
-// are many tokens and still enough workgroups for every compute unit.
+// here (the rotation needs whole sums); two tiles halve the traffic for the tokens, which pays
+// from 9 tokens on where 320 tiles or more leave every compute unit a workgroup (at 384 tiles
+// and K = 4,096: 28 -> 22 us at 32 tokens, 45 -> 31 at 64; at 192 tiles one tile stays the
+// best). Eight waves per workgroup beat four at every size tried.
 template <int MT>
 static void launch_qkv(hipStream_t s, const bf16_t* x, const bf16_t* w, bf16_t* out, int M, int K, int hq, int hkv, int d,
                        const int32_t* positions, const float2* table, bf16_t* kv, const int32_t* write_slot) {
   const int n_tiles = (hq + 2 * hkv) * (d / 16);
-  if (MT >= 3 && n_tiles >= 384) {
-    constexpr int RT = MT >= 3 ? 2 : 1;
-    qkv_rope_append_kernel<MT, RT, 4><<<dim3(static_cast<unsigned>(ceil_div(n_tiles, RT))), dim3(256), 0, s>>>(
+  if (M > 8 && n_tiles >= 320) {
+    qkv_rope_append_kernel<MT, 2, 8><<<dim3(static_cast<unsigned>(ceil_div(n_tiles, 2))), dim3(512), 0, s>>>(
         x, w, out, M, K, hq, hkv, d, positions, table, kv, write_slot);
   } else {
-    qkv_rope_append_kernel<MT, 1, 4><<<dim3(static_cast<unsigned>(n_tiles)), dim3(256), 0, s>>>(
+    qkv_rope_append_kernel<MT, 1, 8><<<dim3(static_cast<unsigned>(n_tiles)), dim3(512), 0, s>>>(
         x, w, out, M, K, hq, hkv, d, positions, table, kv, write_slot);
   }
 }

@@ -291,6 +291,20 @@ def test_linear_swiglu(ops, m, act):
     assert rel(out, want) < (2e-6 if act == torch.float32 else 1e-2)
 
 
+@pytest.mark.parametrize("m", [8, 9, 16, 31, 48, 64])
+def test_linear_swiglu_wide(ops, m):
+    """An intermediate size with 800 or more tiles of gate/up pairs takes four pairs per wave from
+    9 tokens on; a size that is no multiple of the 64 rows of such a group, a K with a partial
+    last step."""
+    k, inter = 72, 12800 + 40
+    x, w = rnd(m, k, dtype=torch.bfloat16, seed=1), rnd(2 * inter, k, dtype=torch.bfloat16, seed=2, scale=0.2)
+    out = torch.full((m + 1, inter), 7.0, dtype=torch.bfloat16, device=DEV)
+    ops.linear_swiglu(x, w, out[:m])
+    gu = x.double() @ w.double().T
+    want = torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:]
+    assert rel(out[:m], want) < 1e-2 and torch.all(out[m] == 7.0)
+
+
 # -------------------------------------------------------------------- attention
 
 def paged_case(ops, act, hq, hkv, d, lens_new, lens_old, window=None, seed=0, num_blocks=64, poison=1e30):
