@@ -553,7 +553,10 @@ int psamd_linear_skinny_ksplit(int M, int n_out, int K) {
   const int64_t groups = ceil_div(ceil_div(n_out, 16), skinny_rt(mt, false));
   const int64_t steps = ceil_div(K, 32);
   // Up to 32 tokens a wave keeps at least two k-steps; above, one is enough (measured).
-  const int64_t split = std::min<int64_t>({8, 512 / std::max<int64_t>(groups, 1), steps / ((mt <= 2 ? 2 : 1) * skinny_wv(mt))});
+  // Workgroups of 4 waves: two per compute unit; of 8 waves: one (4,096 x 4,096 at 64 tokens:
+  // 16.2 us with 8 slices, 14.3 with 4).
+  const int64_t wanted = skinny_wv(mt) == 8 ? 256 : 512;
+  const int64_t split = std::min<int64_t>({8, wanted / std::max<int64_t>(groups, 1), steps / ((mt <= 2 ? 2 : 1) * skinny_wv(mt))});
   return static_cast<int>(std::max<int64_t>(split, 1));
 }
 
