@@ -292,11 +292,12 @@ def test_linear_swiglu(ops, m, act):
 
 
 @pytest.mark.parametrize("m", [8, 9, 16, 31, 48, 64])
-def test_linear_swiglu_wide(ops, m):
+@pytest.mark.parametrize("inter", [12800 + 40, 6400 + 40])
+def test_linear_swiglu_wide(ops, m, inter):
     """An intermediate size with 800 or more tiles of gate/up pairs takes four pairs per wave from
-    9 tokens on; a size that is no multiple of the 64 rows of such a group, a K with a partial
-    last step."""
-    k, inter = 72, 12800 + 40
+    9 tokens on, one with 400 or more two pairs at 9 to 16 tokens; sizes that are no multiple of
+    the rows of such a group, a K with a partial last step."""
+    k = 72
     x, w = rnd(m, k, dtype=torch.bfloat16, seed=1), rnd(2 * inter, k, dtype=torch.bfloat16, seed=2, scale=0.2)
     out = torch.full((m + 1, inter), 7.0, dtype=torch.bfloat16, device=DEV)
     ops.linear_swiglu(x, w, out[:m])
