@@ -41,8 +41,10 @@ int psamd_linear(void* stream, const void* x, int x_dtype, const void* w, int w_
 // descriptors and the chosen algorithm kept per shape. psamd_gemm_lt_available(): 1 if the
 // library is ready on the current device; its first call per device allocates the workspace.
 // use_workspace = 0: only algorithms that need none (for calls under stream capture).
+// psamd_gemm_lt returns 2, not an error, if the library has no algorithm for the shape.
 int psamd_gemm_lt_available();
-int psamd_gemm_lt(void* stream, const void* x, const void* w, void* out, int64_t M, int N, int K, int use_workspace);
+int psamd_gemm_lt(void* stream, const void* x, const void* w, void* out, int out_dtype, int64_t M, int N, int K,
+                  int use_workspace);
 
 // bfloat16 product for M <= 64 on the matrix cores. epilogue 1: w = [gate; up], out = silu(gate) * up.
 // ksplit > 1: out receives ksplit float32 partial sums [ksplit][M, n_out] (plain epilogue only).

@@ -1,10 +1,12 @@
-// The library product for large bfloat16 steps: out[M, N] = x[M, K] * w[N, K]^T through
-// hipBLASLt, called directly. The reference's engine calls a library for these products too
+// The library product for large bfloat16 steps: out[M, N] = x[M, K] * w[N, K]^T (out bfloat16,
+// or float32 for logits) through hipBLASLt, called directly. The reference's engine calls a library for these products too
 // (torch.nn.functional.linear, prefixserve/model/llama.py:113-121); going through torch.mm costs
 // 18 us of host time per call (descriptors and the heuristic search are redone every time),
 // which makes a step of a few hundred tokens host-bound. Here the descriptors and the chosen
 // algorithm are kept per (M, N, K), so that a call is one hipblasLtMatmul.
 //
+// Returns 0, 1 for an error, or 2 if the library has no algorithm for the shape under the
+// given conditions (the caller then takes another path).
 // use_workspace = 0 asks for an algorithm that needs no workspace: what a caller under stream
 // capture wants, since algorithms with a workspace may clear it with a memset, and memset nodes
 // of a captured graph are not to be relied on when the graph is replayed.
@@ -84,7 +86,7 @@ struct Plan {
 struct Device {
   hipblasLtHandle_t handle = nullptr;
   void* workspace = nullptr;
-  std::map<std::tuple<int64_t, int, int, bool>, Plan> plans;
+  std::map<std::tuple<int64_t, int, int, bool, bool>, Plan> plans;
 };
 
 std::mutex g_lock;
@@ -100,14 +102,14 @@ void drop(const Api& a, Plan& p) {
 
 // Row-major out[M, N] = x[M, K] * w[N, K]^T is, in the library's column-major terms,
 // C[N x M] = A^T * B with A = w seen as [K x N] (leading dimension K) and B = x seen as [K x M].
-int make_plan(const Api& a, Device& dev, int64_t M, int N, int K, bool use_workspace, Plan& p) {
+int make_plan(const Api& a, Device& dev, int64_t M, int N, int K, bool use_workspace, bool float_out, Plan& p) {
   const hipblasOperation_t trans = HIPBLAS_OP_T, none = HIPBLAS_OP_N;
   bool ok = a.desc_create(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F) == HIPBLAS_STATUS_SUCCESS &&
             a.desc_set(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &trans, sizeof(trans)) == HIPBLAS_STATUS_SUCCESS &&
             a.desc_set(p.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &none, sizeof(none)) == HIPBLAS_STATUS_SUCCESS &&
             a.layout_create(&p.w, HIP_R_16BF, K, N, K) == HIPBLAS_STATUS_SUCCESS &&
             a.layout_create(&p.x, HIP_R_16BF, K, M, K) == HIPBLAS_STATUS_SUCCESS &&
-            a.layout_create(&p.out, HIP_R_16BF, N, M, N) == HIPBLAS_STATUS_SUCCESS;
+            a.layout_create(&p.out, float_out ? HIP_R_32F : HIP_R_16BF, N, M, N) == HIPBLAS_STATUS_SUCCESS;
   hipblasLtMatmulPreference_t pref = nullptr;
   ok = ok && a.pref_create(&pref) == HIPBLAS_STATUS_SUCCESS;
   const uint64_t room = use_workspace ? kWorkspaceBytes : 0;
@@ -152,8 +154,11 @@ int psamd_gemm_lt_available() {
   return 1;
 }
 
-int psamd_gemm_lt(void* stream, const void* x, const void* w, void* out, int64_t M, int N, int K, int use_workspace) {
+int psamd_gemm_lt(void* stream, const void* x, const void* w, void* out, int out_dtype, int64_t M, int N, int K,
+                  int use_workspace) {
   PSAMD_REQUIRE(M > 0 && N > 0 && K > 0 && M <= INT32_MAX, "bad sizes");
+  PSAMD_REQUIRE(out_dtype == kBF16 || out_dtype == kF32, "the output is bfloat16 or float32");
+  const bool float_out = out_dtype == kF32;
   const Api& a = api();
   int id = 0;
   PSAMD_REQUIRE(a.ok && hipGetDevice(&id) == hipSuccess && id >= 0 && id < kMaxDevices, "hipBLASLt is not available");
@@ -161,7 +166,7 @@ int psamd_gemm_lt(void* stream, const void* x, const void* w, void* out, int64_t
   Device& dev = g_devices[id];
   PSAMD_REQUIRE(dev.handle != nullptr, "call psamd_gemm_lt_available() on this device first");
   const bool roomy = use_workspace != 0;
-  const auto key = std::make_tuple(M, N, K, roomy);
+  const auto key = std::make_tuple(M, N, K, roomy, float_out);
   auto it = dev.plans.find(key);
   if (it == dev.plans.end()) {
     if (dev.plans.size() >= kMaxPlans) {
@@ -169,10 +174,11 @@ int psamd_gemm_lt(void* stream, const void* x, const void* w, void* out, int64_t
       dev.plans.clear();
     }
     Plan p;
-    if (const int rc = make_plan(a, dev, M, N, K, roomy, p)) return rc;
+    make_plan(a, dev, M, N, K, roomy, float_out, p);      // on failure p stays empty, and is kept: the answer will not change
     it = dev.plans.emplace(key, p).first;
   }
   const Plan& p = it->second;
+  if (p.desc == nullptr) return 2;                         // the message of make_plan is the last error
   const float one = 1.f, zero = 0.f;
   const hipblasStatus_t st = a.matmul(dev.handle, p.desc, &one, w, p.w, x, p.x, &zero, out, p.out, out, p.out, &p.algo,
                                       roomy ? dev.workspace : nullptr, roomy ? kWorkspaceBytes : 0,

@@ -44,7 +44,7 @@ _SIGNATURES = {
     "psamd_swiglu": [_vp, _vp, _vp, _i32, _i64, _i32],
     "psamd_rope_kv_append": [_vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp, _vp, _vp, _vp],
     "psamd_linear": [_vp, _vp, _i32, _vp, _i32, _vp, _i32, _i64, _i32, _i32],
-    "psamd_gemm_lt": [_vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32],
+    "psamd_gemm_lt": [_vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32],
     "psamd_linear_skinny": [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32],
     "psamd_linear_skinny_ksplit": [_i32, _i32, _i32],
     "psamd_qkv_rope_append": [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp],
@@ -215,21 +215,21 @@ class HipOps:
         if m == 0:
             return
         if x.dtype == torch.bfloat16 and k % 8 == 0:
+            if m > self.SKINNY_MAX_ROWS and self._direct_library:
+                # Library product, as in the reference (float32 output for more than 64 rows of logits).
+                rc = self.lib.psamd_gemm_lt(self._stream(), x.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out.dtype),
+                                            m, n, k, 0 if self.fixed_kv_len else 1)
+                if rc != 2:                      # 2: no algorithm for this shape (without a workspace): the paths below
+                    self._ok(rc)
+                    return
             if m <= self.SKINNY_MAX_ROWS or out.dtype == torch.float32:
-                # Logits (float32 output) always come from this kernel, whatever the row
-                # count, so that a position's logits do not depend on how the step was cut.
                 for r0 in range(0, m, self.SKINNY_MAX_ROWS):
                     r1 = min(m, r0 + self.SKINNY_MAX_ROWS)
                     self._ok(self.lib.psamd_linear_skinny(self._stream(), x[r0:r1].data_ptr(), w.data_ptr(),
                                                           out[r0:r1].data_ptr(), _code(out.dtype), r1 - r0, n, k, 0, 1))
                 return
             if out.dtype == torch.bfloat16:
-                # Library product, as in the reference.
-                if self._direct_library:
-                    self._ok(self.lib.psamd_gemm_lt(self._stream(), x.data_ptr(), w.data_ptr(), out.data_ptr(), m, n, k,
-                                                    0 if self.fixed_kv_len else 1))
-                else:
-                    torch.matmul(x, w.t(), out=out)
+                torch.matmul(x, w.t(), out=out)
                 return
         self._ok(self.lib.psamd_linear(self._stream(), x.data_ptr(), _code(x.dtype), w.data_ptr(), _code(w.dtype),
                                        out.data_ptr(), _code(out.dtype), m, n, k))

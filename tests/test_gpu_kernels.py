@@ -277,6 +277,14 @@ def test_library_product_called_directly_and_through_torch(ops):
         finally:
             ops._direct_library = True
         assert rel(through_torch, want) < 5e-3
+        for through_library in (True, False):                         # float32 out: more than 64 rows of logits
+            ops._direct_library = through_library
+            try:
+                logits = torch.full((m + 1, n), 7.0, dtype=torch.float32, device=DEV)
+                ops.linear(x, w, logits[:m])
+            finally:
+                ops._direct_library = True
+            assert rel(logits[:m], want) < 2e-5 and torch.all(logits[m] == 7.0)
 
 
 @pytest.mark.parametrize("m", [1, 5, 64, 100])
