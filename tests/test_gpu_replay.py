@@ -121,6 +121,36 @@ def test_graph_replay_equals_eager_decoding(model_dirs):
     assert np.array_equal(out[False], out[True])
 
 
+def test_graph_replay_with_library_products(model_dirs):
+    """Seventy requests decoding together: more than 64 rows, so the products of the captured
+    step are the library's (asked for algorithms without a workspace, which clear nothing with
+    memset nodes). Every replay against the same step launched one by one, with other work
+    between the replays."""
+    n_req, steps = 70, 10
+    reqs = requests_for("C", [40] * n_req, seed=13)
+    out = {}
+    for graphs in (False, True):
+        runner = ModelRunner(model_dirs["C"], dtype="bfloat16", device="cuda:0", num_blocks=n_req * 3 + 8, max_seq_len=64,
+                             max_num_seqs=80, use_graphs=graphs)
+        rp = TraceReplayer(runner)
+        for i in range(0, n_req, 7):
+            rp.run_step({"step": 0, "entries": [{"id": f"r{j}", "tokens": reqs[j][:20], "want": []} for j in range(i, i + 7)],
+                         "end": []})
+        rows = []
+        for k in range(steps):
+            entries = [{"id": f"r{j}", "tokens": [reqs[j][20 + k]], "want": [0]} for j in range(n_req)]
+            rows.append(rp.run_step({"step": k, "entries": entries, "end": []}))
+            if k % 3 == 1:
+                rp.run_step({"step": 100 + k, "entries": [{"id": "x", "tokens": list(range(5, 35)), "want": [29]}], "end": ["x"]})
+        out[graphs] = np.stack(rows)
+        if graphs:
+            assert any(shape[0] == n_req for shape in runner._graphs)
+    scale = np.abs(out[False]).max(axis=-1)
+    err = np.abs(out[False] - out[True]).max(axis=-1) / scale           # [steps, requests]
+    assert err.max() < TOL_BF16 and np.median(err) < 5e-3, f"worst {err.max():.3e} at step {int(err.max(axis=1).argmax())}"
+    assert err[-1].max() < 1.5 * max(err[0].max(), 1e-3)                 # replays do not drift apart
+
+
 def test_first_tokens_of_a_sequence(model_dirs, plain_models):
     """Positions 0, 1, 2: a single key, no rotation at position 0."""
     for dtype in ("float32", "bfloat16"):
