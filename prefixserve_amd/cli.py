@@ -25,7 +25,7 @@ def _add_engine_options(p: argparse.ArgumentParser) -> None:
     p.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
     p.add_argument("--max-seq-len", type=int, default=8192)
     p.add_argument("--num-blocks", type=int, default=None, help="KV blocks; default: sized from free GPU memory")
-    p.add_argument("--max-waiting", type=int, default=1024)
+    p.add_argument("--max-waiting", type=int, default=256)
     p.add_argument("--max-running-requests", type=int, default=64)
     p.add_argument("--chunked-prefill-size", type=int, default=512)
     p.add_argument("--disable-prefix-cache", action="store_true")
