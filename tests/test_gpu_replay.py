@@ -237,17 +237,26 @@ AWKWARD = dict(architectures=["LlamaForCausalLM"], model_type="llama", vocab_siz
                rms_norm_eps=1e-5, rope_theta=10000.0, max_position_embeddings=512, tie_word_embeddings=False)
 
 
-@pytest.mark.parametrize("seed", [0, 1, 2, 3, 4, 5, 6, 7, "awkward"])
+# Sizes at which the small-step kernels take their other forms: 384 tiles of q/k/v columns (two per
+# workgroup), 803 tiles of gate/up pairs (four per wave), 4,125 tiles of vocabulary (wide row groups).
+WIDE = dict(architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=66000, hidden_size=256,
+            intermediate_size=12840, num_hidden_layers=1, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+            rms_norm_eps=1e-5, rope_theta=500000.0, max_position_embeddings=512, tie_word_embeddings=True)
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2, 3, 4, 5, 6, 7, "awkward", "wide"])
 def test_random_configurations_in_both_dtypes(seed, tmp_path):
     """``awkward``: a width and an inner width that are no multiples of 8 (no 16-byte rows: the
     vectorized kernels and the small-step products must refuse and the general ones run), a
-    head size without a matrix-core kernel, an odd vocabulary."""
+    head size without a matrix-core kernel, an odd vocabulary. ``wide``: see above."""
     from configs import INIT_STD
     from plain.llama_plain import PlainLlama
     from prefixserve_amd.weights import write_random_model
 
     if seed == "awkward":
         rng, cfg, seed = np.random.default_rng(999), dict(AWKWARD), 99
+    elif seed == "wide":
+        rng, cfg, seed = np.random.default_rng(998), dict(WIDE), 98
     else:
         rng = np.random.default_rng(1000 + seed)
         cfg = _random_config(rng)
