@@ -191,12 +191,21 @@ def test_random_workloads_through_the_scheduler(seed, model_dirs, plain_models):
         earlier = [rng.integers(3, vocab, int(rng.integers(1, 16 * pages - 3))).tolist() for _ in range(int(rng.integers(1, 5)))]
         generate(eng, earlier, 3, ignore_eos=True, scheduler=sched)
         temperature = float(rng.choice([0.0, 0.0, 0.9]))
-        outs, stats = generate(eng, prompts, new, temperature=temperature, ignore_eos=True, scheduler=sched)
+        truth = [plain_models[name].greedy(p, new)[0] for p in prompts] if temperature == 0.0 else None
+        stops_early = truth is not None and bool(rng.integers(0, 2))
+        if stops_early:
+            # a token that some request does produce ends requests there, in the middle of rounds too
+            sched.stop_token_ids = frozenset([int(rng.choice(truth[int(rng.integers(0, len(truth)))]))])
+        outs, stats = generate(eng, prompts, new, temperature=temperature, ignore_eos=not stops_early, scheduler=sched)
         preemptions += stats.preemptions
         cached += stats.cached_prompt_tokens
-        if temperature == 0.0:
-            for p, o in zip(prompts, outs):
-                assert o.tokens == plain_models[name].greedy(p, new)[0], f"{name}, prompt of {len(p)}, {eng.cfg}"
+        if truth is not None:
+            for p, o, want in zip(prompts, outs, truth):
+                if stops_early:
+                    stop = next(iter(sched.stop_token_ids))
+                    want = want[:want.index(stop) + 1] if stop in want else want
+                    assert o.finish_reason.value == ("stop" if stop in want else "length")
+                assert o.tokens == want, f"{name}, prompt of {len(p)}, {eng.cfg}"
         else:
             key = (name, eng.cfg.sample_seed)
             if key not in roomy:
