@@ -795,9 +795,6 @@ static int launch_prefill(hipStream_t s, const void* qkv, int q_stride, void* ou
       return check_launch("psamd_attention_prefill");                                                             \
     }                                                                                                             \
   }
-#ifdef PSAMD_PF_KP4
-    PSAMD_GROUPED(4)
-#endif
     PSAMD_GROUPED(2)
     PSAMD_GROUPED(1)
 #undef PSAMD_GROUPED
