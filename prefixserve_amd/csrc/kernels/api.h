@@ -13,9 +13,9 @@ extern "C" {
 
 const char* psamd_last_error(void);
 
-// out[t, :] = float(table[ids[t], :])
+// out[t, :] = float(table[ids[t], :]); table is [vocab, hidden]; an id outside [0, vocab) reads the nearest row.
 int psamd_embed(void* stream, const int32_t* ids, const void* table, int table_dtype, float* out, int64_t tokens,
-                int hidden);
+                int hidden, int vocab);
 
 // x = residual + delta, where delta is [rows, hidden] (delta_dtype) or n_partials float32 slices of that
 // shape, partial_stride elements apart (the partial sums of a K-split product).

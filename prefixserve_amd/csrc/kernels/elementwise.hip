@@ -17,9 +17,12 @@ void set_error(const std::string& msg) { g_error = msg; }
 
 template <typename W>
 __global__ void embed_kernel(const int32_t* __restrict__ ids, const W* __restrict__ table,
-                             float* __restrict__ out, int hidden) {
+                             float* __restrict__ out, int hidden, int vocab) {
   const int64_t t = blockIdx.x;
-  const W* row = table + static_cast<int64_t>(ids[t]) * hidden;
+  // Ids are checked on the host, except those a previous step sampled and left on the device:
+  // an id outside the table reads its nearest row instead of memory that is not the table's.
+  const int id = min(max(ids[t], 0), vocab - 1);
+  const W* row = table + static_cast<int64_t>(id) * hidden;
   float* o = out + t * hidden;
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = to_float<W>(row[i]);
 }
@@ -361,14 +364,14 @@ extern "C" {
 const char* psamd_last_error(void) { return g_error.c_str(); }
 
 int psamd_embed(void* stream, const int32_t* ids, const void* table, int table_dtype, float* out, int64_t tokens,
-                int hidden) {
-  PSAMD_REQUIRE(tokens >= 0 && hidden > 0, "bad sizes");
+                int hidden, int vocab) {
+  PSAMD_REQUIRE(tokens >= 0 && hidden > 0 && vocab > 0, "bad sizes");
   if (tokens == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (table_dtype == kBF16) {
-    embed_kernel<bf16_t><<<dim3(tokens), dim3(256), 0, s>>>(ids, static_cast<const bf16_t*>(table), out, hidden);
+    embed_kernel<bf16_t><<<dim3(tokens), dim3(256), 0, s>>>(ids, static_cast<const bf16_t*>(table), out, hidden, vocab);
   } else if (table_dtype == kF32) {
-    embed_kernel<float><<<dim3(tokens), dim3(256), 0, s>>>(ids, static_cast<const float*>(table), out, hidden);
+    embed_kernel<float><<<dim3(tokens), dim3(256), 0, s>>>(ids, static_cast<const float*>(table), out, hidden, vocab);
   } else {
     return fail("psamd_embed: table dtype must be float32 or bfloat16");
   }

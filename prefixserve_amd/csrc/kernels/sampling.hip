@@ -26,6 +26,9 @@ struct RunStat {
   float pad;
 };
 
+// A NaN never wins (both comparisons are false for it): a row of NaNs, or of -inf, keeps the
+// index the search started from, so callers start from an index of the row, never from a
+// sentinel outside it. The token is fed to the next step's embedding on the device.
 __device__ __forceinline__ void take_max(float v, int32_t i, float& best, int32_t& best_i) {
   if (v > best || (v == best && i < best_i)) {
     best = v;
@@ -106,7 +109,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_runs_kernel(const float
   const float* row = logits + static_cast<int64_t>(r) * vocab;
   const int lo = run * run_len, hi = min(lo + run_len, vocab);
   float best = -INFINITY;
-  int32_t best_i = 0x7fffffff;
+  int32_t best_i = lo;
   for_each_in_run(row, lo, hi, [&](float v, int32_t i) { take_max(v, i, best, best_i); });
   block_argmax(best, best_i, red, red_i);
   const float temp = temperature[r];
@@ -133,7 +136,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_pick_kernel(const float
   const int tid = threadIdx.x, r = blockIdx.x;
   const RunStat* st = stats + static_cast<int64_t>(r) * runs;
   float best = -INFINITY;
-  int32_t best_i = 0x7fffffff;
+  int32_t best_i = 0;
   for (int c = 0; c < runs; ++c) take_max(st[c].max, st[c].arg, best, best_i);   // runs in index order: first wins
   const float temp = temperature[r];
   if (!(temp > 0.f)) {
@@ -180,7 +183,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_pick_kernel(const float
     atomicMin(&chosen, pick);
   }
   __syncthreads();
-  if (tid == 0) out[r] = chosen;
+  if (tid == 0) out[r] = min(max(chosen, 0), vocab - 1);
 }
 
 }  // namespace psamd

@@ -39,7 +39,7 @@ def _ptr(t: torch.Tensor | None) -> int | None:
 
 
 _SIGNATURES = {
-    "psamd_embed": [_vp, _vp, _vp, _i32, _vp, _i64, _i32],
+    "psamd_embed": [_vp, _vp, _vp, _i32, _vp, _i64, _i32, _i32],
     "psamd_add_rmsnorm": [_vp, _vp, _vp, _i32, _i32, _i64, _vp, _vp, _i32, _f32, _vp, _i32, _i64, _i32],
     "psamd_swiglu": [_vp, _vp, _vp, _i32, _i64, _i32],
     "psamd_rope_kv_append": [_vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp, _vp, _vp, _vp],
@@ -128,7 +128,7 @@ class HipOps:
         self._need(ids.dtype == torch.int32 and ids.numel() == t, "embed: ids must be int32 [T]")
         self._need(table.shape[1] == h and out.dtype == torch.float32 and out.is_contiguous(), "embed: bad output")
         self._ok(self.lib.psamd_embed(self._stream(), ids.data_ptr(), table.data_ptr(), _code(table.dtype),
-                                      out.data_ptr(), t, h))
+                                      out.data_ptr(), t, h, table.shape[0]))
 
     def _delta_args(self, delta, t: int, h: int, out_dtype: torch.dtype) -> tuple:
         """(pointer, dtype code, slices, stride) of a delta: [T, H] in the activation dtype, or

@@ -481,6 +481,35 @@ def test_sampling_kernel(ops, vocab):
     assert out2.tolist() == [logits_tie] + torch.argmax(logits[1:], -1).tolist()
 
 
+@pytest.mark.parametrize("vocab", [5, 5000, 40001])
+def test_sampling_of_rows_without_a_maximum_stays_in_the_vocabulary(ops, vocab):
+    """Rows of NaN or of -inf have no largest entry. The token is fed to the next step's
+    embedding on the device, so whatever is returned must be an index of the row."""
+    logits = rnd(6, vocab, seed=9)
+    logits[0] = float("nan")
+    logits[1] = float("-inf")
+    logits[2] = float("nan")
+    logits[3] = float("-inf")
+    logits[4, : vocab // 2] = float("nan")                          # NaNs beside numbers: a number wins
+    temps = torch.tensor([0.0, 0.0, 0.9, 0.9, 0.0, 0.0], device=DEV)
+    us = torch.tensor([0.0, 0.0, 0.7, 0.7, 0.0, 0.0], device=DEV)
+    out = torch.full((6,), -7, dtype=torch.int32, device=DEV)
+    ops.sample(logits, temps, us, out)
+    got = out.tolist()
+    assert all(0 <= t < vocab for t in got), got
+    assert got[0] == 0 and got[1] == 0
+    assert got[4] == vocab // 2 + int(torch.argmax(logits[4, vocab // 2:]))
+    assert got[5] == int(torch.argmax(logits[5]))
+
+
+def test_embed_reads_the_nearest_row_for_an_id_outside_the_table(ops):
+    table = rnd(7, 24).to(torch.bfloat16)
+    ids = torch.tensor([3, -5, 0x7FFFFFFF, 6, 7], dtype=torch.int32, device=DEV)
+    out = torch.empty(5, 24, device=DEV)
+    ops.embed(ids, table, out)
+    assert torch.equal(out, table[[3, 0, 6, 6, 6]].float())
+
+
 def test_sampling_frequencies(ops):
     logits = torch.tensor([[0.0, 1.0, 2.0, -1.0, 0.5]], device=DEV).repeat(4000, 1).contiguous()
     g = torch.Generator().manual_seed(0)
