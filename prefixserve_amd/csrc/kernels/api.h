@@ -81,6 +81,18 @@ int64_t psamd_sample_scratch_floats(int rows);
 int psamd_sample(void* stream, const float* logits, const float* temperature, const float* uniform, int32_t* out,
                  float* scratch, int rows, int vocab);
 
+// psamd_sample for callers that cannot allocate or bring a scratch buffer (code under HIP graph
+// capture, serving loops and harnesses that forbid hipMalloc). It has no counterpart in the
+// reference. The run statistics live in a 128 KiB array inside the library that every GPU holds
+// until the process ends, so rows is limited to psamd_sample_static_max_rows() (256); more is an
+// error. The call allocates nothing and calls no library routine that does; the caller passes
+// inputs and outputs as for psamd_sample, with the stream's device current. All calls on one GPU
+// share the array: two calls that overlap there (different streams, or two threads) race, and
+// the caller has to order them. Same kernels and the same result as psamd_sample.
+int psamd_sample_static_max_rows(void);
+int psamd_sample_static(void* stream, const float* logits, const float* temperature, const float* uniform,
+                        int32_t* out, int rows, int vocab);
+
 #ifdef __cplusplus
 }
 #endif

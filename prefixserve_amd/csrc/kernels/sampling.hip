@@ -10,6 +10,7 @@
 // finds the run in which the cumulative sum passes the target and scans only that run.
 
 #include <algorithm>
+#include <mutex>
 
 #include "api.h"
 #include "common.h"
@@ -186,6 +187,51 @@ __global__ __launch_bounds__(kSampleThreads) void sample_pick_kernel(const float
   if (tid == 0) out[r] = min(max(chosen, 0), vocab - 1);
 }
 
+// ---- the entry point that allocates nothing --------------------------------------------
+//
+// The run statistics of psamd_sample_static live in this array instead of a buffer the caller
+// brings: kStaticMaxRows rows x kMaxRuns runs x 16 bytes = 128 KiB, held by every GPU the
+// library runs on until the process ends. Host code never uses the array's name as an
+// address: it asks the runtime once per device for the device's own copy and passes that
+// pointer on.
+constexpr int kStaticMaxRows = 256;
+static __device__ __align__(256) RunStat scratch[kStaticMaxRows * kMaxRuns];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static RunStat* g_scratch_ptr[kMaxDevices] = {};
+
+// The address of `scratch` on the current device, looked up on the first call there.
+static int static_scratch(RunStat** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(std::string("psamd_sample_static: hipGetDevice: ") + hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return fail("psamd_sample_static: device index beyond " + std::to_string(kMaxDevices));
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr)
+      return fail(std::string("psamd_sample_static: hipGetSymbolAddress: ") + hipGetErrorString(e));
+    g_scratch_ptr[dev] = static_cast<RunStat*>(p);
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
+}
+
+static int launch_sample(hipStream_t s, const float* logits, const float* temperature, const float* uniform,
+                         int32_t* out, RunStat* stats, int rows, int vocab) {
+  // Runs of at least 1024 entries, a multiple of 4 long, at most kMaxRuns of them.
+  int run_len = static_cast<int>(ceil_div(vocab, kMaxRuns));
+  run_len = std::max(1024, (run_len + 3) & ~3);
+  const int runs = static_cast<int>(ceil_div(vocab, run_len));
+  sample_runs_kernel<<<dim3(runs, rows), dim3(kSampleThreads), 0, s>>>(logits, temperature, stats, vocab, run_len);
+  if (int rc = check_launch("psamd_sample(runs)")) return rc;
+  sample_pick_kernel<<<dim3(rows), dim3(kSampleThreads), 0, s>>>(logits, temperature, uniform, stats, out, vocab, run_len,
+                                                                runs);
+  return check_launch("psamd_sample(pick)");
+}
+
 }  // namespace psamd
 
 using namespace psamd;
@@ -201,17 +247,24 @@ int psamd_sample(void* stream, const float* logits, const float* temperature, co
   PSAMD_REQUIRE(rows <= 65535, "too many rows for one launch");
   if (rows == 0) return 0;
   PSAMD_REQUIRE(scratch != nullptr, "sampling needs its scratch buffer");
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  // Runs of at least 1024 entries, a multiple of 4 long, at most kMaxRuns of them.
-  int run_len = static_cast<int>(ceil_div(vocab, kMaxRuns));
-  run_len = std::max(1024, (run_len + 3) & ~3);
-  const int runs = static_cast<int>(ceil_div(vocab, run_len));
-  RunStat* stats = reinterpret_cast<RunStat*>(scratch);
-  sample_runs_kernel<<<dim3(runs, rows), dim3(kSampleThreads), 0, s>>>(logits, temperature, stats, vocab, run_len);
-  if (int rc = check_launch("psamd_sample(runs)")) return rc;
-  sample_pick_kernel<<<dim3(rows), dim3(kSampleThreads), 0, s>>>(logits, temperature, uniform, stats, out, vocab, run_len,
-                                                                runs);
-  return check_launch("psamd_sample(pick)");
+  return launch_sample(static_cast<hipStream_t>(stream), logits, temperature, uniform, out,
+                       reinterpret_cast<RunStat*>(scratch), rows, vocab);
+}
+
+int psamd_sample_static_max_rows(void) { return kStaticMaxRows; }
+
+int psamd_sample_static(void* stream, const float* logits, const float* temperature, const float* uniform,
+                        int32_t* out, int rows, int vocab) {
+  PSAMD_REQUIRE(rows >= 0 && vocab > 0, "bad sizes");
+  PSAMD_REQUIRE(rows <= kStaticMaxRows,
+                "at most " + std::to_string(kStaticMaxRows) + " rows fit the built-in scratch array, got " +
+                    std::to_string(rows) + " (psamd_sample takes a buffer of any size)");
+  if (rows == 0) return 0;
+  RunStat* stats = nullptr;
+  if (int rc = static_scratch(&stats)) return rc;
+  // Nothing has to be cleared: the first kernel writes the statistics of every (row, run) of this
+  // call before the second reads exactly those; what an earlier call left beyond them is not read.
+  return launch_sample(static_cast<hipStream_t>(stream), logits, temperature, uniform, out, stats, rows, vocab);
 }
 
 }  // extern "C"
