@@ -7,7 +7,9 @@ is preempted, when a window has passed them, and when cached prefixes are evicte
 room; they are then used again.
 
 Prefix caching needs every key of the prefix to be present, so it is active only when no
-group is windowed. With several groups each has a tree of its own; a match is the shortest
+group is windowed; and it needs everything a request has computed to be in pages, so it is
+off when requests keep state in slots (``bytes_per_slot > 0``): a request that started
+behind a cached prefix would run with a state that never saw the prefix. With several groups each has a tree of its own; a match is the shortest
 of the groups' matches.
 """
 
@@ -41,7 +43,8 @@ class CacheManager:
         if len(self.windows) != self.num_groups:
             raise ValueError("one window entry per group")
         self.pools = [BlockManager(int(n)) for n in num_blocks]
-        self.prefix_cache = bool(enable_prefix_cache) and all(w is None for w in self.windows)
+        self.prefix_cache = (bool(enable_prefix_cache) and all(w is None for w in self.windows)
+                             and int(bytes_per_slot) == 0)
         self.trees = [RadixTree(p, hash_seed) for p in self.pools] if self.prefix_cache else []
         self.slots = StateSlots(int(num_slots), int(bytes_per_slot))
 

@@ -18,6 +18,7 @@ from typing import Any, Mapping
 ARCHITECTURE = "LlamaForCausalLM"
 MODEL_TYPE = "llama"
 DEFAULT_ROPE_THETA = 10000.0
+HIDDEN_ACT = "silu"          # the gate of the feed-forward; the one activation the kernels implement
 
 # dataclass field -> config.json key, for the sizes that must be there and are plain integers
 _INT_KEYS = {
@@ -80,6 +81,7 @@ class LlamaConfig:
     rope_scaling: Llama3RopeScaling | None
     tie_word_embeddings: bool
     stop_token_ids: frozenset[int]
+    hidden_act: str = HIDDEN_ACT
 
     @property
     def q_size(self) -> int:
@@ -120,6 +122,9 @@ class LlamaConfig:
             rope_scaling=scaling,
             tie_word_embeddings=bool(raw.get("tie_word_embeddings", False)),
             stop_token_ids=_stop_ids(raw, gen),
+            # The reference never reads this key and always applies SiLU (prefixserve/model/llama.py:121);
+            # a file that names another activation is refused above rather than run with the wrong one.
+            hidden_act=str(raw.get("hidden_act") or HIDDEN_ACT),
         )
 
     # ------------------------------------------------------------------ writing
@@ -130,7 +135,7 @@ class LlamaConfig:
         out: dict[str, Any] = {"architectures": [ARCHITECTURE], "model_type": MODEL_TYPE}
         out.update({key: getattr(self, name) for name, key in _INT_KEYS.items()})
         out.update(num_key_value_heads=self.num_kv_heads, head_dim=self.head_dim, rms_norm_eps=self.rms_norm_eps,
-                   rope_theta=self.rope_theta, tie_word_embeddings=self.tie_word_embeddings, hidden_act="silu",
+                   rope_theta=self.rope_theta, tie_word_embeddings=self.tie_word_embeddings, hidden_act=self.hidden_act,
                    attention_bias=False, mlp_bias=False,
                    rope_scaling=self.rope_scaling.to_json() if self.rope_scaling is not None else None)
         stops = sorted(self.stop_token_ids)
@@ -146,6 +151,9 @@ def _refuse_what_is_not_llama(raw: Mapping[str, Any]) -> None:
     kind = raw.get("model_type")
     if kind != MODEL_TYPE:
         raise UnsupportedModelError(f"model_type is {kind!r}, expected {MODEL_TYPE!r}")
+    act = raw.get("hidden_act")
+    if act is not None and act != HIDDEN_ACT:
+        raise UnsupportedModelError(f"hidden_act is {act!r}: only the {HIDDEN_ACT!r} gate is implemented")
     for key in ("attention_bias", "mlp_bias"):
         if raw.get(key):
             raise UnsupportedModelError(f"{key} is set: projections with a bias are not implemented")

@@ -50,6 +50,11 @@ class Engine:
         self.sampler = Sampler(self.runner.ops, self.runner.device, max(cfg.max_num_seqs, 1))
         self.capture_logits = False
         self.last_logits: dict[str, torch.Tensor] = {}
+        # Set to a list to have every logits row the engine samples from appended to it as
+        # (request id, position of the token the row belongs to, float32 row on the host), in
+        # single steps and in rounds of several decode steps alike. For tests that judge a run
+        # by its logits; it waits for the device at every step.
+        self.logit_trace: list[tuple[str, int, torch.Tensor]] | None = None
         # req_id -> (request, preemption count, [(array, filled)] per group): block tables as arrays,
         # extended as the lists grow, so a step does not convert whole lists again.
         self._tables: dict[str, tuple[Any, int, list[list]]] = {}
@@ -172,6 +177,9 @@ class Engine:
                      for i, (r, w) in enumerate(zip(reqs, work))]
             logits = self.runner.step(items, token_feed=out_dev[j - 1] if j else None)
             assert logits is not None
+            if self.logit_trace is not None:
+                host = logits.to("cpu", copy=True)
+                self.logit_trace += [(w.req.req_id, w.start + j, host[i]) for i, w in enumerate(batch.work)]
             self.sampler.sample_into(logits, t_dev, u_dev[j], out_dev[j])
         rows = self.sampler.fetch(k, len(reqs))
         return {r.req_id: [rows[j][i] for j in range(k)] for i, r in enumerate(reqs)}
@@ -204,6 +212,10 @@ class Engine:
         assert logits is not None
         if self.capture_logits:
             self.last_logits = {r.req_id: logits[i].to("cpu", copy=True) for i, r in enumerate(sampling)}
+        if self.logit_trace is not None:
+            host = logits.to("cpu", copy=True)
+            # items a batch was filled up with repeat its last request and come last: not traced
+            self.logit_trace += [(r.req_id, r.seq_len - 1, host[i]) for i, r in enumerate(sampling[:len(batch.work)])]
         temps = [r.temperature for r in sampling]
         seeds = [uniform_for(self.cfg.sample_seed ^ r.seed, request_key(r.req_id), len(r.output)) if r.temperature > 0
                  else 0.0 for r in sampling]

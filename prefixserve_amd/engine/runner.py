@@ -131,14 +131,14 @@ class ModelRunner:
         return [n] * len(self.layer_groups)
 
     def _activation_bytes(self, tokens: int) -> int:
+        """Device memory the buffers of a step of ``tokens`` tokens take: what the parts say they
+        ask for (buffers are shared between layers by name, so the largest layer counts), the
+        float32 residual stream, the logits of every request and a margin."""
         s = self.spec
-        widest = 0
-        for layer in s.layers:
-            p = dict(layer.mixer.params) | dict(layer.feed_forward.params)
-            widest = max(widest, 3 * int(p.get("intermediate_size", 0)),
-                         2 * int(p.get("num_heads", 0)) * int(p.get("head_dim", 0)))
-        per_token = 4 * (2 * s.hidden_size + widest) + 4 * s.hidden_size
-        return tokens * per_token + self.max_num_seqs * s.vocab_size * 4 + (256 << 20)
+        itemsize = torch.empty((), dtype=self.dtype).element_size()
+        widest = max((sum(p.activation_bytes(tokens, itemsize) for p in blk.parts()) for blk in self.model.blocks),
+                     default=0)
+        return widest + tokens * s.hidden_size * 4 + self.max_num_seqs * s.vocab_size * 4 + (256 << 20)
 
     # ------------------------------------------------------------------ step
 

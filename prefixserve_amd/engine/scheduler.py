@@ -141,6 +141,8 @@ class Scheduler:
         if req_id in self._live:
             return AddResult.DUPLICATE_ID, None
         longest = int(ids.size) + max_tokens
+        if self.max_seq_len is not None and longest > self.max_seq_len:
+            return AddResult.TOO_LONG, None            # the engine cannot address its last positions
         if any(self.cache.pages_needed(g, longest, self.chunk_size) > self.cache.num_blocks(g)
                for g in range(self.cache.num_groups)):
             return AddResult.TOO_LONG, None            # would not finish with the pool to itself

@@ -33,7 +33,8 @@ def build_llama_spec(cfg: LlamaConfig) -> ModelSpec:
                 "num_heads": cfg.num_heads, "num_kv_heads": cfg.num_kv_heads, "head_dim": cfg.head_dim,
                 "names": ATTENTION_NAMES, "position": "rope",
             }),
-            feed_forward=PartSpec("swiglu", {"intermediate_size": cfg.intermediate_size, "names": MLP_NAMES}),
+            feed_forward=PartSpec("swiglu", {"intermediate_size": cfg.intermediate_size, "names": MLP_NAMES,
+                                               "activation": cfg.hidden_act}),
             mixer_norm=PartSpec("rmsnorm", {"eps": cfg.rms_norm_eps, "name": "input_layernorm.weight"}),
             feed_forward_norm=PartSpec("rmsnorm", {"eps": cfg.rms_norm_eps, "name": "post_attention_layernorm.weight"}),
             block="prenorm",

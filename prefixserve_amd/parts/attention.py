@@ -79,6 +79,11 @@ class PagedAttention(Mixer):
     def weight_bytes(self) -> int:
         return sum(w.numel() * w.element_size() for w in (self.w_qkv, self.w_o))
 
+    def activation_bytes(self, tokens: int, itemsize: int) -> int:
+        # q/k/v, the attention output, the projected output (or its float32 partial sums).
+        return tokens * ((self.q_size + 2 * self.kv_size) + self.q_size) * itemsize + 8 * 64 * self.hidden_size * 4 \
+            + tokens * self.hidden_size * itemsize
+
     def forward(self, x: torch.Tensor, ctx: "StepContext", cache: Any, state: torch.Tensor | None,
                 writes_cache: bool) -> torch.Tensor:
         rt, ops, ws = self.rt, self.rt.ops, self.rt.workspace

@@ -119,6 +119,13 @@ class Part:
         """Bytes of weights a step reads from this part (for roofline accounting)."""
         return 0
 
+    def activation_bytes(self, tokens: int, itemsize: int) -> int:
+        """Bytes of buffers this part asks the workspace for in a step of ``tokens`` tokens with
+        activations of ``itemsize`` bytes. The cache pools are sized from what is free after the
+        largest step's buffers; a part that keeps large buffers and does not say so here may
+        leave too little for them."""
+        return 0
+
 
 class Norm(Part):
     """A normalisation fused with the residual sum that precedes it."""

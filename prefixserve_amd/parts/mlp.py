@@ -17,7 +17,10 @@ class SwiGLU(FeedForward):
     first ``intermediate_size`` columns are the gate (prefixserve/model/llama.py:120-121,
     prefixserve/model/weights.py:120-123)."""
 
-    def __init__(self, hidden_size: int, intermediate_size: int, names: Mapping[str, str]) -> None:
+    def __init__(self, hidden_size: int, intermediate_size: int, names: Mapping[str, str],
+                 activation: str = "silu") -> None:
+        if activation != "silu":
+            raise ValueError(f"the gated feed-forward kernels apply SiLU to the gate; {activation!r} is not implemented")
         self.hidden_size = int(hidden_size)
         self.intermediate_size = int(intermediate_size)
         self.names = dict(names)
@@ -34,6 +37,10 @@ class SwiGLU(FeedForward):
 
     def weight_bytes(self) -> int:
         return sum(w.numel() * w.element_size() for w in (self.w_gate_up, self.w_down))
+
+    def activation_bytes(self, tokens: int, itemsize: int) -> int:
+        # gate and up side by side (large steps), their product, the projected output.
+        return tokens * (3 * self.intermediate_size + self.hidden_size) * itemsize + 8 * 64 * self.hidden_size * 4
 
     def forward(self, x: torch.Tensor, ctx: "StepContext") -> torch.Tensor:
         rt, ops, ws = self.rt, self.rt.ops, self.rt.workspace

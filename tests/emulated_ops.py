@@ -82,6 +82,10 @@ class EmulatedOps:
             kpages[page, :, off, :] = k
             vpages[page, :, :, off] = v
 
+    def expand_kv(self, x, rep):
+        """[keys, kv_heads, d] -> [keys, heads, d]: query head h reads kv head h // rep."""
+        return x.repeat_interleave(rep, dim=1)
+
     def paged_attention(self, qkv, out, kv, ctx, group, hq, hkv, d, scale, window) -> None:
         g = ctx.groups[group]
         t = qkv.shape[0]
@@ -96,8 +100,8 @@ class EmulatedOps:
             pages = g.block_ids[offs[i]: offs[i] + -(-end // PAGE)].long()
             keys = kv[pages, 0].view(-1, hkv, PAGE, d).permute(0, 2, 1, 3).reshape(-1, hkv, d)[:end].float()
             vals = kv[pages, 1].view(-1, hkv, d, PAGE).permute(0, 3, 1, 2).reshape(-1, hkv, d)[:end].float()
-            keys = keys.repeat_interleave(rep, dim=1)
-            vals = vals.repeat_interleave(rep, dim=1)
+            keys = self.expand_kv(keys, rep)
+            vals = self.expand_kv(vals, rep)
             qi = q[t0:t1].transpose(0, 1)                                  # [hq, n, d]
             scores = torch.matmul(qi, keys.permute(1, 2, 0)) * scale        # [hq, n, end]
             qpos = torch.arange(pos0, end)[:, None]

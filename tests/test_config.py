@@ -62,7 +62,8 @@ def test_defaults_and_stop_ids():
 
 
 @pytest.mark.parametrize("change", [dict(model_type="mistral"), dict(rope_scaling={"rope_type": "yarn", "factor": 4.0}),
-                                    dict(attention_bias=True), dict(mlp_bias=True), dict(num_key_value_heads=5)])
+                                    dict(attention_bias=True), dict(mlp_bias=True), dict(num_key_value_heads=5),
+                                    dict(hidden_act="gelu")])
 def test_what_cannot_run_is_refused(change):
     with pytest.raises(UnsupportedModelError):
         parse(**change)

@@ -9,6 +9,7 @@ import pytest
 import torch
 
 import traces
+from checks import CacheWriteWatch
 from configs import TINY, TOL_F32
 from emulated_ops import EmulatedOps
 from prefixserve_amd.engine.batch import EngineError, GroupMeta, StepItem, StepPacker
@@ -115,7 +116,10 @@ def test_scheduler_driven_greedy_generation_equals_plain(name, model_dirs, plain
                               max_prefill_tokens=24, max_seq_len=256, num_blocks=11, use_graphs=False), ops=EmulatedOps())
     eng.capture_logits = True
     times = LoopTimes()
-    outs, stats = generate(eng, prompts, new, ignore_eos=True, times=times)
+    sched = eng.make_scheduler(chunk_size=24)
+    watch = CacheWriteWatch(eng, sched)
+    outs, stats = generate(eng, prompts, new, ignore_eos=True, times=times, scheduler=sched)
+    assert watch.writes >= sum(len(p) for p in prompts) - stats.cached_prompt_tokens
     for p, o in zip(prompts, outs):
         want, _ = plain_models[name].greedy(p, new)
         assert o.tokens == want, f"prompt of {len(p)}: {o.tokens} != {want}"
@@ -205,3 +209,108 @@ def test_a_request_id_that_comes_back_gets_its_own_block_tables(model_dirs, plai
     assert again[0].cached_tokens >= 32                                     # the first prompt came from the cache
     for p, o in zip(first, again):
         assert o.tokens == plain_models["A"].greedy(p, 6)[0]
+
+
+# ------------------------------------------------------------- a mixer that keeps state
+
+def test_a_state_keeping_mixer_through_the_scheduler(tmp_path):
+    """The toy running-mean mixer (state in slots, no pages) through the engine and the
+    scheduler with a shared prefix and a pool so small that requests are sent back: a prefix
+    hit would start a request behind tokens its state never saw, so the cache manager keeps
+    the prefix cache off for such a model, and a request that comes back starts from
+    position 0 with a fresh state. Every token equals the model's own whole-sequence choice."""
+    from toy_parts import write_toy_mean_model
+
+    write_toy_mean_model(tmp_path)
+    rng = np.random.default_rng(3)
+    shared = rng.integers(0, 100, 40).tolist()
+    prompts = [shared + rng.integers(0, 100, n).tolist() for n in (9, 30, 17)] + [shared[:33]]
+    new = 12
+    eng = Engine(EngineConfig(model_path=tmp_path, dtype="float32", device="cpu", max_num_seqs=4,
+                              max_prefill_tokens=24, max_seq_len=256, num_blocks=12, use_graphs=False), ops=EmulatedOps())
+    assert eng.runner.state_bytes_per_slot > 0
+    sched = eng.make_scheduler(chunk_size=24)
+    assert sched.cache.prefix_cache is False and sched.tree is None
+    outs, stats = generate(eng, prompts, new, ignore_eos=True, scheduler=sched)
+    assert stats.preemptions > 0 and stats.cached_prompt_tokens == 0
+    assert sched.cache.num_free(0) == 12 and sched.cache.slots.num_free == 4
+    roomy = make_runner(tmp_path, num_blocks=64)
+    for i, (p, o) in enumerate(zip(prompts, outs)):
+        seq = p + o.tokens
+        rows = TraceReplayer(roomy).run_step(
+            {"step": i, "entries": [{"id": "w", "tokens": seq[:-1], "want": list(range(len(p) - 1, len(seq) - 1))}],
+             "end": ["w"]})
+        assert np.argmax(rows, -1).tolist() == o.tokens, f"request {i}"
+
+
+def test_activation_bytes_come_from_the_parts(model_dirs, tmp_path):
+    """The pool is sized from what the parts say their buffers take, not from parameter
+    names: a part with other names is counted too."""
+    from toy_parts import write_toy_mean_model
+
+    runner = make_runner(model_dirs["A"])
+    cfg = TINY["A"]
+    per_layer = runner._activation_bytes(1000) - runner._activation_bytes(0)
+    assert per_layer >= 1000 * 4 * (3 * cfg["intermediate_size"] + 4 * cfg["hidden_size"])
+    toy = make_runner(write_toy_mean_model(tmp_path))
+    assert toy._activation_bytes(1000) - toy._activation_bytes(0) >= 1000 * 4 * (3 * 96 + 4 * 64)
+
+
+# ------------------------------------------------------------- faults switched on
+
+class _GateUpSwapped(EmulatedOps):
+    def linear_swiglu(self, x, w_gate_up, out) -> None:
+        inter = w_gate_up.shape[0] // 2
+        super().linear_swiglu(x, torch.cat([w_gate_up[inter:], w_gate_up[:inter]]), out)
+
+
+class _KvHeadByRemainder(EmulatedOps):
+    """Query head h reads kv head h % kv_heads instead of h // (heads / kv_heads)."""
+
+    def expand_kv(self, x, rep):
+        return x.repeat(1, rep, 1)
+
+
+def _relative_positions(runner):
+    """The reference's own switchable fault (prefixserve/llama_engine.py:192, ``rope_relative``):
+    positions restart at 0 in every portion."""
+    inner = runner.packer.pack
+
+    def pack(items, **kw):
+        ctx = inner(items, **kw)
+        ctx.positions -= ctx.item_pos0[ctx.tok_item.long()]
+        return ctx
+
+    runner.packer.pack = pack
+
+
+@pytest.mark.parametrize("fault", ["relative positions", "gate and up swapped", "kv head by remainder"])
+def test_the_cuttings_catch_a_fault_that_is_switched_on(fault, model_dirs, plain_models):
+    """What the replay comparisons are worth: each of three plausible faults, switched on in
+    the host stand-in, must fail them (the reference checks its own tests the same way,
+    tests/test_llama_exact.py:227-241). Positions that restart per portion are right for a
+    whole prompt and wrong for every later portion, so only the cut replay sees them."""
+    name = "A"                                              # 4 heads on 2 kv heads: the two head maps differ
+    reqs = requests_for(name, [70, 33, 97])
+    truth = [plain_models[name].logits(t) for t in reqs]
+    ops = {"gate and up swapped": _GateUpSwapped, "kv head by remainder": _KvHeadByRemainder}.get(fault, EmulatedOps)()
+    runner = ModelRunner(model_dirs[name], dtype="float32", device="cpu", num_blocks=64, max_seq_len=512,
+                         max_num_seqs=8, ops=ops, use_graphs=False)
+    if fault == "relative positions":
+        _relative_positions(runner)
+        steps, expect = traces.whole(reqs)
+        traces.compare(TraceReplayer(runner).run_step, steps, expect, truth, TOL_F32)     # whole prompts: no difference
+    steps, expect = traces.portions(reqs)
+    with pytest.raises(AssertionError, match="relative error"):
+        traces.compare(TraceReplayer(runner).run_step, steps, expect, truth, TOL_F32)
+
+
+def test_the_scheduler_refuses_what_the_engine_cannot_address(model_dirs):
+    eng = Engine(EngineConfig(model_path=model_dirs["A"], dtype="float32", device="cpu", max_num_seqs=2,
+                              max_seq_len=64, num_blocks=32, use_graphs=False), ops=EmulatedOps())
+    sched = eng.make_scheduler()
+    from prefixserve_amd.engine.scheduler import AddResult
+
+    assert sched.add_request("long", list(range(3, 60)), 8) is AddResult.TOO_LONG      # 57 + 8 > 64, the pool would do
+    assert sched.add_request("fits", list(range(3, 59)), 8) is AddResult.ACCEPTED
+    assert sched.stats().rejected == 1

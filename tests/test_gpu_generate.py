@@ -10,7 +10,8 @@ from pathlib import Path
 import numpy as np
 import pytest
 
-from configs import TINY
+from checks import CacheWriteWatch, logit_errors
+from configs import TINY, TOL_BF16
 
 pytestmark = pytest.mark.gpu
 ROOT = Path(__file__).resolve().parent.parent
@@ -34,40 +35,85 @@ def test_greedy_generation_equals_plain_in_float32(name, model_dirs, plain_model
     shared = rng.integers(3, vocab, 37).tolist()
     prompts = [shared + rng.integers(3, vocab, n).tolist() for n in (9, 21, 40)] + [rng.integers(3, vocab, 5).tolist()]
     eng = engine_for(model_dirs[name], "float32", 11)
-    eng.capture_logits = True
-    outs, stats = generate(eng, prompts, 12, ignore_eos=True)
+    eng.logit_trace = []
+    sched = eng.make_scheduler(chunk_size=24)
+    watch = CacheWriteWatch(eng, sched)
+    outs, stats = generate(eng, prompts, 12, ignore_eos=True, scheduler=sched)
     for p, o in zip(prompts, outs):
         want, rows = plain_models[name].greedy(p, 12)
         assert o.tokens == want
-    assert stats.preemptions > 0 and stats.cached_prompt_tokens > 0
-    last = outs[-1]
-    seq = prompts[-1] + last.tokens[:-1]
-    truth = plain_models[name].logits(seq)[-1]
-    got = eng.last_logits.get("req-3")
-    if got is not None:
-        assert np.abs(got.numpy() - truth).max() / np.abs(truth).max() < 1e-4
+    assert stats.preemptions > 0 and stats.cached_prompt_tokens > 0 and watch.writes > 0
+    errors = logit_errors(eng.logit_trace, prompts, outs, plain_models[name])
+    assert len(errors) >= 4 * 12 and max(errors) < 1e-4
 
 
-def test_greedy_generation_in_bfloat16_is_teacher_forced_close(model_dirs, plain_models):
-    """Free-running bfloat16 may leave the 32-bit path at a near-tie; where it does, the plain
-    model's two best logits must be close. Everywhere else the tokens are equal."""
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_bfloat16_through_the_scheduler_under_pressure(name, model_dirs, plain_models, plain_bf16_error):
+    """The same schedule in bfloat16: portions under a budget of 24, a shared prefix found in
+    the cache, eviction, requests sent back and recomputed. Judged by the logits of every
+    sampling step, given the tokens the engine produced: each row within the bfloat16 bar and
+    their mean no worse than a plain bfloat16 run of the model."""
+    from prefixserve_amd import generate
+
+    vocab = TINY[name]["vocab_size"]
+    rng = np.random.default_rng(4)
+    shared = rng.integers(3, vocab, 37).tolist()
+    prompts = [shared + rng.integers(3, vocab, n).tolist() for n in (9, 21, 40)] + [rng.integers(3, vocab, 5).tolist()]
+    eng = engine_for(model_dirs[name], "bfloat16", 11)
+    eng.runner.pools.tensors[0].fill_(1e30)                 # a page that is used again never holds zeros
+    eng.logit_trace = []
+    sched = eng.make_scheduler(chunk_size=24)
+    watch = CacheWriteWatch(eng, sched)
+    outs, stats = generate(eng, prompts, 16, ignore_eos=True, scheduler=sched)
+    assert stats.preemptions > 0 and stats.cached_prompt_tokens > 0 and watch.writes > 0
+    assert all(len(o.tokens) == 16 for o in outs)
+    errors = logit_errors(eng.logit_trace, prompts, outs, plain_models[name])
+    assert len(errors) >= 4 * 16
+    assert max(errors) < TOL_BF16 and np.mean(errors) <= plain_bf16_error[name], (max(errors), np.mean(errors))
+    assert sched.cache.num_free(0) + sched.stats().cached_blocks == 11
+
+
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_bfloat16_decode_rounds_through_graphs_after_warm_up(name, model_dirs, plain_models, plain_bf16_error):
+    """The path the benchmark times: bfloat16, warm_up, eight decode steps per scheduler round
+    replayed as graphs with the sampled token fed on the device, batches filled up to the
+    captured sizes. Judged by the logits of every step."""
+    from prefixserve_amd import Engine, EngineConfig, generate
+
+    vocab = TINY[name]["vocab_size"]
+    rng = np.random.default_rng(17)
+    prompts = [rng.integers(3, vocab, n).tolist() for n in (33, 5, 18, 47, 60, 9, 21)]
+    eng = Engine(EngineConfig(model_path=model_dirs[name], dtype="bfloat16", max_num_seqs=12, max_prefill_tokens=64,
+                              max_seq_len=160, num_blocks=80, decode_steps=8))
+    eng.warm_up()
+    captured = set(eng.runner._graphs)
+    eng.logit_trace = []
+    outs, stats = generate(eng, prompts, 40, ignore_eos=True)
+    assert set(eng.runner._graphs) == captured and all(len(o.tokens) == 40 for o in outs)
+    errors = logit_errors(eng.logit_trace, prompts, outs, plain_models[name])
+    assert len(errors) >= 7 * 40
+    assert max(errors) < TOL_BF16 and np.mean(errors) <= plain_bf16_error[name], (max(errors), np.mean(errors))
+
+
+def test_greedy_generation_in_bfloat16_is_close_at_every_step(model_dirs, plain_models, plain_bf16_error):
+    """Free-running bfloat16 may choose another token than the plain model at a near-tie, so
+    the run is judged by its logits: every row the engine sampled from against the plain
+    model given the same tokens, and a token that differs from the plain model's choice only
+    where the plain model's two candidates are close."""
     from prefixserve_amd import generate
 
     name = "B"
     rng = np.random.default_rng(6)
     prompts = [rng.integers(3, 512, n).tolist() for n in (30, 12)]
     eng = engine_for(model_dirs[name], "bfloat16", 32)
+    eng.logit_trace = []
     outs, _ = generate(eng, prompts, 16, ignore_eos=True)
+    errors = logit_errors(eng.logit_trace, prompts, outs, plain_models[name])
+    assert len(errors) == 32 and max(errors) < TOL_BF16 and np.mean(errors) <= plain_bf16_error[name]
     for p, o in zip(prompts, outs):
-        seq = list(p)
-        for tok in o.tokens:
-            row = plain_models[name].logits(seq)[-1]
-            best = int(np.argmax(row))
-            if tok != best:
-                top2 = np.sort(row)[-2:]
-                assert row[best] - row[tok] < 0.05 * np.abs(row).max(), "left the plain model at a clear margin"
-                break
-            seq.append(tok)
+        truth = plain_models[name].logits(p + o.tokens[:-1])[len(p) - 1:]
+        for row, tok in zip(truth, o.tokens):
+            assert row.max() - row[tok] < 2 * TOL_BF16 * np.abs(row).max(), "left the plain model at a clear margin"
 
 
 def test_temperature_sampling_survives_preemption(model_dirs):
@@ -111,7 +157,7 @@ def test_pool_is_sized_from_free_memory(model_dirs):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_a_hundred_requests_decode_together(dtype, model_dirs, plain_models):
+def test_a_hundred_requests_decode_together(dtype, model_dirs, plain_models, plain_bf16_error):
     """More decoding requests in one step than the small-step kernels take (64): the step falls
     back to the general product and the decode attention runs over 100 block tables."""
     from prefixserve_amd import Engine, EngineConfig, generate
@@ -128,20 +174,17 @@ def test_a_hundred_requests_decode_together(dtype, model_dirs, plain_models):
         return step(batch)
 
     eng.step = counting_step
+    eng.logit_trace = []
     outs, stats = generate(eng, prompts, 10, ignore_eos=True)
     assert stats.preemptions == 0 and widest[0] == 100
-    for p, o in list(zip(prompts, outs))[::7]:
-        if dtype == "float32":
+    errors = logit_errors(eng.logit_trace, prompts, outs, plain_models[name])
+    assert len(errors) == 1000
+    if dtype == "float32":
+        assert max(errors) < 1e-4
+        for p, o in list(zip(prompts, outs))[::7]:
             assert o.tokens == plain_models[name].greedy(p, 10)[0]
-            continue
-        seq = list(p)
-        for tok in o.tokens:                                  # teacher-forced: equal, or a near-tie
-            row = plain_models[name].logits(seq)[-1]
-            best = int(np.argmax(row))
-            if tok != best:
-                assert row[best] - row[tok] < 0.05 * np.abs(row).max(), "left the plain model at a clear margin"
-                break
-            seq.append(tok)
+    else:
+        assert max(errors) < TOL_BF16 and np.mean(errors) <= plain_bf16_error[name], (max(errors), np.mean(errors))
 
 
 def test_several_decode_steps_before_the_host_reads(model_dirs, plain_models):

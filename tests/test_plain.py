@@ -71,14 +71,46 @@ def test_llama3_bands():
     assert np.all(got[mid] < base[mid]) and np.all(got[mid] > base[mid] / 8.0)  # a blend in between
 
 
+def _pair_wavelengths(head_dim, theta):
+    return 2 * math.pi * theta ** (np.arange(0, head_dim, 2) / head_dim)
+
+
+def test_llama3_medium_band_falls_from_one_to_one_over_factor():
+    """Several pairs inside the medium band: the ratio to the unscaled frequency is linear in
+    old/wavelength, 1 at the short edge and 1/factor at the long edge, so it falls with the
+    wavelength. A blend with ``smooth`` and ``1 - smooth`` swapped rises instead; one that
+    interpolates in the wavelength rather than its inverse is not linear here."""
+    d, theta = 64, 10000.0
+    rule = dict(factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0, original_max_position_embeddings=256)
+    base = P.rope_inv_freq(d, theta, None).astype(np.float64)
+    got = P.rope_inv_freq(d, theta, rule).astype(np.float64)
+    wl = _pair_wavelengths(d, theta)
+    mid = (wl >= 256 / 4.0) & (wl <= 256 / 1.0)
+    assert mid.sum() >= 4
+    ratio = got[mid] / base[mid]
+    assert np.all(np.diff(ratio) < 0) and ratio[0] < 1.0 and ratio[-1] > 1 / 8.0
+    # Written out independently of the blend: a line through (old/wl = high, 1) and (old/wl = low, 1/factor).
+    x = 256.0 / wl[mid]
+    line = 1 / 8.0 + (1 - 1 / 8.0) * (x - 1.0) / (4.0 - 1.0)
+    np.testing.assert_allclose(ratio, line, rtol=2e-6)
+    # One number by hand: halfway between the edges in old/wl (2.5) the ratio is (1 + 1/8) / 2.
+    assert abs(np.interp(2.5, x[::-1], ratio[::-1]) - 0.5625) < 2e-3
+
+
 def test_llama3_is_continuous_at_the_band_edges():
-    # smooth = 0 at wavelen = old/low and 1 at old/high, so the blend meets both neighbours.
-    old, low, high, factor = 64.0, 1.0, 4.0, 8.0
-    for wl, want_ratio in ((old / low, 1 / factor), (old / high, 1.0)):
-        inv = 2 * math.pi / wl
-        smooth = (old / wl - low) / (high - low)
-        blended = (1 - smooth) * inv / factor + smooth * inv
-        assert abs(blended / inv - want_ratio) < 1e-12
+    """A pair whose wavelength sits exactly on an edge of the medium band gets what the band
+    beyond that edge gets: unchanged at old/high, divided by the factor at old/low. The
+    original length is chosen so that pair j lies on the edge."""
+    d, theta, factor = 32, 500000.0, 8.0
+    base = P.rope_inv_freq(d, theta, None).astype(np.float64)
+    wl = 2 * math.pi / base
+    j = 6
+    for edge_factor, want in ((4.0, 1.0), (1.0, 1 / factor)):          # short edge: old/high; long edge: old/low
+        for nudge in (1 - 1e-9, 1.0, 1 + 1e-9):                        # just inside, on, just outside the band
+            rule = dict(factor=factor, low_freq_factor=1.0, high_freq_factor=4.0,
+                        original_max_position_embeddings=edge_factor * wl[j] * nudge)
+            got = float(P.rope_inv_freq(d, theta, rule)[j])
+            assert abs(got / base[j] - want) < 1e-6, (edge_factor, nudge)
 
 
 def test_rope_position_zero_is_identity_and_norms_are_kept():
@@ -197,6 +229,48 @@ def test_tied_head_equals_untied_copy_of_the_table(model_dirs, tmp_path):
     toks = [5, 17, 3, 200, 41]
     np.testing.assert_allclose(PlainLlama(src).logits(toks), PlainLlama(dst).logits(toks), rtol=1e-12)
     shutil.rmtree(dst)
+
+
+def test_a_layer_is_its_attention_half_followed_by_its_feed_forward_half(plain_models):
+    """The arrangement of a layer, pinned by what each half reduces to. With the output
+    projection zeroed a layer is h + mlp(norm2(h)); with the down projection zeroed it is
+    h + attention(norm1(h)); and the full layer is the second applied to the result of the
+    first. A feed-forward that reads the layer's input instead of the attention's result
+    (a parallel block), a norm after the sum instead of before the part, or a missing
+    residual path each break one of the three."""
+    import copy
+
+    m = plain_models["B"]
+    c = m.cfg
+    n = 21
+    h = rnd(n, c.hidden, seed=8)
+    cos, sin = P.rope_cos_sin(np.arange(n), m.inv_freq)
+    pre = "model.layers.1."
+
+    def variant(zeroed):
+        v = copy.copy(m)
+        v.w = dict(m.w)
+        v.w[pre + zeroed] = np.zeros_like(m.w[pre + zeroed])
+        return v
+
+    only_ff = variant("self_attn.o_proj.weight").layer(1, h, cos, sin)
+    want = h + P.swiglu_mlp(P.rms_norm(h, m.w[pre + "post_attention_layernorm.weight"], c.eps),
+                            m.w[pre + "mlp.gate_proj.weight"], m.w[pre + "mlp.up_proj.weight"], m.w[pre + "mlp.down_proj.weight"])
+    np.testing.assert_allclose(only_ff, want, rtol=1e-10, atol=1e-12)
+
+    only_attn = variant("mlp.down_proj.weight").layer(1, h, cos, sin)
+    x = P.rms_norm(h, m.w[pre + "input_layernorm.weight"], c.eps)
+    q = P.apply_rope((x @ m.w[pre + "self_attn.q_proj.weight"].T).reshape(n, c.heads, c.head_dim), cos, sin)
+    k = P.apply_rope((x @ m.w[pre + "self_attn.k_proj.weight"].T).reshape(n, c.kv_heads, c.head_dim), cos, sin)
+    v = (x @ m.w[pre + "self_attn.v_proj.weight"].T).reshape(n, c.kv_heads, c.head_dim)
+    want = h + P.causal_attention(q, k, v).reshape(n, -1) @ m.w[pre + "self_attn.o_proj.weight"].T
+    np.testing.assert_allclose(only_attn, want, rtol=1e-10, atol=1e-12)
+    assert np.abs(only_attn - h).max() > 1e-3 and np.abs(only_ff - h).max() > 1e-3
+
+    full = m.layer(1, h, cos, sin)
+    np.testing.assert_allclose(full, variant("self_attn.o_proj.weight").layer(1, only_attn, cos, sin), rtol=1e-10, atol=1e-12)
+    parallel = only_attn + only_ff - h
+    assert np.abs(full - parallel).max() > 1e-4
 
 
 def test_logits_do_not_depend_on_a_shift_of_all_positions(plain_models):
