@@ -75,6 +75,10 @@ def main() -> int:
     ap.add_argument("--decode-steps", type=int, default=8,
                     help="decode steps per scheduler round (the host reads the tokens once per round)")
     ap.add_argument("--prefill-reps", type=int, default=5, help="timed repetitions of the 2,048-token prefill")
+    ap.add_argument("--repeats", type=int, default=3,
+                    help="how often the timed region of K steps is run; the line reports the median repeat")
+    ap.add_argument("--long-context", type=int, default=16384,
+                    help="context of the extra decode point (0: skip it); its prompts fill all but 2,048 tokens of it")
     ap.add_argument("--no-peaks", action="store_true", help="skip measuring the copy bandwidth and a large library product")
     ap.add_argument("--model", default=None, help="use this model folder instead of writing random weights")
     ap.add_argument("--shape", choices=sorted(SHAPES), default="llama-3.2-1b", help="layer sizes of the random model")
@@ -116,61 +120,96 @@ def main() -> int:
     def sync() -> None:
         torch.cuda.synchronize()
 
-    def decode_run(batch: int, steps: int, warmup: int) -> dict:
-        sched = engine.make_scheduler(chunk_size=args.prompt_len, enable_prefix_cache=False)
+    def decode_run(engine, batch: int, steps: int, warmup: int, prompt_len: int, context: int, repeats: int = 1) -> dict:
+        """``repeats`` timed regions of exactly ``steps`` decode steps each, every one between two
+        device synchronisations; the result is the median region. Beside the host clock, the
+        device's own time per scheduler round (events on the stream around the round's
+        launches) and the host's shares: scheduling, packing the step's integers, commit."""
+        runner = engine.runner
+        sched = engine.make_scheduler(chunk_size=prompt_len, enable_prefix_cache=False)
         for b in range(batch):
-            sched.add_request(f"d{batch}-{b}", rng.integers(0, vocab, args.prompt_len), args.context - args.prompt_len - 1,
-                              ignore_eos=True)
+            sched.add_request(f"d{batch}-{b}", rng.integers(0, vocab, prompt_len), context - prompt_len - 1, ignore_eos=True)
         # prompts, untimed: one request's prompt per step
         while any(r.num_computed < len(r.prompt) for r in sched.requests()):
-            bt = sched.schedule_step(args.prompt_len, batch)
+            bt = sched.schedule_step(prompt_len, batch)
             sched.commit(bt, engine.step(bt))
         for _ in range(warmup):
-            bt = sched.schedule_step(args.prompt_len, batch)
+            bt = sched.schedule_step(prompt_len, batch)
             sched.commit(bt, engine.step(bt))
-        kv_start = sum(r.num_computed for r in sched.requests())
-        sync()
         clock = time.perf_counter
-        t0 = clock()
-        done = 0
-        in_schedule = in_commit = 0.0
-        while done < steps:
-            t1 = clock()
-            bt = sched.schedule_step(args.prompt_len, batch, min(args.decode_steps, steps - done))
-            assert len(bt.work) == batch and bt.num_tokens == batch
-            t2 = clock()
-            sampled = engine.step(bt)
-            t3 = clock()
-            sched.commit(bt, sampled)
-            in_schedule += t2 - t1
-            in_commit += clock() - t3
-            done += bt.decode_steps
-        sync()
-        dt = clock() - t0
-        kv_end = sum(r.num_computed for r in sched.requests())
+        in_pack = [0.0]
+        inner_pack = runner.packer.pack
+
+        def timed_pack(*a, **kw):
+            t = clock()
+            out = inner_pack(*a, **kw)
+            in_pack[0] += clock() - t
+            return out
+
+        runner.packer.pack = timed_pack
+        regions = []
+        for _ in range(repeats):
+            kv_start = sum(r.num_computed for r in sched.requests())
+            events = []
+            in_pack[0] = 0.0
+            sync()
+            t0 = clock()
+            done = 0
+            in_schedule = in_commit = 0.0
+            while done < steps:
+                t1 = clock()
+                bt = sched.schedule_step(prompt_len, batch, min(args.decode_steps, steps - done))
+                assert len(bt.work) == batch and bt.num_tokens == batch
+                t2 = clock()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                sampled = engine.step(bt)
+                e1.record()
+                t3 = clock()
+                sched.commit(bt, sampled)
+                in_schedule += t2 - t1
+                in_commit += clock() - t3
+                events.append((e0, e1))
+                done += bt.decode_steps
+            sync()
+            dt = clock() - t0
+            kv_end = sum(r.num_computed for r in sched.requests())
+            mean_kv_tokens = 0.5 * (kv_start + kv_end) + 0.5 * batch       # keys read per step, summed over requests
+            bytes_per_step = weight_bytes + mean_kv_tokens * kv_bytes_per_token
+            regions.append({"tok_s": batch * steps / dt, "ms_per_step": 1e3 * dt / steps,
+                            "gbs": bytes_per_step * steps / dt / 1e9, "kv_len": mean_kv_tokens / batch,
+                            "schedule_us": 1e6 * in_schedule / steps, "commit_us": 1e6 * in_commit / steps,
+                            "pack_us": 1e6 * in_pack[0] / steps,
+                            "device_us": 1e3 * sum(a.elapsed_time(b) for a, b in events) / steps})
+        runner.packer.pack = inner_pack
         for rid in [r.req_id for r in sched.requests()]:
             sched.free_request(rid)
-        mean_kv_tokens = 0.5 * (kv_start + kv_end) + 0.5 * batch       # keys read per step, summed over requests
-        bytes_per_step = weight_bytes + mean_kv_tokens * kv_bytes_per_token
-        return {"tok_s": batch * steps / dt, "ms_per_step": 1e3 * dt / steps,
-                "gbs": bytes_per_step * steps / dt / 1e9, "kv_len": mean_kv_tokens / batch,
-                "schedule_us": 1e6 * in_schedule / steps, "commit_us": 1e6 * in_commit / steps}
+        regions.sort(key=lambda r: r["ms_per_step"])
+        out = dict(regions[len(regions) // 2])
+        out["all_ms_per_step"] = [round(r["ms_per_step"], 4) for r in regions]
+        return out
 
-    def prefill_run(reps: int = 5, warm: int = 2) -> dict:
+    def prefill_run(reps: int = 5, warm: int = 2, portion: int | None = None) -> dict:
+        """A prompt of ``--prompt-len`` tokens in one step, or in steps of ``portion`` tokens
+        each over the cache the earlier portions left; the median of ``reps`` timings."""
         from prefixserve_amd.engine.batch import StepItem
 
         n = args.prompt_len
+        portion = portion or n
         table = [list(range(-(-n // 16)))]
         toks = rng.integers(0, vocab, n)
-        item = [StepItem("p", toks, 0, table, 0, [n - 1])]
-        for _ in range(warm):
-            runner.step(item)
-        sync()
-        t0 = time.perf_counter()
-        for _ in range(reps):
-            runner.step(item)
-        sync()
-        ms = 1e3 * (time.perf_counter() - t0) / reps
+        items = [[StepItem("p", toks[a:min(a + portion, n)], a, table, 0, [min(a + portion, n) - a - 1] if a + portion >= n else [])]
+                 for a in range(0, n, portion)]
+        times = []
+        for rep in range(warm + reps):
+            sync()
+            t0 = time.perf_counter()
+            for item in items:
+                runner.step(item)
+            sync()
+            if rep >= warm:
+                times.append(1e3 * (time.perf_counter() - t0))
+        ms = sorted(times)[len(times) // 2]
         flops = prefill_flops(cfg, layers, n)
         return {"value": n / (ms / 1e3), "tokens": n, "ms": ms,
                 "frac": flops / (ms / 1e3) / (MFMA_PEAK_TFLOPS[args.dtype] * 1e12)}
@@ -195,13 +234,30 @@ def main() -> int:
         return out
 
     prefill = prefill_run(reps=args.prefill_reps)
-    main_run = decode_run(args.batch, args.steps, args.warmup)
+    main_run = decode_run(engine, args.batch, args.steps, args.warmup, args.prompt_len, args.context, repeats=max(args.repeats, 1))
     points = {}
     if not args.no_points:
-        points["decode_b1"] = decode_run(1, max(16, args.steps // 2), max(4, args.warmup // 2))["tok_s"]
-        points["decode_b64"] = decode_run(64, max(16, args.steps // 4), max(4, args.warmup // 4))["tok_s"]
+        points["decode_b1"] = decode_run(engine, 1, max(16, args.steps // 2), max(4, args.warmup // 2), args.prompt_len,
+                                         args.context)["tok_s"]
+        points["decode_b64"] = decode_run(engine, 64, max(16, args.steps // 4), max(4, args.warmup // 4), args.prompt_len,
+                                          args.context)["tok_s"]
+        if args.prompt_len > 512:
+            points["prefill_portions_of_512"] = prefill_run(reps=3, warm=1, portion=512)["value"]
 
     peaks = {} if args.no_peaks else measured_peaks()      # last: a long product changes the clocks of what follows
+
+    if not args.no_points and args.long_context > args.context:
+        # The same batch over a long context, where the cache is most of what a step reads.
+        del runner
+        engine = None
+        torch.cuda.empty_cache()
+        ctx_len = args.long_context
+        engine = Engine(EngineConfig(model_path=model_dir, dtype=args.dtype, max_num_seqs=args.batch,
+                                     max_prefill_tokens=ctx_len - 2048, max_seq_len=ctx_len,
+                                     num_blocks=args.batch * (ctx_len // 16) + 64, use_graphs=not args.no_graphs))
+        long_run = decode_run(engine, args.batch, max(16, args.steps // 4), max(4, args.warmup // 4), ctx_len - 2048, ctx_len)
+        points[f"decode_b{args.batch}_context_{ctx_len}"] = long_run["tok_s"]
+        points[f"decode_b{args.batch}_context_{ctx_len}_hbm_frac"] = long_run["gbs"] / HBM_PEAK_GBS
 
     line = {
         "metric": "decode_tokens_per_second", "value": main_run["tok_s"], "unit": "tok/s", "n_gpus": 1,
@@ -214,15 +270,19 @@ def main() -> int:
             "intermediate": cfg["intermediate_size"], "vocab": vocab, "rope_theta": cfg["rope_theta"],
             "rope_factor": (cfg.get("rope_scaling") or {}).get("factor"), "rms_norm_eps": cfg["rms_norm_eps"],
             "tied": cfg.get("tie_word_embeddings", False), "global_batch": args.batch, "seq_len": args.context,
-            "prompt_len": args.prompt_len, "page_tokens": 16, "decode_steps": args.decode_steps, "parallelism": "none",
+            "prompt_len": args.prompt_len, "kv_len": round(main_run["kv_len"], 1), "page_tokens": 16,
+            "decode_steps": args.decode_steps, "parallelism": "none",
         },
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": main_run["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": main_run["gbs"] / HBM_PEAK_GBS},
         "points": points,
-        # host time per decode step inside ms_per_step: the scheduler's two calls (the rest is
-        # engine.step: packing, the device's work, the wait for the tokens)
-        "host_us_per_step": {"schedule": main_run["schedule_us"], "commit": main_run["commit_us"]},
+        # the timed region was run this often; the line is the median region
+        "repeats": {"count": max(args.repeats, 1), "ms_per_step": main_run["all_ms_per_step"]},
+        # per decode step inside ms_per_step: the device's own time (events around each round's
+        # launches) and the host's shares (the scheduler's two calls, packing the step's integers)
+        "us_per_step": {"device": main_run["device_us"], "schedule": main_run["schedule_us"], "pack": main_run["pack_us"],
+                        "commit": main_run["commit_us"]},
         "measured_peaks": peaks,
     }
     print(json.dumps(line), flush=True)

@@ -119,6 +119,11 @@ def core_module_name() -> str:
     return "_core" + (sysconfig.get_config_var("EXT_SUFFIX") or ".so")
 
 
+# Every warning is an error, in the module and in the check program alike.
+CORE_WARNINGS = ["-Wall", "-Wextra", "-Wshadow", "-Wconversion", "-Wsign-conversion", "-Werror"]
+SANITIZE_FLAGS = ["-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer", "-O1", "-g"]
+
+
 def build_core() -> Path:
     import pybind11
 
@@ -126,13 +131,26 @@ def build_core() -> Path:
     out = lib_dir() / core_module_name()
     tmp = out.with_suffix(out.suffix + f".tmp{os.getpid()}")
     cmd = [
-        gxx, "-O2", "-std=c++17", "-shared", "-fPIC", "-fvisibility=hidden",
-        "-Wall", "-Wextra", "-Wshadow", "-Wconversion", "-Wsign-conversion",
-        f"-I{sysconfig.get_paths()['include']}", f"-I{pybind11.get_include()}", f"-I{CSRC / 'core'}",
+        gxx, "-O2", "-std=c++17", "-shared", "-fPIC", "-fvisibility=hidden", *CORE_WARNINGS,
+        # Python's and pybind11's headers as system headers: their own warnings are not this package's errors.
+        "-isystem", sysconfig.get_paths()["include"], "-isystem", pybind11.get_include(), f"-I{CSRC / 'core'}",
         *[str(CSRC / s) for s in CORE_SOURCES], "-o", str(tmp),
     ]
     _run(cmd, "host cache core (g++)")
     os.replace(tmp, out)
+    return out
+
+
+def build_core_program(main_source: Path, out: Path, sanitize: bool = False) -> Path:
+    """A standalone program from ``main_source`` and the core's sources without the Python
+    bindings, for checks of the core that run without an interpreter: with ``sanitize`` the
+    address and undefined-behaviour sanitizers are compiled in (host code only; a sanitized
+    Python module would need the sanitizer's runtime loaded before the interpreter)."""
+    gxx = _find("g++", ["/usr/bin/g++"])
+    sources = [str(CSRC / s) for s in CORE_SOURCES if not s.endswith("bindings.cpp")]
+    cmd = [gxx, "-std=c++17", *CORE_WARNINGS, *(SANITIZE_FLAGS if sanitize else ["-O2"]), f"-I{CSRC / 'core'}",
+           str(main_source), *sources, "-o", str(out)]
+    _run(cmd, f"core check program{' (sanitizers)' if sanitize else ''}")
     return out
 
 

@@ -179,7 +179,8 @@ def round_bf16(x: np.ndarray) -> np.ndarray:
 class PlainLlama:
     """Whole-sequence forward from a model folder (config.json + model.safetensors)."""
 
-    def __init__(self, model_dir: str | Path, dtype: Any = np.float64, bf16: bool = False) -> None:
+    def __init__(self, model_dir: str | Path, dtype: Any = np.float64, bf16: bool = False,
+                 weights: dict[str, np.ndarray] | None = None) -> None:
         """``bf16``: round the result of every operation to bfloat16, as a library that runs
         the reference's model code in bfloat16 does (prefixserve/model/llama.py:105-126 with
         dtype=bfloat16; softmax and the norm's statistics stay float32, llama.py:63-69 and
@@ -190,7 +191,9 @@ class PlainLlama:
         if bf16:
             dtype = np.float32
         self.dtype = dtype
-        self.w = {k: v.astype(dtype) for k, v in read_safetensors(model_dir / "model.safetensors").items()}
+        # ``weights``: arrays another instance read from the same file (a large file is read once).
+        source = weights if weights is not None else read_safetensors(model_dir / "model.safetensors")
+        self.w = {k: v.astype(dtype, copy=False) for k, v in source.items()}
         self.inv_freq = rope_inv_freq(self.cfg.head_dim, self.cfg.theta, self.cfg.scaling)
 
     def _r(self, x: np.ndarray) -> np.ndarray:
@@ -268,6 +271,14 @@ class PlainLlama:
         if self.bf16:
             xf = h / np.sqrt(np.mean(h * h, axis=-1, keepdims=True) + np.float32(self.cfg.eps))
             return round_bf16(round_bf16(self.w["model.norm.weight"] * round_bf16(xf)) @ head.T)
+        return rms_norm(h, self.w["model.norm.weight"], self.cfg.eps) @ head.T
+
+    def logits_at(self, tokens: Any, rows: Any) -> np.ndarray:
+        """The rows ``rows`` of ``logits(tokens)`` without the others: the output matrix of a
+        large vocabulary is most of the work of a long sequence."""
+        assert not self.bf16
+        h = self.hidden(tokens)[np.asarray(rows, dtype=np.int64)]
+        head = self.w["model.embed_tokens.weight"] if self.cfg.tied else self.w["lm_head.weight"]
         return rms_norm(h, self.w["model.norm.weight"], self.cfg.eps) @ head.T
 
     def greedy(self, prompt: Any, steps: int) -> tuple[list[int], list[np.ndarray]]:
