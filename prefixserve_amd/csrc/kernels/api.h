@@ -76,29 +76,6 @@ int psamd_attention_decode(void* stream, const void* qkv, int q_stride, void* ou
                            const int32_t* item_end, const int32_t* table_off, const int32_t* block_ids, int hq,
                            int hkv, int head_dim, int nsplit, float scale, int window);
 
-// Every layer of a decode step of at most 16 requests (one token each, bfloat16) in one persistent kernel:
-// per layer RMSNorm + q/k/v + rotation + cache write, attention over the cache, output projection,
-// RMSNorm + gate/up + SiLU, down projection, the two projections added into `residual` (float32 [tokens, hidden],
-// holding the embeddings on entry and the last layer's output on return). `layers` is a device array of n_layers
-// records of psamd_decode_layers_layer_bytes() bytes (see FusedLayer in decode_fused.hip). table_off, block_ids and
-// write_slot are host arrays of n_groups device pointers, the step's block tables per layer group. `sync` is
-// psamd_decode_layers_sync_bytes() bytes of device memory, zero before the first call and left zero by every call
-// that ends well. Workgroups wait for each other inside the kernel; a wait of more than spin_limit polls ends it,
-// sets *error (device int) to non-zero and lets the kernel run out without waiting again: the results of such a
-// step are void and `sync` has to be zeroed before the next call. One call at a time per `sync`.
-// trace: NULL, or device memory for n_layers x 10 times (100 MHz counter) at which workgroup 0 ended each of a
-// layer's five phases and passed the barrier after it.
-int64_t psamd_decode_layers_sync_bytes(int max_tokens, int hkv);
-int psamd_decode_layers_layer_bytes(void);
-int psamd_decode_layers_supports(int tokens, int hidden, int inter, int hq, int hkv, int head_dim, int norm_dtype);
-int psamd_decode_layers(void* stream, const void* layers, int n_layers, float* residual, void* qkv, void* attn_out,
-                        void* act, float* part_o, float* part_ml, void* sync, int* error, const int32_t* positions,
-                        const int32_t* dec_items, const int32_t* item_start, const int32_t* item_end,
-                        const int32_t* const* table_off, const int32_t* const* block_ids,
-                        const int32_t* const* write_slot, int n_groups, int tokens, int hidden, int inter, int hq,
-                        int hkv, int head_dim, int norm_dtype, int nsplit, float scale, int64_t spin_limit,
-                        int64_t* trace);
-
 // out[r] = argmax (temperature[r] <= 0) or the inverse-CDF draw with uniform[r] in [0, 1).
 int64_t psamd_sample_scratch_floats(int rows);
 int psamd_sample(void* stream, const float* logits, const float* temperature, const float* uniform, int32_t* out,

@@ -182,7 +182,6 @@ class Engine:
                 self.logit_trace += [(w.req.req_id, w.start + j, host[i]) for i, w in enumerate(batch.work)]
             self.sampler.sample_into(logits, t_dev, u_dev[j], out_dev[j])
         rows = self.sampler.fetch(k, len(reqs))
-        self.runner.raise_on_device_error()
         return {r.req_id: [rows[j][i] for j in range(k)] for i, r in enumerate(reqs)}
 
     def step(self, batch: Batch) -> dict[str, int]:
@@ -221,7 +220,6 @@ class Engine:
         seeds = [uniform_for(self.cfg.sample_seed ^ r.seed, request_key(r.req_id), len(r.output)) if r.temperature > 0
                  else 0.0 for r in sampling]
         tokens = self.sampler.sample(logits, temps, seeds)
-        self.runner.raise_on_device_error()
         return {r.req_id: t for r, t in zip(sampling, tokens)}
 
 

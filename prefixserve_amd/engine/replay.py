@@ -75,7 +75,6 @@ class TraceReplayer:
         out = None
         if logits is not None:
             out = logits.detach().to("cpu").numpy().astype(np.float32, copy=True)
-        self.runner.raise_on_device_error()
         for rid in step.get("end", []):
             st = self.live.pop(rid, None)
             if st is None:

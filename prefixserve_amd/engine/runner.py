@@ -163,17 +163,5 @@ class ModelRunner:
             ctx.token_ids.copy_(token_feed)
         return self.model.step(ctx)
 
-    @torch.inference_mode()
-    def raise_on_device_error(self) -> None:
-        """Raises if a kernel of the steps since the last call reported that it gave up (only the
-        fused decode step can); to be called where the host waits for a step's results anyway."""
-        check = getattr(self.ops, "raise_on_device_error", None)
-        if check is not None:
-            try:
-                check()
-            except Exception as e:
-                self._graphs.clear()
-                raise EngineError(str(e)) from e
-
     def pack(self, items: Sequence[StepItem]) -> StepContext:
         return self.packer.pack(items)

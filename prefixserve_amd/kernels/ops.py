@@ -12,7 +12,6 @@ from __future__ import annotations
 
 import contextlib
 import ctypes
-import os
 from typing import Any
 
 import torch
@@ -56,9 +55,6 @@ _SIGNATURES = {
     "psamd_attention_decode": [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32,
                                _i32, _f32, _i32],
     "psamd_sample": [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32],
-    "psamd_decode_layers_supports": [_i32, _i32, _i32, _i32, _i32, _i32, _i32],
-    "psamd_decode_layers": [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
-                            _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i64, _vp],
 }
 
 
@@ -80,17 +76,7 @@ class HipOps:
         self.lib.psamd_last_error.restype = ctypes.c_char_p
         self.lib.psamd_sample_scratch_floats.argtypes = [ctypes.c_int]
         self.lib.psamd_sample_scratch_floats.restype = ctypes.c_int64
-        self.lib.psamd_decode_layers_sync_bytes.argtypes = [_i32, _i32]
-        self.lib.psamd_decode_layers_sync_bytes.restype = ctypes.c_int64
         self.ws = workspace
-        # The layers of a small decode step in one kernel (see ``decode_layers``); with
-        # PREFIXSERVE_AMD_FUSED_DECODE=0 every layer runs kernel by kernel.
-        self.fused_decode = os.environ.get("PREFIXSERVE_AMD_FUSED_DECODE", "0") != "0"
-        self.fused_spin_limit = 1 << 20
-        self.fused_trace: torch.Tensor | None = None     # int64 [layers, 10]: set to have workgroup 0 note its times
-        self._fused_sync: torch.Tensor | None = None
-        self._fused_error: torch.Tensor | None = None
-        self._fused_unchecked = False
         self._sample_scratch: torch.Tensor | None = None
         self._step_stream: int | None = None
         self._slice_views: dict[tuple, tuple] = {}      # (name, slices, rows) -> (buffer, its [slices, rows, N] view)
@@ -332,73 +318,6 @@ class HipOps:
         self._ok(self.lib.psamd_attention_generic(
             s, qkv.data_ptr(), stride, out.data_ptr(), kv.data_ptr(), _code(qkv.dtype), t, ctx.positions.data_ptr(),
             ctx.tok_item.data_ptr(), g.table_off.data_ptr(), g.block_ids.data_ptr(), hq, hkv, d, scale, win))
-
-    # ------------------------------------------------------- fused decode step
-
-    FUSED_MAX_TOKENS = 16
-
-    def decode_layers_supported(self, tokens: int, hidden: int, inter: int, hq: int, hkv: int, d: int,
-                                norm_dtype: torch.dtype) -> bool:
-        return self.fused_decode and bool(self.lib.psamd_decode_layers_supports(tokens, hidden, inter, hq, hkv, d,
-                                                                                _code(norm_dtype)))
-
-    def decode_layers(self, plan: Any, residual: torch.Tensor, ctx: Any) -> None:
-        """Every layer of ``plan`` (``parts.model.FusedDecodePlan``) on a step in which each item
-        brings one token: ``residual`` holds the embeddings on entry and the last layer's output on
-        return. One persistent kernel whose workgroups wait for each other between a layer's
-        phases; a wait that runs out sets a flag that ``raise_on_device_error`` reports."""
-        t, h = residual.shape
-        self._need(ctx.num_tokens == t and ctx.num_decode == t and ctx.num_items == t and 0 < t <= self.FUSED_MAX_TOKENS,
-                   "decode_layers: every item must bring exactly one token, at most 16 items")
-        self._need(residual.dtype == torch.float32 and residual.is_contiguous() and h == plan.hidden, "decode_layers: residual")
-        hq, hkv, d, inter = plan.hq, plan.hkv, plan.d, plan.inter
-        if self._fused_sync is None:
-            n = int(self.lib.psamd_decode_layers_sync_bytes(self.FUSED_MAX_TOKENS, 1024))
-            self._fused_sync = torch.zeros(n, dtype=torch.uint8, device=self.device)
-            self._fused_error = torch.zeros(1, dtype=torch.int32, device=self.device)
-            self._fused_error_host = torch.zeros(1, dtype=torch.int32, pin_memory=True)
-        self._need(hkv <= 1024, "decode_layers: too many kv heads")
-        kv_len = self.fixed_kv_len or ctx.max_kv_len
-        pairs = t * hkv
-        nsplit = 1 if pairs >= 256 else max(1, min(64, 512 // pairs, -(-kv_len // 128)))
-        parts = max(t * nsplit, 512 // hkv)
-        ws = self.ws
-        m = self.FUSED_MAX_TOKENS
-        qkv = ws.get("fused.qkv", (m, (hq + 2 * hkv) * d), torch.bfloat16)
-        attn = ws.get("fused.attn", (m, hq * d), torch.bfloat16)
-        act = ws.get("fused.act", (m, inter), torch.bfloat16)
-        part_o = ws.get("attn.part_o", (parts * hq * d,), torch.float32)
-        part_ml = ws.get("attn.part_ml", (parts * hq * 2,), torch.float32)
-        ng = len(ctx.groups)
-        self._need(max(plan.groups) < ng <= 4, "decode_layers: layer groups")
-        arr = ctypes.c_void_p * ng
-        offs = arr(*[g.table_off.data_ptr() for g in ctx.groups])
-        bids = arr(*[g.block_ids.data_ptr() for g in ctx.groups])
-        slots = arr(*[g.write_slot.data_ptr() for g in ctx.groups])
-        self._fused_unchecked = True
-        self._ok(self.lib.psamd_decode_layers(
-            self._stream(), plan.layers.data_ptr(), plan.n_layers, residual.data_ptr(), qkv.data_ptr(), attn.data_ptr(),
-            act.data_ptr(), part_o.data_ptr(), part_ml.data_ptr(), self._fused_sync.data_ptr(), self._fused_error.data_ptr(),
-            ctx.positions.data_ptr(), ctx.dec_items.data_ptr(), ctx.item_start.data_ptr(), ctx.item_end.data_ptr(),
-            ctypes.cast(offs, ctypes.c_void_p), ctypes.cast(bids, ctypes.c_void_p), ctypes.cast(slots, ctypes.c_void_p),
-            ng, t, h, inter, hq, hkv, d, _code(plan.norm_dtype), nsplit, plan.scale, self.fused_spin_limit,
-            _ptr(self.fused_trace)))
-
-    def raise_on_device_error(self) -> None:
-        """Raises if a kernel reported that it could not finish (a wait between workgroups that
-        ran out): the results of the steps since the last call are void. Waits for the stream;
-        costs nothing when no such kernel ran since the last call."""
-        if not self._fused_unchecked:
-            return
-        self._fused_unchecked = False
-        self._fused_error_host.copy_(self._fused_error, non_blocking=True)
-        torch.cuda.current_stream(self.device).synchronize()
-        code = int(self._fused_error_host[0])
-        if code:
-            self._fused_error.zero_()
-            self._fused_sync.zero_()
-            raise KernelError(f"the fused decode step gave up waiting for its workgroups (code {code}); "
-                              "its results are void. PREFIXSERVE_AMD_FUSED_DECODE=0 runs the layers kernel by kernel")
 
     # ---------------------------------------------------------------- sampling
 

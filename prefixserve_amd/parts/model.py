@@ -4,8 +4,6 @@ scheduler's engine and trace replay all call ``DecoderModel.step``."""
 
 from __future__ import annotations
 
-import struct
-from dataclasses import dataclass
 from typing import TYPE_CHECKING, Any, Mapping
 
 import torch
@@ -20,24 +18,6 @@ from .spec import ModelSpec
 
 if TYPE_CHECKING:
     from prefixserve_amd.engine.batch import StepContext
-
-
-@dataclass
-class FusedDecodePlan:
-    """The layer runs of a model as the fused decode step reads them: one record per run in
-    device memory (``FusedLayer`` in csrc/kernels/decode_fused.hip) and the sizes all runs share."""
-
-    layers: torch.Tensor       # uint8 [n_layers * record size] on the device
-    n_layers: int
-    hidden: int
-    inter: int
-    hq: int
-    hkv: int
-    d: int
-    scale: float
-    norm_dtype: torch.dtype
-    groups: tuple[int, ...]
-    keep: tuple                # the tensors the records point to
 
 
 class DecoderModel:
@@ -58,7 +38,6 @@ class DecoderModel:
         self.caches: dict[int, Any] = {}
         self.states: dict[int, torch.Tensor] = {}
         self.rt: Runtime | None = None
-        self._fused_plan: FusedDecodePlan | None | bool = False
 
     # ---------------------------------------------------------------- weights
 
@@ -132,43 +111,6 @@ class DecoderModel:
     def attach(self, caches: Mapping[int, Any], states: Mapping[int, torch.Tensor]) -> None:
         self.caches = dict(caches)
         self.states = dict(states)
-        self._fused_plan: FusedDecodePlan | None | bool = False        # False: not looked at yet
-
-    def fused_decode_plan(self) -> FusedDecodePlan | None:
-        """The plan for running all layers of a small decode step in one kernel, or None if
-        some layer is not of the kind that kernel runs (another mixer, a window, state, sizes
-        that differ between layers, a dtype other than bfloat16)."""
-        if self._fused_plan is not False:
-            return self._fused_plan
-        self._fused_plan = None
-        rt = self.rt
-        if rt is None or rt.dtype != torch.bfloat16 or self.states or not hasattr(rt.ops, "decode_layers"):
-            return None
-        descs = []
-        for run in self.spec.order:
-            blk = self.blocks[run.layer]
-            desc = blk.fused_decode_layer(self.caches.get(run.cache), run.writes_cache) if hasattr(blk, "fused_decode_layer") else None
-            if desc is None:
-                return None
-            descs.append(desc)
-        first = descs[0]
-        shared = ("hq", "hkv", "d", "scale", "inter", "hidden")
-        if any(d[k] != first[k] for d in descs for k in shared) or any(d["norm1"].dtype != first["norm1"].dtype for d in descs):
-            return None
-        if not rt.ops.decode_layers_supported(1, first["hidden"], first["inter"], first["hq"], first["hkv"], first["d"],
-                                              first["norm1"].dtype):
-            return None
-        code = 1 if first["norm1"].dtype == torch.bfloat16 else 0
-        ptr = lambda t: 0 if t is None else t.data_ptr()
-        raw = b"".join(struct.pack("<8Q2f4i", ptr(d["w_qkv"]), ptr(d["w_o"]), ptr(d["w_gate_up"]), ptr(d["w_down"]),
-                                   ptr(d["norm1"]), ptr(d["norm2"]), ptr(d["kv"]), ptr(d["rope"]), d["eps1"], d["eps2"],
-                                   code, d["group"], int(d["writes_cache"]), 0) for d in descs)
-        layers = torch.frombuffer(bytearray(raw), dtype=torch.uint8).to(rt.device)
-        keep = tuple(t for d in descs for t in d.values() if isinstance(t, torch.Tensor))
-        self._fused_plan = FusedDecodePlan(layers, len(descs), first["hidden"], first["inter"], first["hq"], first["hkv"],
-                                           first["d"], float(first["scale"]), first["norm1"].dtype,
-                                           tuple(d["group"] for d in descs), keep)
-        return self._fused_plan
 
     # ------------------------------------------------------------------- step
 
@@ -185,14 +127,9 @@ class DecoderModel:
             residual = ws.get("residual", (t, s.hidden_size), torch.float32)
             ops.embed(ctx.token_ids, self.embedding, residual)
             pending = None
-            plan = self.fused_decode_plan() if ctx.num_decode == t == ctx.num_items else None
-            if plan is not None and ops.decode_layers_supported(t, plan.hidden, plan.inter, plan.hq, plan.hkv, plan.d,
-                                                                 plan.norm_dtype):
-                ops.decode_layers(plan, residual, ctx)       # every layer, added into the residual
-            else:
-                for i, run in enumerate(s.order):
-                    pending = self.blocks[run.layer].forward(residual, pending, ctx, self.caches.get(run.cache),
-                                                             self.states.get(i), run.writes_cache)
+            for i, run in enumerate(s.order):
+                pending = self.blocks[run.layer].forward(residual, pending, ctx, self.caches.get(run.cache),
+                                                         self.states.get(i), run.writes_cache)
             if ctx.num_logit_rows == 0:
                 return None
             x = self.final_norm.add_norm_rows(residual, pending, ctx.logit_rows, "final.x")
