@@ -720,6 +720,11 @@ __global__ __launch_bounds__(64) void attn_decode_merge_kernel(
   const bool has = lane < nsplit;                       // nsplit <= 64
   const float ms = has ? part_ml[(base + lane) * 2] : -INFINITY;
   const float ls = has ? part_ml[(base + lane) * 2 + 1] : 0.f;
+  // The first splits' partial outputs are asked for together with the statistics, not after them.
+  constexpr int kEarly = 8;
+  float early[kEarly];
+#pragma unroll
+  for (int s = 0; s < kEarly; ++s) early[s] = (s < nsplit && lane < d) ? part_o[(base + s) * d + lane] : 0.f;
   const float mm = wave_max(ms);
   const float w = ms == -INFINITY ? 0.f : __expf(ms - mm);
   const float ll = wave_sum(w * ls);
@@ -727,8 +732,14 @@ __global__ __launch_bounds__(64) void attn_decode_merge_kernel(
   __syncthreads();
   for (int i = lane; i < d; i += kWave) {
     float acc = 0.f;
+    int s0 = 0;
+    if (i == lane) {
+#pragma unroll
+      for (int s = 0; s < kEarly; ++s) acc += (s < nsplit ? wgt_s[s] : 0.f) * early[s];
+      s0 = kEarly;
+    }
 #pragma unroll 8
-    for (int s = 0; s < nsplit; ++s) acc += wgt_s[s] * part_o[(base + s) * d + i];
+    for (int s = s0; s < nsplit; ++s) acc += wgt_s[s] * part_o[(base + s) * d + i];
     out[t * (static_cast<int64_t>(hq) * d) + h * d + i] = float_to_bf16(acc);
   }
 }

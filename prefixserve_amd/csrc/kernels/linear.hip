@@ -420,6 +420,26 @@ __global__ __launch_bounds__(64 * WV) void qkv_rope_append_kernel(
   for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
     for (int i = 0; i < MT; ++i) acc[rt][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // What the finishing waves (wave < MT: one 16-token tile each) need from memory after the
+  // product is asked for now, so that it arrives behind the weights instead of after them: the
+  // token's position, its rotation (a second, dependent trip) and its cache slot.
+  float2 cs_early[RT][4];
+  int slot_early = 0;
+  if (wave < MT) {
+    const int mc = min(wave * 16 + r, M - 1);
+    const int pos = positions[mc];
+    if (kv != nullptr) slot_early = write_slot[mc];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      const int t = min(static_cast<int>(blockIdx.x) * RT + rt, n_tiles - 1);
+      const int head = t / tiles_per_head;
+      const int p = (t - head * tiles_per_head) << 3;
+      const bool rotate = table != nullptr && head < hq + hkv;
+#pragma unroll
+      for (int v = 0; v < 4; ++v)
+        cs_early[rt][v] = rotate ? table[static_cast<int64_t>(pos) * half + p + 4 * (g & 1) + v] : float2{1.f, 0.f};
+    }
+  }
   const int s_full = K >> 5;
   constexpr int U = MT == 1 ? 8 : (MT * RT <= 2 ? 4 : 2);   // steps whose loads are in flight together
   for (int base = wave; base < s_full; base += WV * U) {
@@ -477,18 +497,12 @@ __global__ __launch_bounds__(64 * WV) void qkv_rope_append_kernel(
     const int m = mt * 16 + r;
     const int mc = min(m, M - 1);
     const bool second = g >= 2;
-    const bool rotate = table != nullptr && head < hq + hkv;
-    const int pos = positions[mc];
     f32x4 res;
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
       const float other = __shfl_xor(own[v], 32, kWave);              // the pair's other half
-      float val = own[v];
-      if (rotate) {
-        const float2 cs = table[static_cast<int64_t>(pos) * half + p + 4 * (g & 1) + v];
-        val = second ? own[v] * cs.x + other * cs.y : own[v] * cs.x - other * cs.y;
-      }
-      res[v] = val;
+      const float2 cs = cs_early[rt][v];                              // (1, 0) where nothing rotates
+      res[v] = second ? own[v] * cs.x + other * cs.y : own[v] * cs.x - other * cs.y;
     }
     if (m >= M) continue;
     const int e0 = (second ? half : 0) + p + 4 * (g & 1);              // element of the head, 4 consecutive
@@ -499,7 +513,7 @@ __global__ __launch_bounds__(64 * WV) void qkv_rope_append_kernel(
     pk.w = float_to_bf16(res[3]);
     *reinterpret_cast<ushort4*>(qkv_out + static_cast<int64_t>(m) * ((hq + 2 * hkv) * d) + head * d + e0) = pk;
     if (kv == nullptr || head < hq) continue;
-    const int slot = write_slot[m];
+    const int slot = slot_early;
     const int64_t page_elems = 2LL * hkv * kPage * d;
     bf16_t* page = kv + static_cast<int64_t>(slot / kPage) * page_elems;
     const int off = slot % kPage;

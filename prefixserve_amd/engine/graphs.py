@@ -20,6 +20,7 @@ either is reallocated (their ``version`` changes) the graph is dropped and captu
 
 from __future__ import annotations
 
+import gc
 from typing import TYPE_CHECKING, Any, Sequence
 
 import torch
@@ -52,8 +53,19 @@ def graphed_decode_step(runner: "ModelRunner", items: Sequence[StepItem], token_
         versions = (packer.version, ws.version)
         torch.cuda.synchronize(runner.device)
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            captured = runner.model.step(ctx)
+        # No garbage collection while the stream is capturing: a collection that runs in the
+        # middle of it may destroy what an earlier runner left behind (its graphs, their memory
+        # pools), and releasing those is not allowed during a capture: the process aborts.
+        # What is unreachable now is collected before, the rest after.
+        gc.collect()
+        gc_was_on = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(graph):
+                captured = runner.model.step(ctx)
+        finally:
+            if gc_was_on:
+                gc.enable()
         if (packer.version, ws.version) != versions:
             return logits      # something grew during capture; try again on a later step
         runner._graphs[key] = (graph, captured, versions)
