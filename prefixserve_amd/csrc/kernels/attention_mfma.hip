@@ -50,6 +50,18 @@ __device__ __forceinline__ bf16x8 join(bf16x4 a, bf16x4 b) {
   return r;
 }
 
+// Values of keys no query of the tile can see get probability zero, but zero times what lies in
+// a slot nobody of this request has written (the rest of its last page, a page a window gave
+// back and somebody else took) is NaN if that is a NaN or an infinity: such values are set to
+// zero in the tiles that touch those slots. `keep(e)` tells whether element e's key is visible.
+template <typename Keep>
+__device__ __forceinline__ bf16x8 zero_unless(bf16x8 v, Keep keep) {
+#pragma unroll
+  for (int e = 0; e < 8; ++e)
+    if (!keep(e)) v[e] = static_cast<__bf16>(0.f);
+  return v;
+}
+
 // ------------------------------------------------------------------ prefill
 
 // NS = D / 16. A workgroup owns 32 consecutive queries of one item and one query head; its
@@ -92,7 +104,8 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
   const int last_pos = pos0 + min(q_off + 31, n - 1);
   const int max_key = pos0 + n - 1;
   const int k_lo_q = window > 0 ? max(0, q_pos - window + 1) : 0;
-  const int k_begin = window > 0 ? (max(0, first_pos - window + 1) & ~31) : 0;
+  const int k_begin_vis = window > 0 ? max(0, first_pos - window + 1) : 0;   // the first key any query of the tile sees
+  const int k_begin = k_begin_vis & ~31;
   const float c = scale * 1.44269504088896340736f;  // scores are exponentiated in base 2
   {
     const int32_t* gtable = block_ids + table_off[item];
@@ -136,6 +149,16 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
         const bf16_t* vr = vp + min(32 * dt + col, D - 1) * kPage;
         t.v[cpage][dt] = join(ld4(vr), ld4(vr + 8));
       }
+    }
+    if (k0 + 31 > max_key || k0 < k_begin_vis) {
+#pragma unroll
+      for (int cpage = 0; cpage < 2; ++cpage)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+          t.v[cpage][dt] = zero_unless(t.v[cpage][dt], [&](int e) {
+            const int key = k0 + 16 * cpage + 8 * (e >> 2) + 4 * hi + (e & 3);
+            return key <= max_key && key >= k_begin_vis;
+          });
     }
   };
   auto compute = [&](const Tile& t, int k0) {
@@ -328,7 +351,9 @@ __global__ __launch_bounds__(256 * KP) void attn_prefill_grouped_kernel(
   const int first_pos = pos0 + q_off;
   const int last_pos = pos0 + min(q_off + 31, n - 1);
   const int k_lo_q = window > 0 ? max(0, q_pos - window + 1) : 0;
-  const int k_begin = window > 0 ? (max(0, first_pos - window + 1) & ~(KEYS - 1)) : 0;
+  const int max_key = pos0 + n - 1;
+  const int k_begin_vis = window > 0 ? max(0, first_pos - window + 1) : 0;   // the first key any query of the tile sees
+  const int k_begin = k_begin_vis & ~(KEYS - 1);
   const float c = scale * 1.44269504088896340736f;  // scores are exponentiated in base 2
   {
     const int32_t* gtable = block_ids + table_off[item];
@@ -371,9 +396,10 @@ __global__ __launch_bounds__(256 * KP) void attn_prefill_grouped_kernel(
       }
     }
   };
-  auto store_lds = [&](const Pieces& r, int stage) {
+  auto store_lds = [&](const Pieces& r, int stage, int k0) {
     bf16_t* kd = k_lds + stage * K_STAGE;
     bf16_t* vd = v_lds + stage * V_STAGE;
+    const bool edge = k0 + KEYS - 1 > max_key || k0 < k_begin_vis;   // slots nobody of this request wrote
 #pragma unroll
     for (int i = 0; i < CPT; ++i) {
       const int p = threadIdx.x + THREADS * i;
@@ -381,9 +407,18 @@ __global__ __launch_bounds__(256 * KP) void attn_prefill_grouped_kernel(
         const int key = p / (D / 8), part = p - key * (D / 8);
         *reinterpret_cast<uint4*>(kd + key * KS + 8 * part) = r.k[i];
         const int row = p >> 1, half = p & 1;                     // row = page * D + d
+        uint4 v = r.v[i];
+        if (edge) {
+          const int key0 = k0 + 16 * (row / D) + 8 * half;        // the piece holds the values of keys key0 .. key0 + 7
+          uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (key0 + e > max_key || key0 + e < k_begin_vis) w[e >> 1] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
+          v = uint4{w[0], w[1], w[2], w[3]};
+        }
         uint2* dst = reinterpret_cast<uint2*>(vd + row * VS + 8 * half);
-        dst[0] = uint2{r.v[i].x, r.v[i].y};
-        dst[1] = uint2{r.v[i].z, r.v[i].w};
+        dst[0] = uint2{v.x, v.y};
+        dst[1] = uint2{v.z, v.w};
       }
     }
   };
@@ -463,7 +498,7 @@ __global__ __launch_bounds__(256 * KP) void attn_prefill_grouped_kernel(
     load_global(ra, k0);
     load_global(rb, k0 + KEYS);
     while (true) {
-      store_lds(ra, stage);
+      store_lds(ra, stage, k0);
       load_global(ra, k0 + 2 * KEYS);
       // Every wave is past the iteration that last used this stage: it had to finish it to
       // reach the previous barrier.
@@ -472,7 +507,7 @@ __global__ __launch_bounds__(256 * KP) void attn_prefill_grouped_kernel(
       stage ^= 1;
       k0 += KEYS;
       if (k0 > last_pos) break;
-      store_lds(rb, stage);
+      store_lds(rb, stage, k0);
       load_global(rb, k0 + 2 * KEYS);
       __syncthreads();
       compute(stage, k0);
@@ -617,6 +652,14 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
     for (int ds = 0; ds < NS; ++ds) {
       const int drow = 16 * ds + r;
       va[ds] = join(ld4(vp0 + drow * kPage), ld4(vp1 + drow * kPage));
+    }
+    if (k0 + 31 > pos || k0 < k_lo) {
+#pragma unroll
+      for (int ds = 0; ds < NS; ++ds)
+        va[ds] = zero_unless(va[ds], [&](int e) {
+          const int key = k0 + 16 * (e >> 2) + 4 * g4 + (e & 3);
+          return key <= pos && key >= k_lo;
+        });
     }
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
