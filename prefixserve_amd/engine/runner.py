@@ -57,9 +57,9 @@ class ModelRunner:
             self.ops.ws = self.workspace
         self.rt = Runtime(self.device, self.dtype, self.ops, self.workspace)
 
-        tensors = load_weights(model_dir, self.model.weights(), self.spec.ignored_weights)
-        self.model.bind(tensors, self.rt, self.max_seq_len)
-        del tensors
+        # Read tensor by tensor as the parts bind: the host never holds the whole checkpoint.
+        with load_weights(model_dir, self.model.weights(), self.spec.ignored_weights) as tensors:
+            self.model.bind(tensors, self.rt, self.max_seq_len)
         logger.info("weights bound: %.2f GB read per decode step", self.model.step_weight_bytes() / 1e9)
 
         self.layer_groups = plan_groups(self.model.cache_needs())

@@ -1,8 +1,9 @@
 """Weights from safetensors by tensor name.
 
-Tensors are read one at a time across shards (``model.safetensors.index.json`` or a
-single ``model.safetensors``; prefixserve/model/weights.py:62-70 of the reference) and kept
-as stored: bfloat16 stays bfloat16, a tensor stored in 32-bit stays 32-bit, integer tables
+The whole checkpoint is checked against what the model wants from the files' headers alone;
+tensors are then read one at a time, when a part asks for them, across shards
+(``model.safetensors.index.json`` or a single ``model.safetensors``;
+prefixserve/model/weights.py:62-70 of the reference) and kept as stored: bfloat16 stays bfloat16, a tensor stored in 32-bit stays 32-bit, integer tables
 become int32, other float widths are widened to float32. Everything that is wrong with a
 checkpoint is reported in ONE error that lists missing tensors, unexpected tensors and
 wrong shapes (the reference stops at the first, weights.py:91-96,137-143).
@@ -51,12 +52,45 @@ def _as_kept(t: torch.Tensor) -> torch.Tensor:
     return t.to(torch.int32)
 
 
+class CheckpointTensors(Mapping[str, torch.Tensor]):
+    """name -> tensor on the host, read from its file when asked for and not kept: a part that
+    binds takes its tensors to the device and lets go of the host copies, so the host holds
+    one part's tensors at a time, not the checkpoint (the reference reads tensor by tensor for
+    the same reason, prefixserve/model/weights.py:9-12). ``close()`` lets go of the files."""
+
+    def __init__(self, stack: ExitStack, where: Mapping[str, object], names: Sequence[str]) -> None:
+        self._stack, self._where, self._names = stack, where, list(names)
+        self._wanted = frozenset(self._names)
+
+    def __getitem__(self, name: str) -> torch.Tensor:
+        if name not in self._where or name not in self._wanted:
+            raise KeyError(name)
+        return _as_kept(self._where[name].get_tensor(name))  # type: ignore[attr-defined]
+
+    def __iter__(self):
+        return iter(self._names)
+
+    def __len__(self) -> int:
+        return len(self._names)
+
+    def close(self) -> None:
+        self._stack.close()
+        self._where = {}
+
+    def __enter__(self) -> "CheckpointTensors":
+        return self
+
+    def __exit__(self, *exc) -> None:
+        self.close()
+
+
 def load_weights(model_dir: str | Path, wanted: Mapping[str, WeightWant],
-                 ignored_suffixes: Sequence[str] = ()) -> dict[str, torch.Tensor]:
-    """name -> tensor (on the host) for every wanted name, after checking the whole
-    checkpoint against ``wanted``."""
+                 ignored_suffixes: Sequence[str] = ()) -> CheckpointTensors:
+    """name -> tensor (on the host, read on demand) for every wanted name, after checking the
+    whole checkpoint against ``wanted``: names and shapes come from the files' headers."""
     model_dir = Path(model_dir)
-    with ExitStack() as stack:
+    stack = ExitStack()
+    try:
         where: dict[str, object] = {}
         for f in shard_files(model_dir):
             if not f.exists():
@@ -85,5 +119,7 @@ def load_weights(model_dir: str | Path, wanted: Mapping[str, WeightWant],
                 lines.append(f"  wrong shape ({len(wrong)}): " + ", ".join(
                     f"{n} is {list(got)}, expected {list(exp)}" for n, got, exp in sorted(wrong)))
             raise WeightLoadError("\n".join(lines), missing, unexpected, wrong)
-
-        return {name: _as_kept(where[name].get_tensor(name)) for name in wanted}  # type: ignore[attr-defined]
+        return CheckpointTensors(stack, where, list(wanted))
+    except BaseException:
+        stack.close()
+        raise

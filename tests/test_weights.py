@@ -102,3 +102,27 @@ def test_sharded_checkpoint_and_no_weights(tmp_path):
     empty.mkdir()
     with pytest.raises(WeightLoadError, match="no safetensors"):
         load_weights(empty, want)
+
+
+def test_tensors_are_read_when_asked_for_and_not_kept(tmp_path):
+    """The loader checks the checkpoint from the headers and hands out a mapping that reads a
+    tensor from its file on every access (the host never holds the whole checkpoint); closed,
+    it lets go of the files."""
+    from configs import TINY
+    from prefixserve_amd.config import read_model_dir
+    from prefixserve_amd.parts import DecoderModel
+
+    d = write_random_model(tmp_path, TINY["A"], seed=3, std=0.1)
+    arch, cfg, _ = read_model_dir(d)
+    spec = arch.build_spec(cfg)
+    want = DecoderModel(spec).weights()
+    got = load_weights(d, want, spec.ignored_weights)
+    assert not isinstance(got, dict) and set(got) == set(want) and len(got) == len(want)
+    name = "model.layers.0.mlp.down_proj.weight"
+    first, second = got[name], got[name]
+    assert first is not second and torch.equal(first, second)
+    with pytest.raises(KeyError):
+        got["no.such.tensor"]
+    got.close()
+    with pytest.raises(KeyError):
+        got[name]
