@@ -50,7 +50,6 @@ PackLayout plan_step(const std::vector<PackItem>& items, const std::vector<PackG
       lay.decode_items += 1;
     } else {
       lay.prefill_tiles += ceil_div(n, lim.prefill_tile);
-      lay.prefill_prefix += it.start;
     }
     lay.pages += lim.static_pages >= 0 ? lim.static_pages : pages;
     lay.max_kv_len = std::max(lay.max_kv_len, end);

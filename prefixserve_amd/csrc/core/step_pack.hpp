@@ -53,7 +53,6 @@ struct PackLayout {
   int64_t total = 0;
   int64_t tokens = 0, items = 0, logit_rows = 0, decode_items = 0, prefill_tiles = 0, pages = 0;
   int64_t max_kv_len = 0;
-  int64_t prefill_prefix = 0;   // tokens already cached in front of the step's portions (items of more than one token)
   // offsets into the buffer, in 32-bit words
   int64_t token_ids = 0, positions = 0, tok_item = 0, item_start = 0, item_pos0 = 0, item_end = 0, slots = 0;
   int64_t logit_rows_off = 0, dec_items = 0, pf_tiles = 0;

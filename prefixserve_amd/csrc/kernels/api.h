@@ -66,7 +66,7 @@ int psamd_attention_generic(void* stream, const void* qkv, int q_stride, void* o
 int psamd_attention_mfma_supports(int hq, int hkv, int head_dim);
 
 int psamd_attention_prefill(void* stream, const void* qkv, int q_stride, void* out, const void* kv,
-                            const int32_t* pf_tiles, int n_tiles, int max_kv_len, int64_t prefix_tokens,
+                            const int32_t* pf_tiles, int n_tiles, int max_kv_len,
                             const int32_t* item_start, const int32_t* item_pos0,
                             const int32_t* table_off, const int32_t* block_ids, int hq, int hkv, int head_dim,
                             float scale, int window);

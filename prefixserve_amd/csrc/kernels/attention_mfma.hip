@@ -29,6 +29,9 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
+// A 16-byte piece in registers. A plain vector: HIP's uint4 is a struct, and copies of it in
+// arrays were compiled to copies through scratch memory.
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
 __device__ __forceinline__ bf16x8 ld8(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
 __device__ __forceinline__ bf16x4 ld4(const bf16_t* p) { return *reinterpret_cast<const bf16x4*>(p); }
@@ -86,8 +89,12 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
   __shared__ float sm_m[4][32], sm_l[4][32];
   __shared__ float sm_o[3 * DTC * 16 * 64];
   extern __shared__ int32_t table[];
-  // Late tiles of a prompt see the most keys: start them first.
-  const int tile = gridDim.x - 1 - blockIdx.x, h = blockIdx.y;
+  // Late tiles of a prompt see the most keys: start them first. Workgroups are handed out in
+  // the order x + gridDim.x * y, round robin over the dies: x runs over the kv heads first and
+  // then over the query heads of each, so that with a multiple of 8 kv heads all workgroups of
+  // a kv head run on one die and share its keys and values in that die's L2.
+  const int tile = gridDim.y - 1 - blockIdx.y;
+  const int h = (blockIdx.x % hkv) * (hq / hkv) + blockIdx.x / hkv;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int item = pf_tiles[2 * tile];
   const int q_off = pf_tiles[2 * tile + 1];
@@ -302,14 +309,20 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
 // Up to head size 64 the kernel is held to 128 registers (four waves per SIMD, the second
 // argument of the launch bounds): at 131 only one workgroup of eight waves fitted a compute unit.
 // With two, a prompt of 8,192 tokens, whose 256 tiles are more workgroups than compute units,
-// runs 5% faster (8 layers of the 1B shape: 10.6 -> 10.0 ms); at 2,048 tokens there is one
-// workgroup per compute unit either way.
+// runs 5% faster (8 layers of the 1B shape: 10.6 -> 10.0 ms).
+// The pieces on their way from global memory to LDS are held as plain 4-word vectors: as
+// arrays of HIP's uint4 (a struct) the compiler kept them in scratch memory whenever a thread
+// has two or more pieces (head sizes from 96 on), waiting for each load right after issuing
+// it; without that a 2,048-token prompt at head size 128 went from 75 to 55 us a layer.
+// Measured and not kept: the scores of the next iteration issued before the softmax of the
+// current one (correct, no faster at head size 128, slower at 64 where it costs the second
+// workgroup per compute unit its registers), and the stores to LDS issued behind the barrier.
 template <int NS, int KT, int KP>
 __global__ __launch_bounds__(256 * KP, NS <= 4 ? 4 : 2) void attn_prefill_grouped_kernel(
     const bf16_t* __restrict__ qkv, int q_stride, bf16_t* __restrict__ out, const bf16_t* __restrict__ kv,
     const int32_t* __restrict__ pf_tiles, const int32_t* __restrict__ item_start,
     const int32_t* __restrict__ item_pos0, const int32_t* __restrict__ table_off,
-    const int32_t* __restrict__ block_ids, int n_tiles, int paired, int hq, int hkv, int table_pages, float scale,
+    const int32_t* __restrict__ block_ids, int n_tiles, int hq, int hkv, int table_pages, float scale,
     int window) {
   constexpr int D = 16 * NS;
   constexpr int DT = (D + 31) / 32;
@@ -327,22 +340,19 @@ __global__ __launch_bounds__(256 * KP, NS <= 4 ? 4 : 2) void attn_prefill_groupe
 
   const int group = hq / hkv;
   const int wg_per_kv = (group + 3) >> 2;
-  const int kvh = blockIdx.y / wg_per_kv;
+  // Grid: x = (kv head, block of 4 query heads), y = tile, the late tiles (which see the most
+  // keys) first. Workgroups are handed out in the order x + gridDim.x * y and go round robin over
+  // the dies: the heaviest tiles of every head start first, so no head's long tiles are left
+  // running alone at the end, and with a multiple of 8 workgroups in x a kv head's tiles all run
+  // on one die, whose L2 then holds that head's keys and values for all of them (a 2,048-token
+  // prompt at head size 64 fetched 20 MB from memory with the tile in x and 7 MB this way).
+  const int kvh = blockIdx.x / wg_per_kv;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int part = wave >> 2;                           // which of the iteration's KP runs of keys
-  const int head_in_group = (blockIdx.y - kvh * wg_per_kv) * 4 + (wave & 3);
+  const int head_in_group = (blockIdx.x - kvh * wg_per_kv) * 4 + (wave & 3);
   const bool head_valid = head_in_group < group;       // a spare wave repeats the last head and writes nothing
   const int h = kvh * group + min(head_in_group, group - 1);
-  // With `paired`, a workgroup takes two tiles, one after the other: the b-th from the end and
-  // the b-th from the start. In a causal prompt the first sees the most keys and the second the
-  // fewest, so all workgroups get the same amount of work and none is left running alone at the
-  // end. Without, one tile each, the late ones first.
-  for (int phase = 0; phase < (paired ? 2 : 1); ++phase) {
-  const int tile = phase == 0 ? n_tiles - 1 - static_cast<int>(blockIdx.x) : static_cast<int>(blockIdx.x);
-  if (phase == 1) {
-    if (tile >= n_tiles - 1 - static_cast<int>(blockIdx.x)) break;     // the middle tile is taken once
-    __syncthreads();                                                   // LDS is used again from the start
-  }
+  const int tile = n_tiles - 1 - static_cast<int>(blockIdx.y);
   const int item = pf_tiles[2 * tile];
   const int q_off = pf_tiles[2 * tile + 1];
   const int t0 = item_start[item];
@@ -386,7 +396,7 @@ __global__ __launch_bounds__(256 * KP, NS <= 4 ? 4 : 2) void attn_prefill_groupe
   // Piece p of a tile lies in page p / (2 D) at element 8 * (p % (2 D)) of the head's keys
   // (and likewise of its values): both halves of a page are contiguous per head.
   struct Pieces {
-    uint4 k[CPT], v[CPT];
+    u32x4 k[CPT], v[CPT];
   };
   auto load_global = [&](Pieces& r, int k0) {
 #pragma unroll
@@ -396,8 +406,8 @@ __global__ __launch_bounds__(256 * KP, NS <= 4 ? 4 : 2) void attn_prefill_groupe
         const int page = p / (2 * D), rem = p - page * 2 * D;
         const int64_t base = static_cast<int64_t>(table[min(k0 + 16 * page, last_pos) >> 4]) * page_elems;
         const bf16_t* src = kv + base + 8 * rem;
-        r.k[i] = *reinterpret_cast<const uint4*>(src + khead);
-        r.v[i] = *reinterpret_cast<const uint4*>(src + vhead);
+        r.k[i] = *reinterpret_cast<const u32x4*>(src + khead);
+        r.v[i] = *reinterpret_cast<const u32x4*>(src + vhead);
       }
     }
   };
@@ -410,20 +420,18 @@ __global__ __launch_bounds__(256 * KP, NS <= 4 ? 4 : 2) void attn_prefill_groupe
       const int p = threadIdx.x + THREADS * i;
       if (CHUNKS % THREADS == 0 || p < CHUNKS) {
         const int key = p / (D / 8), part = p - key * (D / 8);
-        *reinterpret_cast<uint4*>(kd + key * KS + 8 * part) = r.k[i];
+        *reinterpret_cast<u32x4*>(kd + key * KS + 8 * part) = r.k[i];
         const int row = p >> 1, half = p & 1;                     // row = page * D + d
-        uint4 v = r.v[i];
+        u32x4 v = r.v[i];
         if (edge) {
           const int key0 = k0 + 16 * (row / D) + 8 * half;        // the piece holds the values of keys key0 .. key0 + 7
-          uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
           for (int e = 0; e < 8; ++e)
-            if (key0 + e > max_key || key0 + e < k_begin_vis) w[e >> 1] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
-          v = uint4{w[0], w[1], w[2], w[3]};
+            if (key0 + e > max_key || key0 + e < k_begin_vis) v[e >> 1] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
         }
         uint2* dst = reinterpret_cast<uint2*>(vd + row * VS + 8 * half);
-        dst[0] = uint2{v.x, v.y};
-        dst[1] = uint2{v.z, v.w};
+        dst[0] = uint2{v[0], v[1]};
+        dst[1] = uint2{v[2], v[3]};
       }
     }
   };
@@ -562,7 +570,7 @@ __global__ __launch_bounds__(256 * KP, NS <= 4 ? 4 : 2) void attn_prefill_groupe
     }
     }
   }
-  if (part != 0 || !head_valid || !q_valid) continue;
+  if (part != 0 || !head_valid || !q_valid) return;
   const float inv = 1.f / l;
   bf16_t* op = out + static_cast<int64_t>(t0 + qi) * (static_cast<int64_t>(hq) * D) + h * D;
 #pragma unroll
@@ -579,7 +587,6 @@ __global__ __launch_bounds__(256 * KP, NS <= 4 ? 4 : 2) void attn_prefill_groupe
         *reinterpret_cast<ushort4*>(op + d) = pk;
       }
     }
-  }
 }
 
 // ------------------------------------------------------------------ decode (split keys)
@@ -811,46 +818,46 @@ static bool lds_allowed(Kernel kernel, size_t bytes) {
 }
 
 // Which kernel a step's portions go to, when three or more query heads share a kv head
-// (measured at head sizes 64 and 128 on 256 compute units; us per layer, per-head / grouped
-// with one tile per workgroup / grouped with paired tiles):
-//   128 new tokens on 1,920 cached   16 / 30 / 56      512 on 1,536     29 / 31 / 52
-//   512 from position 0              12 / 12 / 16      1,024 from 0     31 / 19 / 24
-//   2,048 from position 0            87 / 62 / 39      4,096 from 0    255 / 162 / 128
-//  * few tiles: the per-head kernel, whose grid is four times as large, fills the chip best;
-//  * in between: the grouped kernel, one tile per workgroup;
-//  * two workgroups per compute unit or more AND little cached in front of the portions:
-//    paired tiles. Pairing evens out a causal triangle; on top of a long prefix every tile
-//    has much the same work and pairing only halves the number of workgroups.
-enum class PrefillForm { kPerHead, kGrouped, kGroupedPaired };
+// (measured on 256 compute units with 32 query heads on 8 kv heads; us per layer, per-head /
+// grouped, at head size 64 and at head size 128):
+//   256 on 1,792 cached     18 / 30      31 / 43       384 on 3,712 cached     48 / 53      94 / 78
+//   512 from position 0     11 / 12      21 / 18       512 on 7,680 cached     91 / 101    180 / 148
+//   768 on 2,304 cached     50 / 42     104 / 63       1,024 on 3,072 cached   84 / 56     176 / 88
+//   2,048 from position 0   57 / 36     142 / 58       8,192 from 0             - / 355      - / 655
+// The per-head kernel, whose grid is four times as large, fills the chip better while the grouped
+// one has few workgroups: up to 128 of them at head sizes up to 64, up to 80 above (the grouped
+// kernel's advantage, every key and value read once for four heads, grows with the head size).
+// Two tiles per workgroup (the b-th from the end and the b-th from the start of a causal prompt,
+// to even out the triangle) were measured against the order of workgroups described in the kernel
+// and dropped: within 3% at best, 12% slower at 3,072 tokens, up to 15% slower on top of a cached
+// prefix.
+enum class PrefillForm { kPerHead, kGrouped };
 
-static PrefillForm prefill_form(int n_tiles, int64_t prefix_tokens, int hq, int hkv) {
+static PrefillForm prefill_form(int n_tiles, int hq, int hkv, int head_dim) {
   const int group = hq / hkv;
   if (group < 3) return PrefillForm::kPerHead;
   const int64_t workgroups = static_cast<int64_t>(n_tiles) * hkv * ((group + 3) / 4);
-  if (workgroups < 128) return PrefillForm::kPerHead;
-  if (workgroups >= 512 && 4 * prefix_tokens <= 32LL * n_tiles) return PrefillForm::kGroupedPaired;
-  return PrefillForm::kGrouped;
+  return workgroups <= (head_dim <= 64 ? 128 : 80) ? PrefillForm::kPerHead : PrefillForm::kGrouped;
 }
 
 template <int NS>
 static int launch_prefill(hipStream_t s, const void* qkv, int q_stride, void* out, const void* kv,
-                          const int32_t* pf_tiles, int n_tiles, int64_t prefix_tokens, int table_pages,
+                          const int32_t* pf_tiles, int n_tiles, int table_pages,
                           const int32_t* item_start, const int32_t* item_pos0,
                           const int32_t* table_off, const int32_t* block_ids, int hq, int hkv, float scale, int window) {
   const int group = hq / hkv;
-  const PrefillForm form = prefill_form(n_tiles, prefix_tokens, hq, hkv);
+  const PrefillForm form = prefill_form(n_tiles, hq, hkv, 16 * NS);
   // The heads of a kv head share its keys and values through LDS, two waves per head (each its
   // own run of keys) if the stages fit, else one.
   if (form != PrefillForm::kPerHead) {
-    const int paired = form == PrefillForm::kGroupedPaired ? 1 : 0;
-    const dim3 grid(paired ? (n_tiles + 1) / 2 : n_tiles, hkv * ((group + 3) / 4));
+    const dim3 grid(hkv * ((group + 3) / 4), n_tiles);
 #define PSAMD_GROUPED(KP_)                                                                                         \
   {                                                                                                               \
     const size_t smem = grouped_smem(16 * NS, 1, KP_, table_pages);                                               \
     if (lds_allowed(attn_prefill_grouped_kernel<NS, 1, KP_>, smem)) {                                             \
       attn_prefill_grouped_kernel<NS, 1, KP_><<<grid, dim3(256 * KP_), smem, s>>>(                                \
           static_cast<const bf16_t*>(qkv), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(kv),   \
-          pf_tiles, item_start, item_pos0, table_off, block_ids, n_tiles, paired, hq, hkv, table_pages, scale, window); \
+          pf_tiles, item_start, item_pos0, table_off, block_ids, n_tiles, hq, hkv, table_pages, scale, window); \
       return check_launch("psamd_attention_prefill");                                                             \
     }                                                                                                             \
   }
@@ -858,7 +865,7 @@ static int launch_prefill(hipStream_t s, const void* qkv, int q_stride, void* ou
     PSAMD_GROUPED(1)
 #undef PSAMD_GROUPED
   }
-  attn_prefill_mfma_kernel<NS><<<dim3(n_tiles, hq), dim3(256), sizeof(int32_t) * static_cast<size_t>(table_pages), s>>>(
+  attn_prefill_mfma_kernel<NS><<<dim3(hq, n_tiles), dim3(256), sizeof(int32_t) * static_cast<size_t>(table_pages), s>>>(
       static_cast<const bf16_t*>(qkv), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(kv), pf_tiles,
       item_start, item_pos0, table_off, block_ids, hq, hkv, scale, window);
   return check_launch("psamd_attention_prefill");
@@ -910,10 +917,8 @@ int psamd_attention_mfma_supports(int hq, int hkv, int head_dim) {
 }
 
 // max_kv_len: the longest request of the step after it (sizes the block table staged in LDS).
-// prefix_tokens: tokens already cached in front of the portions, summed over them (with the
-// number of tiles it decides which form of the kernel runs).
 int psamd_attention_prefill(void* stream, const void* qkv, int q_stride, void* out, const void* kv,
-                            const int32_t* pf_tiles, int n_tiles, int max_kv_len, int64_t prefix_tokens,
+                            const int32_t* pf_tiles, int n_tiles, int max_kv_len,
                             const int32_t* item_start,
                             const int32_t* item_pos0, const int32_t* table_off, const int32_t* block_ids, int hq,
                             int hkv, int head_dim, float scale, int window) {
@@ -921,10 +926,11 @@ int psamd_attention_prefill(void* stream, const void* qkv, int q_stride, void* o
   PSAMD_REQUIRE(q_stride % 8 == 0, "query row stride must be a multiple of 8 elements");
   PSAMD_REQUIRE(max_kv_len >= 1 && max_kv_len <= 8192 * kPage, "context too long for the block table staged in LDS");
   if (n_tiles == 0) return 0;
+  PSAMD_REQUIRE(n_tiles <= 65535, "too many query tiles for one launch");
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int table_pages = static_cast<int>(ceil_div(max_kv_len, kPage));
 #define PSAMD_PF(NS_)                                                                                           \
-  return launch_prefill<NS_>(s, qkv, q_stride, out, kv, pf_tiles, n_tiles, prefix_tokens, table_pages, item_start, \
+  return launch_prefill<NS_>(s, qkv, q_stride, out, kv, pf_tiles, n_tiles, table_pages, item_start, \
                              item_pos0, table_off, block_ids, hq, hkv, scale, window)
   switch (head_dim / 16) {
     case 1: PSAMD_PF(1);

@@ -63,7 +63,6 @@ class StepContext:
     num_decode: int            # items with exactly one token (served by the decode kernel)
     num_prefill_tiles: int
     max_kv_len: int
-    prefill_prefix_tokens: int  # tokens already cached in front of the step's portions, summed
     token_ids: torch.Tensor    # [T]
     positions: torch.Tensor    # [T] absolute
     tok_item: torch.Tensor     # [T] item of each token
@@ -121,7 +120,7 @@ class StepPacker:
                                       self.num_slots, self.prefill_tile, static_pages)
         except ValueError as e:
             raise EngineError(str(e)) from None
-        _, total, t_n, b, s_n, n_dec, n_tiles, p_total, max_kv_len, prefix, offs, group_offs = res
+        _, total, t_n, b, s_n, n_dec, n_tiles, p_total, max_kv_len, offs, group_offs = res
         o_ids, o_pos, o_item, o_start, o_pos0, o_end, o_slots, o_rows, o_dec, o_tiles = offs
 
         if self.on_gpu:
@@ -145,6 +144,6 @@ class StepPacker:
         _, on_dev, host, groups = self._views
         return StepContext(
             num_tokens=t_n, num_items=b, num_logit_rows=s_n, num_decode=n_dec, num_prefill_tiles=n_tiles,
-            max_kv_len=max_kv_len, prefill_prefix_tokens=prefix, groups=groups, keys=[it.key for it in items],
+            max_kv_len=max_kv_len, groups=groups, keys=[it.key for it in items],
             want_counts=[len(it.want) for it in items], host=host, **on_dev,
         )

@@ -50,7 +50,7 @@ _SIGNATURES = {
     "psamd_qkv_rope_append": [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp],
     "psamd_attention_generic": [_vp, _vp, _i32, _vp, _vp, _i32, _i64, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _f32, _i32],
     "psamd_attention_mfma_supports": [_i32, _i32, _i32],
-    "psamd_attention_prefill": [_vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _i64, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _f32,
+    "psamd_attention_prefill": [_vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _f32,
                                 _i32],
     "psamd_attention_decode": [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32,
                                _i32, _f32, _i32],
@@ -293,7 +293,7 @@ class HipOps:
             if ctx.num_prefill_tiles:
                 self._ok(self.lib.psamd_attention_prefill(
                     s, qkv.data_ptr(), stride, out.data_ptr(), kv.data_ptr(), ctx.pf_tiles.data_ptr(),
-                    ctx.num_prefill_tiles, self.fixed_kv_len or ctx.max_kv_len, ctx.prefill_prefix_tokens,
+                    ctx.num_prefill_tiles, self.fixed_kv_len or ctx.max_kv_len,
                     ctx.item_start.data_ptr(), ctx.item_pos0.data_ptr(),
                     g.table_off.data_ptr(), g.block_ids.data_ptr(), hq, hkv, d, scale, win))
             if ctx.num_decode:
