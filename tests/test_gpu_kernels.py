@@ -385,20 +385,23 @@ def test_paged_attention_mixed_batch(ops, act, hq, hkv, d):
 
 
 @pytest.mark.parametrize("hq,hkv,d,new,old,window", [
-    (32, 8, 64, [2048], [0], None),              # 512 workgroups, nothing cached: grouped, paired tiles
+    (32, 8, 64, [2048], [0], None),              # 512 workgroups, nothing cached: grouped, a kv head's tiles on one die
     (24, 8, 128, [2100], [0], None),             # three heads per kv head, an odd number of tiles, a last tile of 20
-    (16, 4, 64, [2048, 2100], [0, 0], None),     # two prompts from position 0 in one step, paired
-    (32, 8, 64, [512], [1536], None),            # 128 workgroups on a long prefix: grouped, one tile each
-    (32, 8, 64, [2048, 3], [2048, 7], None),     # 512 workgroups but much cached: one tile each
+    (16, 4, 64, [2048, 2100], [0, 0], None),     # two prompts from position 0 in one step, 4 workgroups per tile
+    (32, 8, 64, [512], [1536], None),            # 128 workgroups on a long prefix: the per-head kernel at this head size
+    (32, 8, 64, [768], [1536], None),            # 192 workgroups on a long prefix: grouped
+    (32, 8, 128, [512], [1536], None),           # 128 workgroups at head size 128: grouped
+    (32, 8, 64, [2048, 3], [2048, 7], None),     # 512 workgroups, much cached, beside a short portion
     (40, 2, 64, [500, 77], [100, 0], None),      # twenty heads per kv head: five workgroups per kv head
     (6, 2, 256, [1500, 1000], [0, 200], None),   # head size 256
-    (16, 4, 64, [700, 300], [50, 0], 100),       # one tile each, with a window
-    (32, 8, 64, [2048], [0], 300),               # paired tiles, with a window
+    (16, 4, 64, [700, 300], [50, 0], 100),       # grouped, with a window
+    (32, 8, 64, [2048], [0], 300),               # a long prompt with a window
     (32, 8, 64, [100], [1948], None),            # few tiles: the per-head kernel
 ])
 def test_prefill_attention_in_each_form(ops, hq, hkv, d, new, old, window):
-    """The portions of a step go to one of three forms of the kernel by their number of tiles and
-    by how much is cached in front of them; each form at sizes that select it."""
+    """The portions of a step go to the per-head or to the grouped kernel by their number of tiles
+    and the head size; each at sizes that select it, with grids that are and are not multiples of
+    the eight dies in their fast index."""
     pages = sum(-(-(n + o) // 16) for n, o in zip(new, old)) + 8
     got, want = paged_case(ops, torch.bfloat16, hq, hkv, d, new, old, window=window, seed=len(new) + d, num_blocks=pages)
     assert rel(got, want) < 2e-2
@@ -406,8 +409,9 @@ def test_prefill_attention_in_each_form(ops, hq, hkv, d, new, old, window):
 
 @pytest.mark.parametrize("hq,hkv,d,new,old,window", [
     (8, 2, 64, [37, 1, 130, 1, 2, 16, 1, 1], [0, 15, 50, 31, 94, 16, 0, 200], None),   # decode and the per-head prefill kernel
-    (32, 8, 64, [2040], [0], None),                 # grouped, paired tiles; the last page has 8 slots nobody wrote
-    (32, 8, 64, [500], [1530], None),               # grouped, one tile each
+    (32, 8, 64, [2040], [0], None),                 # grouped; the last page has 8 slots nobody wrote
+    (32, 8, 64, [500], [1530], None),               # the per-head kernel on a cached prefix
+    (32, 8, 64, [700], [1330], None),               # grouped on a cached prefix
     (24, 8, 128, [2100, 1], [0, 77], None),
     (8, 2, 64, [70, 1, 1, 9], [0, 40, 130, 64], 33),        # windows whose first pages were given back
     (16, 4, 64, [700, 300, 1], [150, 0, 900], 100),
@@ -479,11 +483,12 @@ def test_attention_finds_one_far_key_among_hundreds(ops, act):
 
 @pytest.mark.parametrize("hq,hkv,d,new,old,window", [
     (32, 8, 64, 100, 1948, None),       # few tiles: the per-head kernel, keys split over its four waves
-    (32, 8, 64, 512, 1536, None),       # grouped, one tile per workgroup, on a cached prefix
-    (32, 8, 64, 2048, 0, None),         # grouped, paired tiles
+    (32, 8, 64, 512, 1536, None),       # the per-head kernel on a cached prefix, 128 workgroups' worth
+    (32, 8, 64, 800, 1248, None),       # grouped, on a cached prefix
+    (32, 8, 64, 2048, 0, None),         # grouped, a whole prompt
     (24, 8, 128, 700, 500, None),       # head size 128, three heads per kv head
-    (32, 8, 64, 2048, 0, 300),          # paired tiles with a window
-    (16, 4, 64, 600, 200, 100),         # one tile each with a window
+    (32, 8, 64, 2048, 0, 300),          # a whole prompt with a window
+    (16, 4, 64, 600, 200, 100),         # grouped with a window
 ])
 def test_prefill_attention_finds_one_planted_key(ops, hq, hkv, d, new, old, window):
     """With random keys a 32-key tile that is dropped or read twice far from the diagonal moves
