@@ -391,6 +391,7 @@ def test_paged_attention_mixed_batch(ops, act, hq, hkv, d):
     (32, 8, 64, [512], [1536], None),            # 128 workgroups on a long prefix: the per-head kernel at this head size
     (32, 8, 64, [768], [1536], None),            # 192 workgroups on a long prefix: grouped
     (32, 8, 128, [512], [1536], None),           # 128 workgroups at head size 128: grouped
+    (32, 8, 128, [4100], [0], None),             # 1,032 workgroups at head size 128: grouped, one wave per head
     (32, 8, 64, [2048, 3], [2048, 7], None),     # 512 workgroups, much cached, beside a short portion
     (40, 2, 64, [500, 77], [100, 0], None),      # twenty heads per kv head: five workgroups per kv head
     (6, 2, 256, [1500, 1000], [0, 200], None),   # head size 256
@@ -487,6 +488,7 @@ def test_attention_finds_one_far_key_among_hundreds(ops, act):
     (32, 8, 64, 800, 1248, None),       # grouped, on a cached prefix
     (32, 8, 64, 2048, 0, None),         # grouped, a whole prompt
     (24, 8, 128, 700, 500, None),       # head size 128, three heads per kv head
+    (32, 8, 128, 4100, 0, None),        # head size 128, a long prompt: one wave per head
     (32, 8, 64, 2048, 0, 300),          # a whole prompt with a window
     (16, 4, 64, 600, 200, 100),         # grouped with a window
 ])
