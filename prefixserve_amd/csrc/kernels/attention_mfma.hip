@@ -510,24 +510,25 @@ __global__ __launch_bounds__(256 * KP, NS <= 4 ? 4 : 2) void attn_prefill_groupe
     int k0 = k_begin, stage = 0;
     load_global(ra, k0);
     load_global(rb, k0 + KEYS);
-    while (true) {
-      store_lds(ra, stage, k0);
-      load_global(ra, k0 + 2 * KEYS);
+    auto iteration = [&](Pieces& r) {
+      store_lds(r, stage, k0);
+      load_global(r, k0 + 2 * KEYS);
       // Every wave is past the iteration that last used this stage: it had to finish it to
       // reach the previous barrier.
       __syncthreads();
       compute(stage, k0);
       stage ^= 1;
       k0 += KEYS;
-      if (k0 > last_pos) break;
-      store_lds(rb, stage, k0);
-      load_global(rb, k0 + 2 * KEYS);
-      __syncthreads();
-      compute(stage, k0);
-      stage ^= 1;
-      k0 += KEYS;
-      if (k0 > last_pos) break;
-    }
+    };
+    // Always two iterations per turn, the second perhaps on keys past the last query (its
+    // loads are clamped, its stores go to a free stage and compute() skips it): a way out of
+    // the loop between the two would, as the compiler lays the loop out, also be a way back to
+    // its head, and the wait in front of the first store would then be for all loads but one
+    // instead of all but three, which waits for the set that has just been asked for.
+    do {
+      iteration(ra);
+      iteration(rb);
+    } while (k0 <= last_pos);
   }
 
   if (KP > 1) {
