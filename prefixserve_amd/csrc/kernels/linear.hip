@@ -333,6 +333,28 @@ constexpr int wide_depth(int mt) { return mt <= 2 ? 2 : 1; }
 template <int MT, bool SWIGLU>
 static int launch_skinny1(hipStream_t s, const void* x, const void* w, void* out, int out_dtype, int M, int n_out,
                           int K, int ksplit) {
+  if constexpr (!SWIGLU && MT == 1) {
+    // Up to 8 tokens and row groups to spare (the output matrix): one row tile (two from 5 tokens
+    // on) per workgroup of eight waves that split K, every wave's eight k-steps in flight at once.
+    // Against four waves with a row tile each over all of K, at 128,256 columns and K = 2,048:
+    // 93 -> 84 us at 1 token, 95 -> 87 at 2, 101 -> 96 at 4, 113 -> 111 at 8; the same order at
+    // K = 4,096 (193 -> 172 us at 1 token).
+    if (M <= 8 && ksplit == 1 && ceil_div(n_out, 16) >= 2048) {
+      const bf16_t* xp = static_cast<const bf16_t*>(x);
+      const bf16_t* wp = static_cast<const bf16_t*>(w);
+      const dim3 block(64 * 8);
+      if (M <= 4) {
+        const dim3 grid(static_cast<unsigned>(ceil_div(n_out, 16)), 1u);
+        if (out_dtype == kBF16) skinny_mfma_kernel<1, 1, 8, false, true, bf16_t, 8><<<grid, block, 0, s>>>(xp, wp, static_cast<bf16_t*>(out), M, n_out, K);
+        else skinny_mfma_kernel<1, 1, 8, false, true, float, 8><<<grid, block, 0, s>>>(xp, wp, static_cast<float*>(out), M, n_out, K);
+      } else {
+        const dim3 grid(static_cast<unsigned>(ceil_div(ceil_div(n_out, 16), 2)), 1u);
+        if (out_dtype == kBF16) skinny_mfma_kernel<1, 2, 8, false, true, bf16_t, 8><<<grid, block, 0, s>>>(xp, wp, static_cast<bf16_t*>(out), M, n_out, K);
+        else skinny_mfma_kernel<1, 2, 8, false, true, float, 8><<<grid, block, 0, s>>>(xp, wp, static_cast<float*>(out), M, n_out, K);
+      }
+      return check_launch("psamd_linear_skinny");
+    }
+  }
   if constexpr (!SWIGLU) {
     if (M > 8 && ksplit == 1 && ceil_div(n_out, 16) >= kManyRowTiles) {
       constexpr int RT = wide_rt(MT), WV = wide_wv(MT), U = wide_depth(MT);
