@@ -142,10 +142,23 @@ __global__ __launch_bounds__(kThreads) void add_rmsnorm_vec8_kernel(
           v[j][2 * i + 1] += __uint_as_float(w4[i] & 0xffff0000u);
         }
       } else {
-        const float4 x0 = *reinterpret_cast<const float4*>(dp);
-        const float4 x1 = *reinterpret_cast<const float4*>(dp + 4);
-        v[j][0] += x0.x; v[j][1] += x0.y; v[j][2] += x0.z; v[j][3] += x0.w;
-        v[j][4] += x1.x; v[j][5] += x1.y; v[j][6] += x1.z; v[j][7] += x1.w;
+        // Up to eight slices are asked for together (one trip to memory, not one per slice) and
+        // added in ascending order; slots past the last slice repeat it and are not added.
+        float4 x0[8], x1[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const DT* du = d0 + min(p + u, np - 1) * partial_stride + e;
+          x0[u] = *reinterpret_cast<const float4*>(du);
+          x1[u] = *reinterpret_cast<const float4*>(du + 4);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          if (p + u < np) {
+            v[j][0] += x0[u].x; v[j][1] += x0[u].y; v[j][2] += x0[u].z; v[j][3] += x0[u].w;
+            v[j][4] += x1[u].x; v[j][5] += x1[u].y; v[j][6] += x1[u].z; v[j][7] += x1[u].w;
+          }
+        }
+        p += 7;
       }
     }
     if (cidx < chunks) {

@@ -601,6 +601,15 @@ int psamd_linear_skinny_ksplit(int M, int n_out, int K) {
   // Up to 32 tokens a wave keeps at least two k-steps; above, one is enough (measured).
   // Workgroups of 4 waves: two per compute unit; of 8 waves: one (4,096 x 4,096 at 64 tokens:
   // 16.2 us with 8 slices, 14.3 with 4).
+  if (mt == 1) {
+    // Up to 16 tokens: as many slices as give a wave about eight k-steps, all of which it has
+    // in flight at once, whatever the number of workgroups up to 2,048 (measured at 1 and 8
+    // tokens: 2,048 x 8,192 10.0 -> 8.6 us with 8 slices instead of 4, 3,072 x 8,192 15.3 -> 12.0,
+    // 4,096 x 14,336 27.9 -> 24 us; 2,048 x 2,048 4.0 -> 3.8 us with 2 instead of 4).
+    const int64_t per_slice = 8 * skinny_wv(mt);
+    const int64_t split = std::min<int64_t>({8, std::max<int64_t>(2048 / std::max<int64_t>(groups, 1), 1), (steps + per_slice / 2) / per_slice});
+    return static_cast<int>(std::max<int64_t>(split, 1));
+  }
   const int64_t wanted = skinny_wv(mt) == 8 ? 256 : 512;
   const int64_t split = std::min<int64_t>({8, wanted / std::max<int64_t>(groups, 1), steps / ((mt <= 2 ? 2 : 1) * skinny_wv(mt))});
   return static_cast<int>(std::max<int64_t>(split, 1));

@@ -237,12 +237,12 @@ def test_linear_bf16_very_many_columns(ops, m, n, k, out_dtype):
 
 
 @pytest.mark.parametrize("m", [1, 8, 33, 64])
-@pytest.mark.parametrize("n,k", [(2048, 2048), (200, 8192), (72, 520), (256, 688)])
+@pytest.mark.parametrize("n,k", [(2048, 2048), (200, 8192), (72, 2056), (256, 2744), (72, 520), (256, 688)])
 def test_linear_to_residual_splits_k(ops, m, n, k):
     x, w = rnd(m, k, dtype=torch.bfloat16, seed=1), rnd(n, k, dtype=torch.bfloat16, seed=2, scale=0.05)
     out = ops.linear_to_residual(x, w, "test.delta")
     split = ops.lib.psamd_linear_skinny_ksplit(m, n, k)
-    assert split > 1 or (m > 32 and k < 1024)         # these shapes do split, but for many tokens and a short K
+    assert split > 1 or k < 1024                      # these shapes do split, but for a short K (a wave wants about eight k-steps)
     if split > 1:
         assert out.dim() == 3 and out.dtype == torch.float32 and out.shape[0] == split
         assert rel(out.sum(0), x.double() @ w.double().T) < 1e-5
