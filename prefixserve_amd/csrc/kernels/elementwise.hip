@@ -310,6 +310,16 @@ __global__ __launch_bounds__(256) void rope_kv_append_vec_kernel(bf16_t* __restr
   const int64_t page_elems = 2LL * hkv * kPage * d;
   const int chunks_per_head = half >> 3;                 // groups of 8 pairs
   const int chunks_per_token = (hq + hkv) * chunks_per_head;
+  const int vw = hkv * d;
+  const int c_lo = static_cast<int>(static_cast<int64_t>(vw >> 3) * blockIdx.y / gridDim.y);      // 8-element columns
+  const int c_hi = static_cast<int>(static_cast<int64_t>(vw >> 3) * (blockIdx.y + 1) / gridDim.y);
+  const int nc = c_hi - c_lo, vs = 8 * nc + 8;
+  // The values are asked for first: they are on their way into LDS while q and k are rotated.
+  for (int idx = threadIdx.x; kv != nullptr && idx < nt * nc; idx += blockDim.x) {
+    const int j = idx / nc, c = idx - j * nc;
+    *reinterpret_cast<uint4*>(v_lds + j * vs + 8 * c) =
+        *reinterpret_cast<const uint4*>(qkv + static_cast<int64_t>(t0 + j) * width + (hq + hkv) * d + 8 * (c_lo + c));
+  }
   // blockIdx.y takes its share of the rotation work and of the value columns.
   const int rot_total = nt * chunks_per_token;
   const int rot_lo = static_cast<int>(static_cast<int64_t>(rot_total) * blockIdx.y / gridDim.y);
@@ -349,15 +359,6 @@ __global__ __launch_bounds__(256) void rope_kv_append_vec_kernel(bf16_t* __restr
     }
   }
   if (kv == nullptr) return;
-  const int vw = hkv * d;
-  const int c_lo = static_cast<int>(static_cast<int64_t>(vw >> 3) * blockIdx.y / gridDim.y);      // 8-element columns
-  const int c_hi = static_cast<int>(static_cast<int64_t>(vw >> 3) * (blockIdx.y + 1) / gridDim.y);
-  const int nc = c_hi - c_lo, vs = 8 * nc + 8;
-  for (int idx = threadIdx.x; idx < nt * nc; idx += blockDim.x) {
-    const int j = idx / nc, c = idx - j * nc;
-    *reinterpret_cast<uint4*>(v_lds + j * vs + 8 * c) =
-        *reinterpret_cast<const uint4*>(qkv + static_cast<int64_t>(t0 + j) * width + (hq + hkv) * d + 8 * (c_lo + c));
-  }
   __syncthreads();
   const int j = threadIdx.x & 15;
   if (j < nt) {
