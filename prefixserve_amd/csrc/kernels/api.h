@@ -45,6 +45,15 @@ int psamd_linear(void* stream, const void* x, int x_dtype, const void* w, int w_
 int psamd_gemm_lt_available();
 int psamd_gemm_lt(void* stream, const void* x, const void* w, void* out, int out_dtype, int64_t M, int N, int K,
                   int use_workspace);
+// Times every algorithm the library has for the shape on the given buffers (the n_ws matrices of
+// that shape in turn, so that each call reads its matrix from memory) and keeps the fastest
+// for it (and for row counts within a quarter of it) if it beats the heuristic's choice by 3%;
+// out and ref_out receive the product by the kept and by the heuristic's algorithm. For warm-up:
+// takes a second or two and waits for the stream. 2: library or its extension interface missing.
+int psamd_gemm_lt_tune(void* stream, const void* x, const void* const* ws, int n_ws, void* out, void* ref_out, int out_dtype,
+                       int64_t M, int N, int K, float* us_before, float* us_after);
+int psamd_gemm_lt_untune(int out_dtype, int64_t M, int N, int K);
+
 
 // bfloat16 product for M <= 64 on the matrix cores. epilogue 1: w = [gate; up], out = silu(gate) * up.
 // ksplit > 1: out receives ksplit float32 partial sums [ksplit][M, n_out] (plain epilogue only).

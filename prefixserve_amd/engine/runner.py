@@ -165,3 +165,27 @@ class ModelRunner:
 
     def pack(self, items: Sequence[StepItem]) -> StepContext:
         return self.packer.pack(items)
+
+    def tune_products(self, token_counts: Sequence[int]) -> list[tuple[int, tuple[int, int], float, float]]:
+        """Lets the product library time its algorithms for steps of the given token counts,
+        once per distinct matrix shape of the model's parts, and keep the fastest: the library's
+        own choice is made without running anything. The same product of every layer shares a
+        shape; its matrices are timed in turn, so that each call reads its matrix from memory as
+        a step does. Returns (tokens, (out, in), microseconds before, after) per tuned product.
+        For warm-up: a second or so per shape."""
+        tune = getattr(self.ops, "tune_linear", None)
+        done: list[tuple[int, tuple[int, int], float, float]] = []
+        if tune is None or self.dtype != torch.bfloat16:
+            return done
+        by_shape: dict[tuple[int, int], list[torch.Tensor]] = {}
+        for blk in self.model.blocks:
+            for part in blk.parts():
+                for w in part.product_weights():
+                    by_shape.setdefault((int(w.shape[0]), int(w.shape[1])), []).append(w)
+        for shape, weights in by_shape.items():
+            for t in dict.fromkeys(int(t) for t in token_counts):
+                res = tune(t, weights)
+                if res is not None:
+                    done.append((t, shape, res[0], res[1]))
+                    logger.info("product of %d tokens by [%d, %d]: %.1f -> %.1f us", t, shape[0], shape[1], *res)
+        return done

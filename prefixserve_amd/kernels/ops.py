@@ -12,7 +12,8 @@ from __future__ import annotations
 
 import contextlib
 import ctypes
-from typing import Any
+import logging
+from typing import Any, Sequence
 
 import torch
 
@@ -38,6 +39,8 @@ def _ptr(t: torch.Tensor | None) -> int | None:
     return None if t is None else t.data_ptr()
 
 
+logger = logging.getLogger(__name__)
+
 _SIGNATURES = {
     "psamd_embed": [_vp, _vp, _vp, _i32, _vp, _i64, _i32, _i32],
     "psamd_add_rmsnorm": [_vp, _vp, _vp, _i32, _i32, _i64, _vp, _vp, _i32, _f32, _vp, _i32, _i64, _i32],
@@ -45,6 +48,8 @@ _SIGNATURES = {
     "psamd_rope_kv_append": [_vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp, _vp, _vp, _vp],
     "psamd_linear": [_vp, _vp, _i32, _vp, _i32, _vp, _i32, _i64, _i32, _i32],
     "psamd_gemm_lt": [_vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32],
+    "psamd_gemm_lt_tune": [_vp, _vp, _vp, _i32, _vp, _vp, _i32, _i64, _i32, _i32, _vp, _vp],
+    "psamd_gemm_lt_untune": [_i32, _i64, _i32, _i32],
     "psamd_linear_skinny": [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32],
     "psamd_linear_skinny_ksplit": [_i32, _i32, _i32],
     "psamd_qkv_rope_append": [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp],
@@ -233,6 +238,44 @@ class HipOps:
                 return
         self._ok(self.lib.psamd_linear(self._stream(), x.data_ptr(), _code(x.dtype), w.data_ptr(), _code(w.dtype),
                                        out.data_ptr(), _code(out.dtype), m, n, k))
+
+    def tune_linear(self, rows: int, weights: Sequence[torch.Tensor],
+                    out_dtype: torch.dtype | None = None) -> tuple[float, float] | None:
+        """Lets the library time its algorithms for ``rows`` tokens times each of ``weights`` in turn
+        (matrices of one shape [N, K], bfloat16: the layers of a model, so that a call reads its
+        matrix from memory as a step does) and keep the fastest for that shape and for row
+        counts within a quarter of it. Returns
+        (microseconds with the heuristic's choice, microseconds with what is kept now), or None
+        where the library product does not apply. The kept algorithm's product is compared with
+        the heuristic's here, and dropped again if they differ by more than rounding. Takes a
+        second or two and waits for the device: for warm-up, outside any capture."""
+        w = weights[0]
+        if not (self._direct_library and rows > self.SKINNY_MAX_ROWS and all(
+                v.dtype == torch.bfloat16 and v.shape == w.shape and v.dim() == 2 and v.is_contiguous() for v in weights)):
+            return None
+        n, k = w.shape
+        pointers = (ctypes.c_void_p * len(weights))(*[v.data_ptr() for v in weights])
+        out_dtype = out_dtype or torch.bfloat16
+        gen = torch.Generator(device=self.device).manual_seed(rows + n)
+        x = torch.randn(rows, k, device=self.device, generator=gen).to(torch.bfloat16)
+        got = torch.empty(rows, n, dtype=out_dtype, device=self.device)
+        ref = torch.empty_like(got)
+        before, after = ctypes.c_float(0.0), ctypes.c_float(0.0)
+        rc = self.lib.psamd_gemm_lt_tune(self._stream(), x.data_ptr(), pointers, len(weights), got.data_ptr(), ref.data_ptr(),
+                                         _code(out_dtype), rows, n, k, ctypes.byref(before), ctypes.byref(after))
+        if rc == 2:
+            return None
+        self._ok(rc)
+        torch.cuda.synchronize(self.device)
+        # Two correct algorithms differ by the order of their sums: a few units of bfloat16's last place.
+        scale = float(ref.float().abs().max())
+        apart = float((got.float() - ref.float()).abs().max())
+        if not apart <= 2.0 ** -6 * max(scale, 1e-30):
+            self.lib.psamd_gemm_lt_untune(_code(out_dtype), rows, n, k)
+            logger.warning("tuned product for %d x [%d, %d] differs from the heuristic's by %.3g of %.3g: not kept",
+                           rows, n, k, apart, scale)
+            return before.value, before.value
+        return before.value, after.value
 
     def linear_to_residual(self, x, w, name: str) -> torch.Tensor:
         """x @ w^T for a consumer that adds it to the residual stream (the fused add+norm).

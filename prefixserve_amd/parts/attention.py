@@ -79,6 +79,9 @@ class PagedAttention(Mixer):
     def weight_bytes(self) -> int:
         return sum(w.numel() * w.element_size() for w in (self.w_qkv, self.w_o))
 
+    def product_weights(self) -> list[torch.Tensor]:
+        return [self.w_qkv, self.w_o]
+
     def activation_bytes(self, tokens: int, itemsize: int) -> int:
         # q/k/v, the attention output, the projected output (or its float32 partial sums).
         return tokens * ((self.q_size + 2 * self.kv_size) + self.q_size) * itemsize + 8 * 64 * self.hidden_size * 4 \

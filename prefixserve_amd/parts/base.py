@@ -119,6 +119,11 @@ class Part:
         """Bytes of weights a step reads from this part (for roofline accounting)."""
         return 0
 
+    def product_weights(self) -> list[torch.Tensor]:
+        """The [out, in] matrices this part multiplies every token of a step by (for a runner
+        that lets the product library time its algorithms for them before the first request)."""
+        return []
+
     def activation_bytes(self, tokens: int, itemsize: int) -> int:
         """Bytes of buffers this part asks the workspace for in a step of ``tokens`` tokens with
         activations of ``itemsize`` bytes. The cache pools are sized from what is free after the

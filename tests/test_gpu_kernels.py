@@ -261,6 +261,32 @@ def test_linear_bf16_other_paths(ops, m, n, k):
         assert rel(out, x.double() @ w.double().T) < (2e-5 if out_dtype == torch.float32 else 5e-3)
 
 
+def test_library_product_with_a_timed_algorithm(ops):
+    """The library times its algorithms for a shape (three matrices in turn) and keeps the
+    fastest, also for row counts within a quarter of the timed one: the products by what it
+    kept agree with float64, and what it kept is no slower than what it started from."""
+    assert ops._direct_library, "hipBLASLt was not found in the process"
+    n, k = 1000, 520
+    ws = [rnd(n, k, dtype=torch.bfloat16, seed=5 + i, scale=0.1) for i in range(3)]
+    res = ops.tune_linear(300, ws)
+    if res is None:
+        pytest.skip("this copy of hipBLASLt has no extension interface")
+    before, after = res
+    assert 0 < after <= before
+    for m in (300, 330, 250, 100):                    # the timed count, two neighbours, one too far to borrow
+        x = rnd(m, k, dtype=torch.bfloat16, seed=m)
+        for w in ws[:2]:
+            out = torch.full((m + 1, n), 7.0, dtype=torch.bfloat16, device=DEV)
+            ops.linear(x, w, out[:m])
+            assert rel(out[:m], x.double() @ w.double().T) < 5e-3 and torch.all(out[m] == 7.0)
+    assert ops.tune_linear(32, ws) is None            # small steps do not go to the library
+    assert ops.lib.psamd_gemm_lt_untune(1, 300, n, k) == 0
+    x = rnd(300, k, dtype=torch.bfloat16, seed=1)
+    out = torch.empty(300, n, dtype=torch.bfloat16, device=DEV)
+    ops.linear(x, ws[0], out)
+    assert rel(out, x.double() @ ws[0].double().T) < 5e-3
+
+
 def test_library_product_called_directly_and_through_torch(ops):
     """Large bfloat16 products go to hipBLASLt through the kernel library's own call (plans kept
     per shape); torch.mm is what remains if the library cannot be found. Both against float64,
