@@ -818,7 +818,7 @@ static bool lds_allowed(Kernel kernel, size_t bytes) {
                              static_cast<int>(bytes)) == hipSuccess;
 }
 
-// Which kernel a step's portions go to, when three or more query heads share a kv head
+// Which kernel a step's portions go to, when two or more query heads share a kv head
 // (measured on 256 compute units with 32 query heads on 8 kv heads; us per layer, per-head /
 // grouped, at head size 64 and at head size 128):
 //   256 on 1,792 cached     18 / 30      31 / 43       384 on 3,712 cached     48 / 53      94 / 78
@@ -836,8 +836,11 @@ enum class PrefillForm { kPerHead, kGrouped };
 
 static PrefillForm prefill_form(int n_tiles, int hq, int hkv, int head_dim) {
   const int group = hq / hkv;
-  if (group < 3) return PrefillForm::kPerHead;
   const int64_t workgroups = static_cast<int64_t>(n_tiles) * hkv * ((group + 3) / 4);
+  // Two query heads per kv head leave half of the grouped kernel's waves idle; sharing the keys
+  // and values still pays above head size 64 from one workgroup per compute unit on (16 heads on
+  // 8 at head size 128: 2,048 tokens 71 -> 55 us, 8,192 tokens 779 -> 647; at head size 64 a tie).
+  if (group < 2 || (group == 2 && (head_dim <= 64 || workgroups < 256))) return PrefillForm::kPerHead;
   return workgroups <= (head_dim <= 64 ? 128 : 80) ? PrefillForm::kPerHead : PrefillForm::kGrouped;
 }
 

@@ -415,6 +415,8 @@ def test_paged_attention_mixed_batch(ops, act, hq, hkv, d):
 @pytest.mark.parametrize("hq,hkv,d,new,old,window", [
     (32, 8, 64, [2048], [0], None),              # 512 workgroups, nothing cached: grouped, a kv head's tiles on one die
     (24, 8, 128, [2100], [0], None),             # three heads per kv head, an odd number of tiles, a last tile of 20
+    (16, 8, 128, [1100], [0], None),             # two heads per kv head at head size 128: grouped, half its waves spare
+    (16, 8, 128, [500], [600], None),            # the same with few workgroups: the per-head kernel
     (16, 4, 64, [2048, 2100], [0, 0], None),     # two prompts from position 0 in one step, 4 workgroups per tile
     (32, 8, 64, [512], [1536], None),            # 128 workgroups on a long prefix: the per-head kernel at this head size
     (32, 8, 64, [768], [1536], None),            # 192 workgroups on a long prefix: grouped
@@ -516,6 +518,7 @@ def test_attention_finds_one_far_key_among_hundreds(ops, act):
     (32, 8, 64, 800, 1248, None),       # grouped, on a cached prefix
     (32, 8, 64, 2048, 0, None),         # grouped, a whole prompt
     (24, 8, 128, 700, 500, None),       # head size 128, three heads per kv head
+    (16, 8, 128, 1100, 100, None),      # head size 128, two heads per kv head: grouped with spare waves
     (32, 8, 128, 4100, 0, None),        # head size 128, a long prompt: one wave per head
     (32, 8, 64, 2048, 0, 300),          # a whole prompt with a window
     (16, 4, 64, 600, 200, 100),         # grouped with a window
