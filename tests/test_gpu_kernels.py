@@ -412,6 +412,26 @@ def test_paged_attention_mixed_batch(ops, act, hq, hkv, d):
     assert rel(got, want) < (2e-5 if act == torch.float32 else 2e-2)
 
 
+@pytest.mark.parametrize("hq,hkv,d,longest,window", [
+    (32, 8, 64, 700, None),        # 40 requests x 8 kv heads: keys not split over workgroups
+    (32, 8, 64, 700, 150),         # the same with a window whose first pages were given back
+    (16, 8, 128, 3300, None),      # head size 128, long contexts
+    (16, 8, 128, 700, None),       # and short ones
+    (6, 3, 48, 300, None),         # a head size the matrix-core kernels do not take: the generic kernel
+])
+def test_decode_attention_of_many_requests(ops, hq, hkv, d, longest, window):
+    """Forty requests decode together, their contexts from 0 to ``longest`` tokens (empty, one
+    token, a page's edge, a tile's edge among them): with 256 (request, kv head) pairs or more
+    the keys are not split over workgroups and a wave runs through many tiles."""
+    rng = np.random.default_rng(longest + d)
+    old = [0, 1, 15, 16, 31, 32, 33, 63, 64, 127, 128, longest] + rng.integers(0, longest, 28).tolist()
+    new = [1] * len(old)
+    pages = sum(-(-(o + 1) // 16) for o in old) + 8
+    got, want = paged_case(ops, torch.bfloat16, hq, hkv, d, new, old, window=window, seed=7, num_blocks=pages,
+                           poison=float("nan"), give_back=window is not None)
+    assert rel(got, want) < 2e-2
+
+
 @pytest.mark.parametrize("hq,hkv,d,new,old,window", [
     (32, 8, 64, [2048], [0], None),              # 512 workgroups, nothing cached: grouped, a kv head's tiles on one die
     (24, 8, 128, [2100], [0], None),             # three heads per kv head, an odd number of tiles, a last tile of 20
