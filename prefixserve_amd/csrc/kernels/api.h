@@ -74,11 +74,16 @@ int psamd_attention_generic(void* stream, const void* qkv, int q_stride, void* o
 
 int psamd_attention_mfma_supports(int hq, int hkv, int head_dim);
 
+// Few query tiles on long contexts: their keys are cut into nsplit runs (what
+// psamd_attention_prefill_nsplit allows for the step's sizes, or fewer; 1: no cut) that
+// part_o [32 * n_tiles * hq * nsplit * head_dim] and part_ml [32 * n_tiles * hq * nsplit * 2] carry
+// to a merge kernel.
+int psamd_attention_prefill_nsplit(int n_tiles, int max_kv_len, int hq, int hkv, int head_dim);
 int psamd_attention_prefill(void* stream, const void* qkv, int q_stride, void* out, const void* kv,
                             const int32_t* pf_tiles, int n_tiles, int max_kv_len,
                             const int32_t* item_start, const int32_t* item_pos0,
                             const int32_t* table_off, const int32_t* block_ids, int hq, int hkv, int head_dim,
-                            float scale, int window);
+                            float scale, int window, float* part_o, float* part_ml, int nsplit);
 
 int psamd_attention_decode(void* stream, const void* qkv, int q_stride, void* out, const void* kv, float* part_o,
                            float* part_ml, const int32_t* dec_items, int n_dec, const int32_t* item_start,

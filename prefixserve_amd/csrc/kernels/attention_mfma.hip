@@ -317,13 +317,15 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
 // Measured and not kept: the scores of the next iteration issued before the softmax of the
 // current one (correct, no faster at head size 128, slower at 64 where it costs the second
 // workgroup per compute unit its registers), and the stores to LDS issued behind the barrier.
+constexpr int kMinSplitKeys = 512;   // a workgroup's share of a tile's keys is not cut below this
+
 template <int NS, int KT, int KP>
 __global__ __launch_bounds__(256 * KP, NS <= 4 ? 4 : 2) void attn_prefill_grouped_kernel(
     const bf16_t* __restrict__ qkv, int q_stride, bf16_t* __restrict__ out, const bf16_t* __restrict__ kv,
     const int32_t* __restrict__ pf_tiles, const int32_t* __restrict__ item_start,
     const int32_t* __restrict__ item_pos0, const int32_t* __restrict__ table_off,
     const int32_t* __restrict__ block_ids, int n_tiles, int hq, int hkv, int table_pages, float scale,
-    int window) {
+    int window, float* __restrict__ part_o, float* __restrict__ part_ml) {
   constexpr int D = 16 * NS;
   constexpr int DT = (D + 31) / 32;
   constexpr int KS = D + 8;                      // elements per key row in LDS
@@ -370,6 +372,28 @@ __global__ __launch_bounds__(256 * KP, NS <= 4 ? 4 : 2) void attn_prefill_groupe
   const int k_begin_vis = window > 0 ? max(0, first_pos - window + 1) : 0;   // the first key any query of the tile sees
   const int k_begin = k_begin_vis & ~(KEYS - 1);
   const float c = scale * 1.44269504088896340736f;  // scores are exponentiated in base 2
+  // With gridDim.z > 1 the tile's keys are dealt out to that many workgroups in runs of whole
+  // pairs of iterations, at least kMinSplitKeys each; every workgroup leaves its sum, its
+  // maximum and its unnormalized output in part_ml / part_o for the merge kernel. A tile with
+  // too few keys for all of them leaves the last ones nothing: they write an empty sum.
+  const int nsplit = gridDim.z;
+  int k_first = k_begin, k_last = last_pos;
+  int64_t part_slot = 0;
+  if (nsplit > 1) {
+    constexpr int PAIR = 2 * KEYS;
+    const int pairs = (last_pos - k_begin) / PAIR + 1;
+    const int per = max((pairs + nsplit - 1) / nsplit, kMinSplitKeys / PAIR);
+    k_first = k_begin + static_cast<int>(blockIdx.z) * per * PAIR;
+    k_last = min(last_pos, k_first + per * PAIR - 1);
+    part_slot = (static_cast<int64_t>(tile * 32 + col) * hq + h) * nsplit + blockIdx.z;
+    if (k_first > last_pos) {
+      if (part == 0 && head_valid && q_valid && hi == 0) {
+        part_ml[2 * part_slot] = -INFINITY;
+        part_ml[2 * part_slot + 1] = 0.f;
+      }
+      return;
+    }
+  }
   {
     const int32_t* gtable = block_ids + table_off[item];
     for (int i = threadIdx.x; i <= (last_pos >> 4); i += blockDim.x) table[i] = gtable[i];
@@ -507,7 +531,7 @@ __global__ __launch_bounds__(256 * KP, NS <= 4 ? 4 : 2) void attn_prefill_groupe
     // longer than one iteration, and with no branch around the loads the wait in front of a
     // store to LDS counts exactly the older set and leaves the newer one in flight.
     Pieces ra, rb;
-    int k0 = k_begin, stage = 0;
+    int k0 = k_first, stage = 0;
     load_global(ra, k0);
     load_global(rb, k0 + KEYS);
     auto iteration = [&](Pieces& r) {
@@ -528,7 +552,7 @@ __global__ __launch_bounds__(256 * KP, NS <= 4 ? 4 : 2) void attn_prefill_groupe
     do {
       iteration(ra);
       iteration(rb);
-    } while (k0 <= last_pos);
+    } while (k0 <= k_last);
   }
 
   if (KP > 1) {
@@ -569,9 +593,28 @@ __global__ __launch_bounds__(256 * KP, NS <= 4 ? 4 : 2) void attn_prefill_groupe
 #pragma unroll
         for (int v = 0; v < 16; ++v) o[dt][v] += f * src[(dt * 16 + v) * 64 + lane];
     }
+    m = mm;
     }
   }
   if (part != 0 || !head_valid || !q_valid) return;
+  if (nsplit > 1) {
+    // m is in units of the base-2 exponent; a query with no key in this run has m = -inf, l = 0.
+    if (hi == 0) {
+      part_ml[2 * part_slot] = m;
+      part_ml[2 * part_slot + 1] = l;
+    }
+    float* po = part_o + part_slot * D;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int v4 = 0; v4 < 4; ++v4) {
+        const int d = 32 * dt + 8 * v4 + 4 * hi;
+        if (d < D)
+          *reinterpret_cast<float4*>(po + d) =
+              float4{o[dt][4 * v4 + 0], o[dt][4 * v4 + 1], o[dt][4 * v4 + 2], o[dt][4 * v4 + 3]};
+      }
+    return;
+  }
   const float inv = 1.f / l;
   bf16_t* op = out + static_cast<int64_t>(t0 + qi) * (static_cast<int64_t>(hq) * D) + h * D;
 #pragma unroll
@@ -588,6 +631,40 @@ __global__ __launch_bounds__(256 * KP, NS <= 4 ? 4 : 2) void attn_prefill_groupe
         *reinterpret_cast<ushort4*>(op + d) = pk;
       }
     }
+}
+
+// One wave per (query, head) of the tiles whose keys were dealt out to nsplit workgroups above:
+// weighs their unnormalized outputs by 2^(m_s - max m), in the order of the runs, and writes
+// bfloat16. A run that held no key this query sees (m = -inf) is left out, its output unread.
+__global__ __launch_bounds__(256) void attn_prefill_merge_kernel(
+    const float* __restrict__ part_o, const float* __restrict__ part_ml, bf16_t* __restrict__ out,
+    const int32_t* __restrict__ pf_tiles, const int32_t* __restrict__ item_start, int hq, int d, int nsplit) {
+  const int row = blockIdx.x, tile = row >> 5, col = row & 31;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int h = blockIdx.y * 4 + wave;
+  const int item = pf_tiles[2 * tile];
+  const int q = pf_tiles[2 * tile + 1] + col;
+  const int t0 = item_start[item];
+  if (h >= hq || q >= item_start[item + 1] - t0) return;
+  const int64_t base = (static_cast<int64_t>(row) * hq + h) * nsplit;
+  float mm = -INFINITY;
+  for (int s = 0; s < nsplit; ++s) mm = fmaxf(mm, part_ml[2 * (base + s)]);
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};      // head sizes up to 256
+  float ll = 0.f;
+  for (int s = 0; s < nsplit; ++s) {
+    const float ms = part_ml[2 * (base + s)];
+    if (ms == -INFINITY) continue;
+    const float w = __builtin_amdgcn_exp2f(ms - mm);
+    ll += w * part_ml[2 * (base + s) + 1];
+    const float* po = part_o + (base + s) * d;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (lane + 64 * j < d) acc[j] += w * po[lane + 64 * j];
+  }
+  bf16_t* op = out + static_cast<int64_t>(t0 + q) * (static_cast<int64_t>(hq) * d) + static_cast<int64_t>(h) * d;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    if (lane + 64 * j < d) op[lane + 64 * j] = float_to_bf16(acc[j] / ll);
 }
 
 // ------------------------------------------------------------------ decode (split keys)
@@ -848,34 +925,65 @@ static PrefillForm prefill_form(int n_tiles, int hq, int hkv, int head_dim) {
   return workgroups <= (head_dim <= 64 ? 128 : 80) ? PrefillForm::kPerHead : PrefillForm::kGrouped;
 }
 
+// Into how many runs the grouped kernel cuts a tile's keys (1: not at all). Few query tiles on
+// many keys (a portion of a long prompt, a short tail behind a long context) are too few
+// workgroups for 256 compute units: their keys are then dealt out to more of them, up to as many
+// workgroups as run at once (two per compute unit up to head size 64, one above), each run no
+// shorter than 1,024 keys, and a merge kernel puts the runs together. Measured with 32 query heads
+// on 8 kv heads, us per layer at head size 64 / 128, no cut -> cut: 512 tokens on 7,680 cached
+// 90 -> 63 / 149 -> 96; 512 on 60,000 626 -> 334 / 1,057 -> 581; 128 on 8,064 48 -> 31 / 91 -> 42;
+// 20 on 16,000 89 -> 32 / 172 -> 45. Where the per-head kernel would run (few workgroups), fewer
+// than four runs lose to it (256 on 1,792: 17 -> 23 / 30 -> 34 with two); where the grouped
+// kernel would run without a cut, two runs pay from 4,096 keys on (512 on 3,584 at head size 128:
+// 78 -> 60) and, above 128 workgroups, from 8,192 on (1,024 on 3,072: 57 -> 65; on 15,000: 200 -> 193).
+static int prefill_nsplit(int n_tiles, int max_kv_len, int hq, int hkv, int head_dim) {
+  const int group = hq / hkv;
+  if (group < 2 || (group == 2 && head_dim <= 64)) return 1;      // these go to the per-head kernel
+  const int64_t workgroups = static_cast<int64_t>(n_tiles) * hkv * ((group + 3) / 4);
+  const int at_once = head_dim <= 64 ? 512 : 256;
+  if (2 * workgroups > at_once) return 1;
+  if (grouped_smem(head_dim, 1, 1, static_cast<int>(ceil_div(max_kv_len, kPage))) > 160 * 1024) return 1;
+  const int nsplit = static_cast<int>(std::min<int64_t>({at_once / workgroups, max_kv_len / 1024, 16}));
+  const bool per_head_else = workgroups <= (head_dim <= 64 ? 128 : 80);
+  if (per_head_else ? nsplit < 4 : max_kv_len < (workgroups <= 128 ? 4096 : 8192)) return 1;
+  return std::max(nsplit, 1);
+}
+
 template <int NS>
 static int launch_prefill(hipStream_t s, const void* qkv, int q_stride, void* out, const void* kv,
                           const int32_t* pf_tiles, int n_tiles, int table_pages,
                           const int32_t* item_start, const int32_t* item_pos0,
-                          const int32_t* table_off, const int32_t* block_ids, int hq, int hkv, float scale, int window) {
+                          const int32_t* table_off, const int32_t* block_ids, int hq, int hkv, float scale, int window,
+                          float* part_o, float* part_ml, int nsplit) {
   const int group = hq / hkv;
-  const PrefillForm form = prefill_form(n_tiles, hq, hkv, 16 * NS);
+  const PrefillForm form = nsplit > 1 ? PrefillForm::kGrouped : prefill_form(n_tiles, hq, hkv, 16 * NS);
   // The heads of a kv head share its keys and values through LDS, two waves per head (each its
   // own run of keys) if the stages fit, else one.
   if (form != PrefillForm::kPerHead) {
-    const dim3 grid(hkv * ((group + 3) / 4), n_tiles);
+    const dim3 grid(hkv * ((group + 3) / 4), n_tiles, nsplit);
 #define PSAMD_GROUPED(KP_)                                                                                         \
   {                                                                                                               \
     const size_t smem = grouped_smem(16 * NS, 1, KP_, table_pages);                                               \
     if (lds_allowed(attn_prefill_grouped_kernel<NS, 1, KP_>, smem)) {                                             \
       attn_prefill_grouped_kernel<NS, 1, KP_><<<grid, dim3(256 * KP_), smem, s>>>(                                \
           static_cast<const bf16_t*>(qkv), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(kv),   \
-          pf_tiles, item_start, item_pos0, table_off, block_ids, n_tiles, hq, hkv, table_pages, scale, window); \
-      return check_launch("psamd_attention_prefill");                                                             \
+          pf_tiles, item_start, item_pos0, table_off, block_ids, n_tiles, hq, hkv, table_pages, scale, window,   \
+          part_o, part_ml);                                                                                       \
+      const int rc = check_launch("psamd_attention_prefill");                                                     \
+      if (rc != 0 || nsplit == 1) return rc;                                                                      \
+      attn_prefill_merge_kernel<<<dim3(32 * n_tiles, (hq + 3) / 4), dim3(256), 0, s>>>(                           \
+          part_o, part_ml, static_cast<bf16_t*>(out), pf_tiles, item_start, hq, 16 * NS, nsplit);                 \
+      return check_launch("psamd_attention_prefill(merge)");                                                      \
     }                                                                                                             \
   }
     // From head size 96 on, where a compute unit holds one workgroup of eight waves, four
     // workgroups per compute unit's worth of tiles run 5% faster as two workgroups of four waves
     // (one wave per head): two barriers' worth of waves that do not wait for each other
     // (head size 128: 4,096 tokens 181 -> 171 us, 8,192 tokens 657 -> 623 us; 2,048 tokens 56 -> 67).
-    if (NS < 6 || static_cast<int64_t>(grid.x) * grid.y < 1024) PSAMD_GROUPED(2)
+    if (NS < 6 || static_cast<int64_t>(grid.x) * grid.y * grid.z < 1024) PSAMD_GROUPED(2)
     PSAMD_GROUPED(1)
 #undef PSAMD_GROUPED
+    PSAMD_REQUIRE(nsplit == 1, "no room in LDS for the kernel that splits a tile's keys");
   }
   attn_prefill_mfma_kernel<NS><<<dim3(hq, n_tiles), dim3(256), sizeof(int32_t) * static_cast<size_t>(table_pages), s>>>(
       static_cast<const bf16_t*>(qkv), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(kv), pf_tiles,
@@ -928,22 +1036,34 @@ int psamd_attention_mfma_supports(int hq, int hkv, int head_dim) {
   return dim_ok && group <= 64 && smem <= 64 * 1024 && hq <= 65535 && hkv <= 65535;
 }
 
+// Into how many runs psamd_attention_prefill may cut the keys of this step's query tiles; from 2
+// on it needs part_o and part_ml.
+int psamd_attention_prefill_nsplit(int n_tiles, int max_kv_len, int hq, int hkv, int head_dim) {
+  if (!psamd_attention_mfma_supports(hq, hkv, head_dim) || n_tiles <= 0) return 1;
+  return prefill_nsplit(n_tiles, max_kv_len, hq, hkv, head_dim);
+}
+
 // max_kv_len: the longest request of the step after it (sizes the block table staged in LDS).
+// nsplit: 1, or what psamd_attention_prefill_nsplit gave for these sizes (or less); part_o then
+// has room for 32 * n_tiles * hq * nsplit * head_dim floats and part_ml for 32 * n_tiles * hq * nsplit * 2.
 int psamd_attention_prefill(void* stream, const void* qkv, int q_stride, void* out, const void* kv,
                             const int32_t* pf_tiles, int n_tiles, int max_kv_len,
                             const int32_t* item_start,
                             const int32_t* item_pos0, const int32_t* table_off, const int32_t* block_ids, int hq,
-                            int hkv, int head_dim, float scale, int window) {
+                            int hkv, int head_dim, float scale, int window, float* part_o, float* part_ml, int nsplit) {
   PSAMD_REQUIRE(psamd_attention_mfma_supports(hq, hkv, head_dim), "shape not supported by the matrix-core kernels");
   PSAMD_REQUIRE(q_stride % 8 == 0, "query row stride must be a multiple of 8 elements");
   PSAMD_REQUIRE(max_kv_len >= 1 && max_kv_len <= 8192 * kPage, "context too long for the block table staged in LDS");
   if (n_tiles == 0) return 0;
   PSAMD_REQUIRE(n_tiles <= 65535, "too many query tiles for one launch");
+  PSAMD_REQUIRE(nsplit >= 1 && nsplit <= 16 && (nsplit == 1 || hq / hkv >= 2),
+                "nsplit must be in [1, 16], and 1 without shared kv heads");
+  PSAMD_REQUIRE(nsplit == 1 || (part_o != nullptr && part_ml != nullptr), "split keys need part_o and part_ml");
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int table_pages = static_cast<int>(ceil_div(max_kv_len, kPage));
 #define PSAMD_PF(NS_)                                                                                           \
   return launch_prefill<NS_>(s, qkv, q_stride, out, kv, pf_tiles, n_tiles, table_pages, item_start, \
-                             item_pos0, table_off, block_ids, hq, hkv, scale, window)
+                             item_pos0, table_off, block_ids, hq, hkv, scale, window, part_o, part_ml, nsplit)
   switch (head_dim / 16) {
     case 1: PSAMD_PF(1);
     case 2: PSAMD_PF(2);

@@ -55,8 +55,9 @@ _SIGNATURES = {
     "psamd_qkv_rope_append": [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp],
     "psamd_attention_generic": [_vp, _vp, _i32, _vp, _vp, _i32, _i64, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _f32, _i32],
     "psamd_attention_mfma_supports": [_i32, _i32, _i32],
+    "psamd_attention_prefill_nsplit": [_i32, _i32, _i32, _i32, _i32],
     "psamd_attention_prefill": [_vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _f32,
-                                _i32],
+                                _i32, _vp, _vp, _i32],
     "psamd_attention_decode": [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32,
                                _i32, _f32, _i32],
     "psamd_sample": [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32],
@@ -334,11 +335,22 @@ class HipOps:
         s = self._stream()
         if qkv.dtype == torch.bfloat16 and stride % 8 == 0 and self.mfma_attention_supported(hq, hkv, d):
             if ctx.num_prefill_tiles:
+                kv_len = self.fixed_kv_len or ctx.max_kv_len
+                # Few query tiles on a long context: the kernel deals their keys out to several
+                # workgroups, whose partial results pass through these buffers. They are asked
+                # for at the largest size such a step can need, so they never grow.
+                nsplit = self.lib.psamd_attention_prefill_nsplit(ctx.num_prefill_tiles, kv_len, hq, hkv, d)
+                part_o = part_ml = None
+                if nsplit > 1:
+                    rows = 32 * (512 // (hkv * (-(-(hq // hkv) // 4))))
+                    self._need(32 * ctx.num_prefill_tiles * nsplit <= rows, "attention: more split tiles than planned for")
+                    part_o = self.ws.get("attn.prefill_part_o", (rows * hq * d,), torch.float32).data_ptr()
+                    part_ml = self.ws.get("attn.prefill_part_ml", (rows * hq * 2,), torch.float32).data_ptr()
                 self._ok(self.lib.psamd_attention_prefill(
                     s, qkv.data_ptr(), stride, out.data_ptr(), kv.data_ptr(), ctx.pf_tiles.data_ptr(),
-                    ctx.num_prefill_tiles, self.fixed_kv_len or ctx.max_kv_len,
+                    ctx.num_prefill_tiles, kv_len,
                     ctx.item_start.data_ptr(), ctx.item_pos0.data_ptr(),
-                    g.table_off.data_ptr(), g.block_ids.data_ptr(), hq, hkv, d, scale, win))
+                    g.table_off.data_ptr(), g.block_ids.data_ptr(), hq, hkv, d, scale, win, part_o, part_ml, nsplit))
             if ctx.num_decode:
                 kv_len = self.fixed_kv_len or ctx.max_kv_len
                 if win:

@@ -84,8 +84,10 @@ class PagedAttention(Mixer):
 
     def activation_bytes(self, tokens: int, itemsize: int) -> int:
         # q/k/v, the attention output, the projected output (or its float32 partial sums).
+        # ... and what the attention kernels pass between the workgroups that share a query's keys.
+        split_rows = 32 * (512 // (self.num_kv_heads * -(-(self.num_heads // self.num_kv_heads) // 4)))
         return tokens * ((self.q_size + 2 * self.kv_size) + self.q_size) * itemsize + 8 * 64 * self.hidden_size * 4 \
-            + tokens * self.hidden_size * itemsize
+            + tokens * self.hidden_size * itemsize + split_rows * self.num_heads * (self.head_dim + 2) * 4
 
     def forward(self, x: torch.Tensor, ctx: "StepContext", cache: Any, state: torch.Tensor | None,
                 writes_cache: bool) -> torch.Tensor:

@@ -438,7 +438,13 @@ def test_decode_attention_of_many_requests(ops, hq, hkv, d, longest, window):
     (16, 8, 128, [1100], [0], None),             # two heads per kv head at head size 128: grouped, half its waves spare
     (16, 8, 128, [500], [600], None),            # the same with few workgroups: the per-head kernel
     (16, 4, 64, [2048, 2100], [0, 0], None),     # two prompts from position 0 in one step, 4 workgroups per tile
-    (32, 8, 64, [512], [1536], None),            # 128 workgroups on a long prefix: the per-head kernel at this head size
+    (32, 8, 64, [512], [1536], None),            # 128 workgroups on a prefix: the per-head kernel at this head size
+    (32, 8, 64, [512], [7680], None),            # a portion of a long prompt: each tile's keys in four runs
+    (32, 8, 128, [40], [16000], None),           # a short tail behind a long context: sixteen workgroups, fifteen runs each
+    (24, 8, 128, [20, 300], [9000, 100], None),  # runs that a short request leaves empty, beside a long one; a spare wave
+    (16, 4, 64, [64], [5000], 1500),             # split runs inside a window
+    (40, 2, 64, [33], [6000], None),             # five workgroups per kv head, each tile's keys in five runs
+    (32, 8, 128, [512], [3584], None),           # 128 workgroups at head size 128: two runs
     (32, 8, 64, [768], [1536], None),            # 192 workgroups on a long prefix: grouped
     (32, 8, 128, [512], [1536], None),           # 128 workgroups at head size 128: grouped
     (32, 8, 128, [4100], [0], None),             # 1,032 workgroups at head size 128: grouped, one wave per head
@@ -447,7 +453,7 @@ def test_decode_attention_of_many_requests(ops, hq, hkv, d, longest, window):
     (6, 2, 256, [1500, 1000], [0, 200], None),   # head size 256
     (16, 4, 64, [700, 300], [50, 0], 100),       # grouped, with a window
     (32, 8, 64, [2048], [0], 300),               # a long prompt with a window
-    (32, 8, 64, [100], [1948], None),            # few tiles: the per-head kernel
+    (32, 8, 64, [100], [1948], None),            # few tiles on few keys: the per-head kernel
 ])
 def test_prefill_attention_in_each_form(ops, hq, hkv, d, new, old, window):
     """The portions of a step go to the per-head or to the grouped kernel by their number of tiles
@@ -463,6 +469,8 @@ def test_prefill_attention_in_each_form(ops, hq, hkv, d, new, old, window):
     (32, 8, 64, [2040], [0], None),                 # grouped; the last page has 8 slots nobody wrote
     (32, 8, 64, [500], [1530], None),               # the per-head kernel on a cached prefix
     (32, 8, 64, [700], [1330], None),               # grouped on a cached prefix
+    (32, 8, 64, [300], [5000], None),               # grouped, the keys of a tile in five runs
+    (24, 8, 128, [20, 300], [9000, 100], None),     # runs left empty
     (24, 8, 128, [2100, 1], [0, 77], None),
     (8, 2, 64, [70, 1, 1, 9], [0, 40, 130, 64], 33),        # windows whose first pages were given back
     (16, 4, 64, [700, 300, 1], [150, 0, 900], 100),
@@ -535,6 +543,9 @@ def test_attention_finds_one_far_key_among_hundreds(ops, act):
 @pytest.mark.parametrize("hq,hkv,d,new,old,window", [
     (32, 8, 64, 100, 1948, None),       # few tiles: the per-head kernel, keys split over its four waves
     (32, 8, 64, 512, 1536, None),       # the per-head kernel on a cached prefix, 128 workgroups' worth
+    (32, 8, 64, 512, 7680, None),       # four runs of 2,048 keys
+    (32, 8, 128, 40, 8000, None),       # head size 128, seven runs of 1,152 keys
+    (16, 4, 64, 64, 5000, 1500),        # runs inside a window
     (32, 8, 64, 800, 1248, None),       # grouped, on a cached prefix
     (32, 8, 64, 2048, 0, None),         # grouped, a whole prompt
     (24, 8, 128, 700, 500, None),       # head size 128, three heads per kv head
@@ -568,10 +579,13 @@ def test_prefill_attention_finds_one_planted_key(ops, hq, hkv, d, new, old, wind
               (last, 64, True), (last, old - 1 if old else 95, True), (last, old, True), (last, last - 32, True),
               (last, last, True), (old + 33, 32, True), (old + 33, old + 33, True), (old + new // 2, 127, True),
               (old + new // 2, 128, True), (old + 1, 0, True)]
+    # where runs of keys that different workgroups take may begin and end
+    plants += [(last, p + e, True) for p in range(512, total, 128) for e in (-1, 0)]
     if window is not None:
         plants = [(q, max(q - window + 1, 0), True) for q, _, _ in plants[:4]] + \
                  [(last, last - window + 1, True), (last, last - window, False), (old + new // 2, old + new // 2 - window, False),
-                  (old + 40, max(old + 40 - window + 1, 0), True), (last, last - 5, True)]
+                  (old + 40, max(old + 40 - window + 1, 0), True), (last, last - 5, True)] + \
+                 [(last, p + e, True) for p in range((last - window + 512) & ~127, last, 128) for e in (-1, 0)]
     for q_pos, far, seen in plants:
         if not 0 <= far <= q_pos:
             continue
