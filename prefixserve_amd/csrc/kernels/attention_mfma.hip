@@ -67,6 +67,8 @@ __device__ __forceinline__ bf16x8 zero_unless(bf16x8 v, Keep keep) {
 
 // ------------------------------------------------------------------ prefill
 
+constexpr int kMinSplitKeys = 512;   // a workgroup's share of a tile's keys is not cut below this
+
 // NS = D / 16. A workgroup owns 32 consecutive queries of one item and one query head; its
 // 4 waves take the 32-key tiles in turn and merge by log-sum-exp through LDS. Splitting the
 // keys (not the queries) over the waves keeps the longest dependent chain of tiles four
@@ -82,7 +84,8 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
     const bf16_t* __restrict__ qkv, int q_stride, bf16_t* __restrict__ out, const bf16_t* __restrict__ kv,
     const int32_t* __restrict__ pf_tiles, const int32_t* __restrict__ item_start,
     const int32_t* __restrict__ item_pos0, const int32_t* __restrict__ table_off,
-    const int32_t* __restrict__ block_ids, int hq, int hkv, float scale, int window) {
+    const int32_t* __restrict__ block_ids, int hq, int hkv, float scale, int window,
+    float* __restrict__ part_o, float* __restrict__ part_ml) {
   constexpr int D = 16 * NS;
   constexpr int DT = (D + 31) / 32;
   constexpr int DTC = DT < 2 ? DT : 2;      // d-tiles merged per pass (bounds the LDS buffer)
@@ -114,6 +117,26 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
   const int k_begin_vis = window > 0 ? max(0, first_pos - window + 1) : 0;   // the first key any query of the tile sees
   const int k_begin = k_begin_vis & ~31;
   const float c = scale * 1.44269504088896340736f;  // scores are exponentiated in base 2
+  // With gridDim.z > 1 the tile's keys are dealt out to that many workgroups in runs of whole
+  // rounds of the four waves, at least kMinSplitKeys each, for the merge kernel to put together
+  // (see the grouped kernel below); a tile with too few keys leaves the last runs empty.
+  const int nsplit = gridDim.z;
+  int k_first = k_begin, k_last = last_pos;
+  int64_t part_slot = 0;
+  if (nsplit > 1) {
+    const int rounds = (last_pos - k_begin) / 128 + 1;
+    const int per = max((rounds + nsplit - 1) / nsplit, kMinSplitKeys / 128);
+    k_first = k_begin + static_cast<int>(blockIdx.z) * per * 128;
+    k_last = min(last_pos, k_first + per * 128 - 1);
+    part_slot = (static_cast<int64_t>(tile * 32 + col) * hq + h) * nsplit + blockIdx.z;
+    if (k_first > last_pos) {
+      if (wave == 0 && q_valid && hi == 0) {
+        part_ml[2 * part_slot] = -INFINITY;
+        part_ml[2 * part_slot + 1] = 0.f;
+      }
+      return;
+    }
+  }
   {
     const int32_t* gtable = block_ids + table_off[item];
     for (int i = threadIdx.x; i <= (last_pos >> 4); i += blockDim.x) table[i] = gtable[i];
@@ -218,8 +241,8 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
 
   {
     Tile ta, tb;
-    int k0 = k_begin + 32 * wave;
-    if (k0 <= last_pos) {
+    int k0 = k_first + 32 * wave;
+    if (k0 <= k_last) {
       load_tile(ta, k0);
       while (true) {
         // The next tile is loaded whether or not it exists (addresses are clamped to the last
@@ -228,11 +251,11 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
         load_tile(tb, k0 + 128);
         compute(ta, k0);
         k0 += 128;
-        if (k0 > last_pos) break;
+        if (k0 > k_last) break;
         load_tile(ta, k0 + 128);
         compute(tb, k0);
         k0 += 128;
-        if (k0 > last_pos) break;
+        if (k0 > k_last) break;
       }
     }
   }
@@ -254,7 +277,12 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
     ll += f * sm_l[w][col];
     if (w == wave) mine = f;
   }
-  const float inv = 1.f / ll;
+  // One run of several: the sum, the maximum and the output as it is go to the merge kernel.
+  const float inv = nsplit > 1 ? 1.f : 1.f / ll;
+  if (nsplit > 1 && wave == 0 && q_valid && hi == 0) {
+    part_ml[2 * part_slot] = mm;
+    part_ml[2 * part_slot + 1] = ll;
+  }
   bf16_t* op = out + static_cast<int64_t>(t0 + qi) * (static_cast<int64_t>(hq) * D) + h * D;
 #pragma unroll
   for (int d0 = 0; d0 < DT; d0 += DTC) {
@@ -280,7 +308,10 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
 #pragma unroll
         for (int v4 = 0; v4 < 4; ++v4) {
           const int d = 32 * (d0 + dt) + 8 * v4 + 4 * hi;
-          if (d < D) {
+          if (d < D && nsplit > 1) {
+            *reinterpret_cast<float4*>(part_o + part_slot * D + d) =
+                float4{r[4 * v4 + 0], r[4 * v4 + 1], r[4 * v4 + 2], r[4 * v4 + 3]};
+          } else if (d < D) {
             ushort4 pk;
             pk.x = float_to_bf16(r[4 * v4 + 0] * inv);
             pk.y = float_to_bf16(r[4 * v4 + 1] * inv);
@@ -317,8 +348,6 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
 // Measured and not kept: the scores of the next iteration issued before the softmax of the
 // current one (correct, no faster at head size 128, slower at 64 where it costs the second
 // workgroup per compute unit its registers), and the stores to LDS issued behind the barrier.
-constexpr int kMinSplitKeys = 512;   // a workgroup's share of a tile's keys is not cut below this
-
 template <int NS, int KT, int KP>
 __global__ __launch_bounds__(256 * KP, NS <= 4 ? 4 : 2) void attn_prefill_grouped_kernel(
     const bf16_t* __restrict__ qkv, int q_stride, bf16_t* __restrict__ out, const bf16_t* __restrict__ kv,
@@ -938,7 +967,15 @@ static PrefillForm prefill_form(int n_tiles, int hq, int hkv, int head_dim) {
 // 78 -> 60) and, above 128 workgroups, from 8,192 on (1,024 on 3,072: 57 -> 65; on 15,000: 200 -> 193).
 static int prefill_nsplit(int n_tiles, int max_kv_len, int hq, int hkv, int head_dim) {
   const int group = hq / hkv;
-  if (group < 2 || (group == 2 && head_dim <= 64)) return 1;      // these go to the per-head kernel
+  if (group <= 2) {
+    // The per-head kernel, a workgroup per (tile, query head): runs of 1,024 keys or more, up to
+    // one workgroup per compute unit (more lost again). 32 heads on 32 at head size 128: 64 tokens
+    // on 4,032 cached 51 -> 26 us, 20 on 16,000 172 -> 56; 16 heads on 8: 256 on 7,936 93 -> 57,
+    // 256 on 60,000 622 -> 323.
+    const int64_t workgroups = static_cast<int64_t>(n_tiles) * hq;
+    if (2 * workgroups > 256) return 1;
+    return static_cast<int>(std::max<int64_t>(1, std::min<int64_t>({256 / workgroups, max_kv_len / 1024, 16})));
+  }
   const int64_t workgroups = static_cast<int64_t>(n_tiles) * hkv * ((group + 3) / 4);
   const int at_once = head_dim <= 64 ? 512 : 256;
   if (2 * workgroups > at_once) return 1;
@@ -956,7 +993,8 @@ static int launch_prefill(hipStream_t s, const void* qkv, int q_stride, void* ou
                           const int32_t* table_off, const int32_t* block_ids, int hq, int hkv, float scale, int window,
                           float* part_o, float* part_ml, int nsplit) {
   const int group = hq / hkv;
-  const PrefillForm form = nsplit > 1 ? PrefillForm::kGrouped : prefill_form(n_tiles, hq, hkv, 16 * NS);
+  const PrefillForm form = nsplit > 1 ? (group <= 2 ? PrefillForm::kPerHead : PrefillForm::kGrouped)
+                                      : prefill_form(n_tiles, hq, hkv, 16 * NS);
   // The heads of a kv head share its keys and values through LDS, two waves per head (each its
   // own run of keys) if the stages fit, else one.
   if (form != PrefillForm::kPerHead) {
@@ -983,12 +1021,15 @@ static int launch_prefill(hipStream_t s, const void* qkv, int q_stride, void* ou
     if (NS < 6 || static_cast<int64_t>(grid.x) * grid.y * grid.z < 1024) PSAMD_GROUPED(2)
     PSAMD_GROUPED(1)
 #undef PSAMD_GROUPED
-    PSAMD_REQUIRE(nsplit == 1, "no room in LDS for the kernel that splits a tile's keys");
   }
-  attn_prefill_mfma_kernel<NS><<<dim3(hq, n_tiles), dim3(256), sizeof(int32_t) * static_cast<size_t>(table_pages), s>>>(
+  attn_prefill_mfma_kernel<NS><<<dim3(hq, n_tiles, nsplit), dim3(256), sizeof(int32_t) * static_cast<size_t>(table_pages), s>>>(
       static_cast<const bf16_t*>(qkv), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(kv), pf_tiles,
-      item_start, item_pos0, table_off, block_ids, hq, hkv, scale, window);
-  return check_launch("psamd_attention_prefill");
+      item_start, item_pos0, table_off, block_ids, hq, hkv, scale, window, part_o, part_ml);
+  const int rc = check_launch("psamd_attention_prefill");
+  if (rc != 0 || nsplit == 1) return rc;
+  attn_prefill_merge_kernel<<<dim3(32 * n_tiles, (hq + 3) / 4), dim3(256), 0, s>>>(
+      part_o, part_ml, static_cast<bf16_t*>(out), pf_tiles, item_start, hq, 16 * NS, nsplit);
+  return check_launch("psamd_attention_prefill(merge)");
 }
 
 template <int NS, int CT>
@@ -1056,8 +1097,7 @@ int psamd_attention_prefill(void* stream, const void* qkv, int q_stride, void* o
   PSAMD_REQUIRE(max_kv_len >= 1 && max_kv_len <= 8192 * kPage, "context too long for the block table staged in LDS");
   if (n_tiles == 0) return 0;
   PSAMD_REQUIRE(n_tiles <= 65535, "too many query tiles for one launch");
-  PSAMD_REQUIRE(nsplit >= 1 && nsplit <= 16 && (nsplit == 1 || hq / hkv >= 2),
-                "nsplit must be in [1, 16], and 1 without shared kv heads");
+  PSAMD_REQUIRE(nsplit >= 1 && nsplit <= 16, "nsplit must be in [1, 16]");
   PSAMD_REQUIRE(nsplit == 1 || (part_o != nullptr && part_ml != nullptr), "split keys need part_o and part_ml");
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int table_pages = static_cast<int>(ceil_div(max_kv_len, kPage));

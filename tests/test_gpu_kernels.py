@@ -445,6 +445,8 @@ def test_decode_attention_of_many_requests(ops, hq, hkv, d, longest, window):
     (16, 4, 64, [64], [5000], 1500),             # split runs inside a window
     (40, 2, 64, [33], [6000], None),             # five workgroups per kv head, each tile's keys in five runs
     (32, 8, 128, [512], [3584], None),           # 128 workgroups at head size 128: two runs
+    (8, 8, 128, [100, 40], [5000, 300], None),   # one query head per kv head: the per-head kernel, eight runs, some empty
+    (16, 8, 64, [200], [3000], 2500),            # two query heads per kv head, a window: the per-head kernel, two runs
     (32, 8, 64, [768], [1536], None),            # 192 workgroups on a long prefix: grouped
     (32, 8, 128, [512], [1536], None),           # 128 workgroups at head size 128: grouped
     (32, 8, 128, [4100], [0], None),             # 1,032 workgroups at head size 128: grouped, one wave per head
@@ -471,6 +473,7 @@ def test_prefill_attention_in_each_form(ops, hq, hkv, d, new, old, window):
     (32, 8, 64, [700], [1330], None),               # grouped on a cached prefix
     (32, 8, 64, [300], [5000], None),               # grouped, the keys of a tile in five runs
     (24, 8, 128, [20, 300], [9000, 100], None),     # runs left empty
+    (8, 8, 128, [100, 40], [5000, 300], None),      # the per-head kernel with runs
     (24, 8, 128, [2100, 1], [0, 77], None),
     (8, 2, 64, [70, 1, 1, 9], [0, 40, 130, 64], 33),        # windows whose first pages were given back
     (16, 4, 64, [700, 300, 1], [150, 0, 900], 100),
@@ -546,6 +549,8 @@ def test_attention_finds_one_far_key_among_hundreds(ops, act):
     (32, 8, 64, 512, 7680, None),       # four runs of 2,048 keys
     (32, 8, 128, 40, 8000, None),       # head size 128, seven runs of 1,152 keys
     (16, 4, 64, 64, 5000, 1500),        # runs inside a window
+    (4, 4, 128, 70, 6000, None),        # the per-head kernel, five runs
+    (16, 8, 64, 90, 4100, None),        # two query heads per kv head: the per-head kernel, four runs
     (32, 8, 64, 800, 1248, None),       # grouped, on a cached prefix
     (32, 8, 64, 2048, 0, None),         # grouped, a whole prompt
     (24, 8, 128, 700, 500, None),       # head size 128, three heads per kv head
