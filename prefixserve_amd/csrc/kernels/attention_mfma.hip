@@ -662,38 +662,63 @@ __global__ __launch_bounds__(256 * KP, NS <= 4 ? 4 : 2) void attn_prefill_groupe
     }
 }
 
-// One wave per (query, head) of the tiles whose keys were dealt out to nsplit workgroups above:
-// weighs their unnormalized outputs by 2^(m_s - max m), in the order of the runs, and writes
-// bfloat16. A run that held no key this query sees (m = -inf) is left out, its output unread.
+// Puts together the runs that the two kernels above cut a tile's keys into: for each (query,
+// head) the unnormalized outputs are weighed by 2^(m_s - max m), added in the order of the runs,
+// divided by the weighed sum and written as bfloat16. A thread owns four dimensions of one
+// (query, head) pair, D / 4 threads a pair, the pairs of a workgroup next to each other in
+// memory; the statistics of all runs are asked for at once, then all partial outputs. A run that
+// held no key this query sees (m = -inf) counts as nothing whatever its output holds: it was
+// never written.
+constexpr int kMaxPrefillSplit = 16;
+
 __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, bf16_t* __restrict__ out,
-    const int32_t* __restrict__ pf_tiles, const int32_t* __restrict__ item_start, int hq, int d, int nsplit) {
-  const int row = blockIdx.x, tile = row >> 5, col = row & 31;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int h = blockIdx.y * 4 + wave;
+    const int32_t* __restrict__ pf_tiles, const int32_t* __restrict__ item_start, int64_t pairs, int hq, int d,
+    int nsplit) {
+  const int per_pair = d >> 2;                         // threads per pair
+  const int pairs_per_block = 256 / per_pair;
+  const int sub = threadIdx.x / per_pair, chunk = threadIdx.x - sub * per_pair;
+  const int64_t pair = static_cast<int64_t>(blockIdx.x) * pairs_per_block + sub;
+  if (sub >= pairs_per_block || pair >= pairs) return;
+  const int row = static_cast<int>(pair / hq), h = static_cast<int>(pair - static_cast<int64_t>(row) * hq);
+  const int tile = row >> 5, col = row & 31;
   const int item = pf_tiles[2 * tile];
   const int q = pf_tiles[2 * tile + 1] + col;
   const int t0 = item_start[item];
-  if (h >= hq || q >= item_start[item + 1] - t0) return;
-  const int64_t base = (static_cast<int64_t>(row) * hq + h) * nsplit;
+  if (q >= item_start[item + 1] - t0) return;
+  const float2* ml = reinterpret_cast<const float2*>(part_ml) + pair * nsplit;
+  const float4* po = reinterpret_cast<const float4*>(part_o + pair * nsplit * d) + chunk;
+  float2 st[kMaxPrefillSplit];
+#pragma unroll
+  for (int s = 0; s < kMaxPrefillSplit; ++s) st[s] = s < nsplit ? ml[s] : float2{-INFINITY, 0.f};
+  float4 part[kMaxPrefillSplit];
+#pragma unroll
+  for (int s = 0; s < kMaxPrefillSplit; ++s)
+    if (s < nsplit) part[s] = po[s * per_pair];
   float mm = -INFINITY;
-  for (int s = 0; s < nsplit; ++s) mm = fmaxf(mm, part_ml[2 * (base + s)]);
-  float acc[4] = {0.f, 0.f, 0.f, 0.f};      // head sizes up to 256
+#pragma unroll
+  for (int s = 0; s < kMaxPrefillSplit; ++s) mm = fmaxf(mm, st[s].x);
+  float4 acc = {0.f, 0.f, 0.f, 0.f};
   float ll = 0.f;
-  for (int s = 0; s < nsplit; ++s) {
-    const float ms = part_ml[2 * (base + s)];
-    if (ms == -INFINITY) continue;
-    const float w = __builtin_amdgcn_exp2f(ms - mm);
-    ll += w * part_ml[2 * (base + s) + 1];
-    const float* po = part_o + (base + s) * d;
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      if (lane + 64 * j < d) acc[j] += w * po[lane + 64 * j];
+  for (int s = 0; s < kMaxPrefillSplit; ++s) {
+    if (s < nsplit && st[s].x != -INFINITY) {
+      const float w = __builtin_amdgcn_exp2f(st[s].x - mm);
+      ll += w * st[s].y;
+      acc.x += w * part[s].x;
+      acc.y += w * part[s].y;
+      acc.z += w * part[s].z;
+      acc.w += w * part[s].w;
+    }
   }
-  bf16_t* op = out + static_cast<int64_t>(t0 + q) * (static_cast<int64_t>(hq) * d) + static_cast<int64_t>(h) * d;
-#pragma unroll
-  for (int j = 0; j < 4; ++j)
-    if (lane + 64 * j < d) op[lane + 64 * j] = float_to_bf16(acc[j] / ll);
+  const float inv = 1.f / ll;
+  ushort4 pk;
+  pk.x = float_to_bf16(acc.x * inv);
+  pk.y = float_to_bf16(acc.y * inv);
+  pk.z = float_to_bf16(acc.z * inv);
+  pk.w = float_to_bf16(acc.w * inv);
+  *reinterpret_cast<ushort4*>(out + static_cast<int64_t>(t0 + q) * (static_cast<int64_t>(hq) * d) +
+                              static_cast<int64_t>(h) * d + 4 * chunk) = pk;
 }
 
 // ------------------------------------------------------------------ decode (split keys)
@@ -954,17 +979,28 @@ static PrefillForm prefill_form(int n_tiles, int hq, int hkv, int head_dim) {
   return workgroups <= (head_dim <= 64 ? 128 : 80) ? PrefillForm::kPerHead : PrefillForm::kGrouped;
 }
 
+static int launch_prefill_merge(hipStream_t s, const float* part_o, const float* part_ml, void* out,
+                                const int32_t* pf_tiles, const int32_t* item_start, int n_tiles, int hq, int head_dim,
+                                int nsplit) {
+  const int64_t pairs = 32LL * n_tiles * hq;
+  const int pairs_per_block = 256 / (head_dim / 4);
+  attn_prefill_merge_kernel<<<dim3(static_cast<unsigned>(ceil_div(pairs, pairs_per_block))), dim3(256), 0, s>>>(
+      part_o, part_ml, static_cast<bf16_t*>(out), pf_tiles, item_start, pairs, hq, head_dim, nsplit);
+  return check_launch("psamd_attention_prefill(merge)");
+}
+
 // Into how many runs the grouped kernel cuts a tile's keys (1: not at all). Few query tiles on
 // many keys (a portion of a long prompt, a short tail behind a long context) are too few
 // workgroups for 256 compute units: their keys are then dealt out to more of them, up to as many
 // workgroups as run at once (two per compute unit up to head size 64, one above), each run no
-// shorter than 1,024 keys, and a merge kernel puts the runs together. Measured with 32 query heads
+// shorter than 512 keys, and a merge kernel puts the runs together. Measured with 32 query heads
 // on 8 kv heads, us per layer at head size 64 / 128, no cut -> cut: 512 tokens on 7,680 cached
-// 90 -> 63 / 149 -> 96; 512 on 60,000 626 -> 334 / 1,057 -> 581; 128 on 8,064 48 -> 31 / 91 -> 42;
-// 20 on 16,000 89 -> 32 / 172 -> 45. Where the per-head kernel would run (few workgroups), fewer
-// than four runs lose to it (256 on 1,792: 17 -> 23 / 30 -> 34 with two); where the grouped
-// kernel would run without a cut, two runs pay from 4,096 keys on (512 on 3,584 at head size 128:
-// 78 -> 60) and, above 128 workgroups, from 8,192 on (1,024 on 3,072: 57 -> 65; on 15,000: 200 -> 193).
+// 92 -> 60 / 148 -> 94; 512 on 60,000 625 -> 332 / 1,045 -> 590; 128 on 8,064 48 -> 27 / 92 -> 37;
+// 20 on 16,000 88 -> 23 / 170 -> 32. Where the per-head kernel would run (few workgroups), fewer
+// than four runs lose to it, and so do runs of under 1,024 keys once it has a workgroup per
+// compute unit itself (256 on 1,792: 17 -> 20 with four); where the grouped kernel would run
+// without a cut, two runs pay from 4,096 keys on (512 on 3,584 at head size 128: 78 -> 58) and,
+// above 128 workgroups, from 8,192 on (1,024 on 3,072: 56 -> 60; on 15,000: 199 -> 183).
 static int prefill_nsplit(int n_tiles, int max_kv_len, int hq, int hkv, int head_dim) {
   const int group = hq / hkv;
   if (group <= 2) {
@@ -980,9 +1016,13 @@ static int prefill_nsplit(int n_tiles, int max_kv_len, int hq, int hkv, int head
   const int at_once = head_dim <= 64 ? 512 : 256;
   if (2 * workgroups > at_once) return 1;
   if (grouped_smem(head_dim, 1, 1, static_cast<int>(ceil_div(max_kv_len, kPage))) > 160 * 1024) return 1;
-  const int nsplit = static_cast<int>(std::min<int64_t>({at_once / workgroups, max_kv_len / 1024, 16}));
+  const int nsplit = static_cast<int>(std::min<int64_t>({at_once / workgroups, max_kv_len / kMinSplitKeys, kMaxPrefillSplit}));
   const bool per_head_else = workgroups <= (head_dim <= 64 ? 128 : 80);
-  if (per_head_else ? nsplit < 4 : max_kv_len < (workgroups <= 128 ? 4096 : 8192)) return 1;
+  if (per_head_else) {
+    if (nsplit < 4 || (static_cast<int64_t>(n_tiles) * hq >= 256 && max_kv_len < 4096)) return 1;
+  } else if (max_kv_len < (workgroups <= 128 ? 4096 : 8192)) {
+    return 1;
+  }
   return std::max(nsplit, 1);
 }
 
@@ -1009,9 +1049,7 @@ static int launch_prefill(hipStream_t s, const void* qkv, int q_stride, void* ou
           part_o, part_ml);                                                                                       \
       const int rc = check_launch("psamd_attention_prefill");                                                     \
       if (rc != 0 || nsplit == 1) return rc;                                                                      \
-      attn_prefill_merge_kernel<<<dim3(32 * n_tiles, (hq + 3) / 4), dim3(256), 0, s>>>(                           \
-          part_o, part_ml, static_cast<bf16_t*>(out), pf_tiles, item_start, hq, 16 * NS, nsplit);                 \
-      return check_launch("psamd_attention_prefill(merge)");                                                      \
+      return launch_prefill_merge(s, part_o, part_ml, out, pf_tiles, item_start, n_tiles, hq, 16 * NS, nsplit);   \
     }                                                                                                             \
   }
     // From head size 96 on, where a compute unit holds one workgroup of eight waves, four
@@ -1027,9 +1065,7 @@ static int launch_prefill(hipStream_t s, const void* qkv, int q_stride, void* ou
       item_start, item_pos0, table_off, block_ids, hq, hkv, scale, window, part_o, part_ml);
   const int rc = check_launch("psamd_attention_prefill");
   if (rc != 0 || nsplit == 1) return rc;
-  attn_prefill_merge_kernel<<<dim3(32 * n_tiles, (hq + 3) / 4), dim3(256), 0, s>>>(
-      part_o, part_ml, static_cast<bf16_t*>(out), pf_tiles, item_start, hq, 16 * NS, nsplit);
-  return check_launch("psamd_attention_prefill(merge)");
+  return launch_prefill_merge(s, part_o, part_ml, out, pf_tiles, item_start, n_tiles, hq, 16 * NS, nsplit);
 }
 
 template <int NS, int CT>
@@ -1097,7 +1133,7 @@ int psamd_attention_prefill(void* stream, const void* qkv, int q_stride, void* o
   PSAMD_REQUIRE(max_kv_len >= 1 && max_kv_len <= 8192 * kPage, "context too long for the block table staged in LDS");
   if (n_tiles == 0) return 0;
   PSAMD_REQUIRE(n_tiles <= 65535, "too many query tiles for one launch");
-  PSAMD_REQUIRE(nsplit >= 1 && nsplit <= 16, "nsplit must be in [1, 16]");
+  PSAMD_REQUIRE(nsplit >= 1 && nsplit <= kMaxPrefillSplit, "nsplit must be in [1, 16]");
   PSAMD_REQUIRE(nsplit == 1 || (part_o != nullptr && part_ml != nullptr), "split keys need part_o and part_ml");
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int table_pages = static_cast<int>(ceil_div(max_kv_len, kPage));

@@ -455,7 +455,8 @@ def test_decode_attention_of_many_requests(ops, hq, hkv, d, longest, window):
     (6, 2, 256, [1500, 1000], [0, 200], None),   # head size 256
     (16, 4, 64, [700, 300], [50, 0], 100),       # grouped, with a window
     (32, 8, 64, [2048], [0], 300),               # a long prompt with a window
-    (32, 8, 64, [100], [1948], None),            # few tiles on few keys: the per-head kernel
+    (32, 8, 64, [100], [1948], None),            # few tiles: grouped, four runs of 512 keys
+    (32, 8, 64, [100], [600], None),             # few tiles on few keys: the per-head kernel
 ])
 def test_prefill_attention_in_each_form(ops, hq, hkv, d, new, old, window):
     """The portions of a step go to the per-head or to the grouped kernel by their number of tiles
@@ -544,7 +545,8 @@ def test_attention_finds_one_far_key_among_hundreds(ops, act):
 
 
 @pytest.mark.parametrize("hq,hkv,d,new,old,window", [
-    (32, 8, 64, 100, 1948, None),       # few tiles: the per-head kernel, keys split over its four waves
+    (32, 8, 64, 100, 1948, None),       # few tiles: grouped, four runs of 512 keys
+    (32, 8, 64, 100, 600, None),        # few tiles on few keys: the per-head kernel, keys split over its four waves
     (32, 8, 64, 512, 1536, None),       # the per-head kernel on a cached prefix, 128 workgroups' worth
     (32, 8, 64, 512, 7680, None),       # four runs of 2,048 keys
     (32, 8, 128, 40, 8000, None),       # head size 128, seven runs of 1,152 keys
