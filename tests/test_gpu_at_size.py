@@ -110,3 +110,26 @@ def test_decoding_behind_long_prompts_at_the_benchmarked_layer_sizes(dtype, size
     assert max(errors) < (2e-5 if dtype == "float32" else TOL_BF16)
     if dtype == "bfloat16":
         assert np.mean(errors) <= yardstick
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_short_portion_behind_a_long_prefix_at_the_benchmarked_layer_sizes(dtype, sized):
+    """The tail of a long prompt as a portion of its own, beside a short fresh prompt: seven query
+    tiles on 2,250 keys, which the bfloat16 attention deals out to four workgroups per tile and
+    merges (the fresh prompt's tiles leave all runs but the first empty)."""
+    name, model_dir, plain, yardstick = sized
+    rng = np.random.default_rng(10)
+    vocab = SIZES[name]["vocab_size"]
+    long, short = rng.integers(0, vocab, 2250).tolist(), rng.integers(0, vocab, 40).tolist()
+    places = [0, 31, 32, 100, 149]
+    truth = list(plain.logits_at(long, [2100 + p for p in places])) + [plain.logits_at(short, [39])[0]]
+    runner = ModelRunner(model_dir, dtype=dtype, device="cuda:0", num_blocks=160, max_seq_len=2304, max_num_seqs=4)
+    rp = TraceReplayer(runner)
+    assert rp.run_step({"step": 0, "entries": [{"id": "a", "tokens": long[:2100], "want": []}], "end": []}) is None
+    got = rp.run_step({"step": 1, "entries": [{"id": "a", "tokens": long[2100:], "want": places},
+                                              {"id": "b", "tokens": short, "want": [39]}], "end": ["a", "b"]})
+    errors = [float(np.abs(g - w).max() / np.abs(w).max()) for g, w in zip(got, truth)]
+    print(name, dtype, f"worst {max(errors):.2e} mean {np.mean(errors):.2e} (plain bf16 {yardstick:.2e})", flush=True)
+    assert max(errors) < (2e-5 if dtype == "float32" else TOL_BF16)
+    if dtype == "bfloat16":
+        assert np.mean(errors) <= yardstick
