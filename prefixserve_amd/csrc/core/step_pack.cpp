@@ -48,6 +48,8 @@ PackLayout plan_step(const std::vector<PackItem>& items, const std::vector<PackG
     lay.logit_rows += it.want.size;
     if (n == 1) {
       lay.decode_items += 1;
+      lay.decode_max_kv = std::max(lay.decode_max_kv, end);
+      lay.decode_sum_kv += end;
     } else {
       lay.prefill_tiles += ceil_div(n, lim.prefill_tile);
     }

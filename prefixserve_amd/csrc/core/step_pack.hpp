@@ -53,6 +53,8 @@ struct PackLayout {
   int64_t total = 0;
   int64_t tokens = 0, items = 0, logit_rows = 0, decode_items = 0, prefill_tiles = 0, pages = 0;
   int64_t max_kv_len = 0;
+  // over the items that bring one token: the longest context after the step and the sum of them
+  int64_t decode_max_kv = 0, decode_sum_kv = 0;
   // offsets into the buffer, in 32-bit words
   int64_t token_ids = 0, positions = 0, tok_item = 0, item_start = 0, item_pos0 = 0, item_end = 0, slots = 0;
   int64_t logit_rows_off = 0, dec_items = 0, pf_tiles = 0;

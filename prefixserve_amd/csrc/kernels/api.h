@@ -88,7 +88,7 @@ int psamd_attention_prefill(void* stream, const void* qkv, int q_stride, void* o
 int psamd_attention_decode(void* stream, const void* qkv, int q_stride, void* out, const void* kv, float* part_o,
                            float* part_ml, const int32_t* dec_items, int n_dec, const int32_t* item_start,
                            const int32_t* item_end, const int32_t* table_off, const int32_t* block_ids, int hq,
-                           int hkv, int head_dim, int nsplit, float scale, int window);
+                           int hkv, int head_dim, int nsplit, float scale, int window, int min_split_keys);
 
 // out[r] = argmax (temperature[r] <= 0) or the inverse-CDF draw with uniform[r] in [0, 1).
 int64_t psamd_sample_scratch_floats(int rows);

@@ -731,11 +731,30 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
     float* __restrict__ part_o, float* __restrict__ part_ml, const int32_t* __restrict__ dec_items,
     const int32_t* __restrict__ item_start,
     const int32_t* __restrict__ item_end, const int32_t* __restrict__ table_off,
-    const int32_t* __restrict__ block_ids, int hq, int hkv, int nsplit, float scale, int window) {
+    const int32_t* __restrict__ block_ids, int hq, int hkv, int nsplit, float scale, int window, int min_tiles,
+    int n_dec) {
   constexpr int D = 16 * NS;
   constexpr int KS = (D + 31) / 32;
   extern __shared__ float smem[];
-  const int di = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
+  // Workgroups are handed out in the order of blockIdx.x, round robin over the eight dies. The
+  // (request, split) pairs are laid out eight at a time, one per die, with the kv heads of a pair
+  // 8 apart, so on the same die (a die's address translation then sees an eighth of the
+  // requests' pages; with the heads of a pair on eight dies a batch of 64 was 4% slower). The
+  // pairs follow each other request by request, the splits of a request turned by its number:
+  // the splits of one request go to different dies, and so do the first splits (the only ones
+  // with keys where a request is short) of different requests. With the request as the fast
+  // index of a three-dimensional grid and a multiple of eight requests, all workgroups of a
+  // request ran on one die, and a request with a long context among short ones was read at an
+  // eighth of the memory bandwidth (31 requests of 1,024 keys and one of 60,000 at head size
+  // 128: 687 us whatever the number of splits). The grid is rounded up to whole groups of eight
+  // pairs; the workgroups of the pairs that do not exist leave at once.
+  // Grid: x = die slot + 8 * kv head, y = group of eight pairs.
+  const int kvh = blockIdx.x >> 3;
+  const int at = blockIdx.y * 8 + (blockIdx.x & 7);
+  const int di = at / nsplit;
+  if (di >= n_dec) return;
+  const int turned = at - di * nsplit + nsplit - (di < nsplit ? di : di % nsplit);     // in [1, 2 nsplit)
+  const int split = turned >= nsplit ? turned - nsplit : turned;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r = lane & 15, g4 = lane >> 4;
   const int item = dec_items[di];
@@ -745,9 +764,25 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
   const int32_t* table = block_ids + table_off[item];
   const int k_lo = window > 0 ? max(0, pos - window + 1) : 0;
   const int tile_lo = k_lo >> 5, tile_hi = pos >> 5;
-  const int tps = (tile_hi - tile_lo + nsplit) / nsplit;   // ceil(ntiles / nsplit)
+  // ceil(ntiles / nsplit), but no fewer than min_tiles: a short request beside a long one is
+  // not cut into as many runs as the long one needs, and leaves the last splits empty.
+  const int tps = max((tile_hi - tile_lo + nsplit) / nsplit, min_tiles);
   const int my_lo = tile_lo + split * tps;
   const int my_hi = min(my_lo + tps, tile_hi + 1);
+  if (my_lo >= my_hi) {
+    // No keys left for this split (only with nsplit > 1): an empty sum and an output of zeros,
+    // which the merge kernel multiplies by a weight of zero (what lay there before might be NaN).
+    for (int idx = threadIdx.x; idx < group * D; idx += blockDim.x) {
+      const int hh = idx / D, d = idx - hh * D;
+      const int64_t slot = (static_cast<int64_t>(di) * hq + kvh * group + hh) * nsplit + split;
+      part_o[slot * D + d] = 0.f;
+      if (d == 0) {
+        part_ml[slot * 2 + 0] = -INFINITY;
+        part_ml[slot * 2 + 1] = 0.f;
+      }
+    }
+    return;
+  }
 
   const int64_t page_elems = 2LL * hkv * kPage * D;
   const int64_t khead = static_cast<int64_t>(kvh) * kPage * D;
@@ -1072,12 +1107,13 @@ template <int NS, int CT>
 static int launch_decode(hipStream_t s, const void* qkv, int q_stride, const void* kv, void* out, float* part_o,
                          float* part_ml, const int32_t* dec_items, int n_dec, const int32_t* item_start, const int32_t* item_end,
                          const int32_t* table_off, const int32_t* block_ids, int hq, int hkv, int nsplit, float scale,
-                         int window) {
+                         int window, int min_tiles) {
   const int group = hq / hkv;
   const size_t smem = sizeof(float) * (8 * group + 4 * static_cast<size_t>(group) * 16 * NS);
-  attn_decode_mfma_kernel<NS, CT><<<dim3(n_dec, hkv, nsplit), dim3(256), smem, s>>>(
+  const int64_t groups_of_8 = ceil_div(static_cast<int64_t>(n_dec) * nsplit, 8);
+  attn_decode_mfma_kernel<NS, CT><<<dim3(8 * hkv, static_cast<unsigned>(groups_of_8)), dim3(256), smem, s>>>(
       static_cast<const bf16_t*>(qkv), q_stride, static_cast<const bf16_t*>(kv), static_cast<bf16_t*>(out), part_o,
-      part_ml, dec_items, item_start, item_end, table_off, block_ids, hq, hkv, nsplit, scale, window);
+      part_ml, dec_items, item_start, item_end, table_off, block_ids, hq, hkv, nsplit, scale, window, min_tiles, n_dec);
   return check_launch("psamd_attention_decode");
 }
 
@@ -1085,10 +1121,10 @@ template <int NS>
 static int dispatch_decode_ct(int ct, hipStream_t s, const void* qkv, int q_stride, const void* kv, void* out,
                               float* part_o, float* part_ml, const int32_t* dec_items, int n_dec, const int32_t* item_start,
                               const int32_t* item_end, const int32_t* table_off, const int32_t* block_ids, int hq,
-                              int hkv, int nsplit, float scale, int window) {
+                              int hkv, int nsplit, float scale, int window, int min_tiles) {
 #define PSAMD_DEC(CT_)                                                                                             \
   return launch_decode<NS, CT_>(s, qkv, q_stride, kv, out, part_o, part_ml, dec_items, n_dec, item_start, item_end, \
-                                table_off, block_ids, hq, hkv, nsplit, scale, window)
+                                table_off, block_ids, hq, hkv, nsplit, scale, window, min_tiles)
   switch (ct) {
     case 1: PSAMD_DEC(1);
     case 2: PSAMD_DEC(2);
@@ -1152,13 +1188,18 @@ int psamd_attention_prefill(void* stream, const void* qkv, int q_stride, void* o
 }
 
 // part_o needs n_dec * hq * nsplit * head_dim floats, part_ml n_dec * hq * nsplit * 2.
+// min_split_keys: a request's keys are cut into runs no shorter than this (a multiple of 32), so
+// that nsplit can follow the longest request of a step without cutting the short ones to pieces.
 int psamd_attention_decode(void* stream, const void* qkv, int q_stride, void* out, const void* kv, float* part_o,
                            float* part_ml, const int32_t* dec_items, int n_dec, const int32_t* item_start,
                            const int32_t* item_end, const int32_t* table_off, const int32_t* block_ids, int hq,
-                           int hkv, int head_dim, int nsplit, float scale, int window) {
+                           int hkv, int head_dim, int nsplit, float scale, int window, int min_split_keys) {
   PSAMD_REQUIRE(psamd_attention_mfma_supports(hq, hkv, head_dim), "shape not supported by the matrix-core kernels");
   PSAMD_REQUIRE(q_stride % 8 == 0, "query row stride must be a multiple of 8 elements");
   PSAMD_REQUIRE(nsplit >= 1 && nsplit <= 64, "nsplit must be in [1, 64]");
+  PSAMD_REQUIRE(min_split_keys >= 32 && min_split_keys % 32 == 0, "min_split_keys must be a positive multiple of 32");
+  const int min_tiles = min_split_keys / 32;
+  PSAMD_REQUIRE(static_cast<int64_t>(n_dec) * nsplit <= 8 * 65535, "too many (request, split) pairs for one launch");
   if (n_dec == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int group = hq / hkv;
@@ -1166,7 +1207,7 @@ int psamd_attention_decode(void* stream, const void* qkv, int q_stride, void* ou
   int rc;
 #define PSAMD_DEC_NS(NS_)                                                                                          \
   rc = dispatch_decode_ct<NS_>(ct, s, qkv, q_stride, kv, out, part_o, part_ml, dec_items, n_dec, item_start,    \
-                               item_end, table_off, block_ids, hq, hkv, nsplit, scale, window);                  \
+                               item_end, table_off, block_ids, hq, hkv, nsplit, scale, window, min_tiles);       \
   break
   switch (head_dim / 16) {
     case 1: PSAMD_DEC_NS(1);

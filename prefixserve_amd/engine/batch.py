@@ -22,6 +22,17 @@ from ..build import ensure_core
 PAGE = 16  # tokens per page; equals the cache core's BLOCK_SIZE
 
 
+def decode_is_skewed(count: int, longest: int, total: int) -> bool:
+    """Whether the single-token items of a step have one context far longer than the rest: more
+    than four times their mean and 4,096 tokens beyond that. The decode attention then cuts every
+    request's keys into runs of 1,024 or more, as many as the longest request needs, instead of
+    as many as fill the chip with requests of equal length; a long request among short ones is
+    otherwise read by a few workgroups while the rest of the chip waits (31 requests of 1,024 tokens
+    and one of 60,000: 429 -> 55 us a layer at head size 64). Steps of equal lengths pay 10 to 25 us
+    a layer for the extra runs, so it is decided step by step; a captured graph is keyed by it."""
+    return count > 1 and longest * count > 4 * total + 4096 * count
+
+
 class EngineError(RuntimeError):
     """The engine was given a batch it cannot run: a configuration or scheduler bug."""
 
@@ -63,6 +74,7 @@ class StepContext:
     num_decode: int            # items with exactly one token (served by the decode kernel)
     num_prefill_tiles: int
     max_kv_len: int
+    decode_skewed: bool        # one single-token item's context is far longer than the others'
     token_ids: torch.Tensor    # [T]
     positions: torch.Tensor    # [T] absolute
     tok_item: torch.Tensor     # [T] item of each token
@@ -120,7 +132,7 @@ class StepPacker:
                                       self.num_slots, self.prefill_tile, static_pages)
         except ValueError as e:
             raise EngineError(str(e)) from None
-        _, total, t_n, b, s_n, n_dec, n_tiles, p_total, max_kv_len, offs, group_offs = res
+        _, total, t_n, b, s_n, n_dec, n_tiles, p_total, max_kv_len, dec_max_kv, dec_sum_kv, offs, group_offs = res
         o_ids, o_pos, o_item, o_start, o_pos0, o_end, o_slots, o_rows, o_dec, o_tiles = offs
 
         if self.on_gpu:
@@ -144,6 +156,7 @@ class StepPacker:
         _, on_dev, host, groups = self._views
         return StepContext(
             num_tokens=t_n, num_items=b, num_logit_rows=s_n, num_decode=n_dec, num_prefill_tiles=n_tiles,
-            max_kv_len=max_kv_len, groups=groups, keys=[it.key for it in items],
+            max_kv_len=max_kv_len, decode_skewed=decode_is_skewed(n_dec, dec_max_kv, dec_sum_kv), groups=groups,
+            keys=[it.key for it in items],
             want_counts=[len(it.want) for it in items], host=host, **on_dev,
         )

@@ -33,10 +33,12 @@ if TYPE_CHECKING:
 
 def graphed_decode_step(runner: "ModelRunner", items: Sequence[StepItem], token_feed: Any = None) -> Any:
     wanted = sum(len(it.want) for it in items)
-    key = (len(items), wanted)
     static_pages = -(-runner.max_seq_len // PAGE)
     ops, ws, packer = runner.ops, runner.workspace, runner.packer
     ctx = packer.pack(items, static_pages=static_pages)
+    # The attention's grid follows from the batch size, from max_seq_len and from whether one
+    # context is far longer than the others: steps that differ in that are different graphs.
+    key = (len(items), wanted, ctx.decode_skewed)
     if token_feed is not None:
         ctx.token_ids.copy_(token_feed)    # in stream order after the packed integers, before the graph
     entry = runner._graphs.get(key)
@@ -44,8 +46,8 @@ def graphed_decode_step(runner: "ModelRunner", items: Sequence[StepItem], token_
         entry[0].replay()
         return entry[1]
 
-    previous = ops.fixed_kv_len
-    ops.fixed_kv_len = runner.max_seq_len
+    previous = ops.fixed_kv_len, ops.fixed_skew
+    ops.fixed_kv_len, ops.fixed_skew = runner.max_seq_len, ctx.decode_skewed
     try:
         # An eager run first: it sizes every workspace buffer (and is this step's result if
         # capture is not possible). Then capture the same sequence and replay it.
@@ -72,4 +74,4 @@ def graphed_decode_step(runner: "ModelRunner", items: Sequence[StepItem], token_
         graph.replay()         # idempotent: same inputs, same cache writes as the eager run
         return captured
     finally:
-        ops.fixed_kv_len = previous
+        ops.fixed_kv_len, ops.fixed_skew = previous

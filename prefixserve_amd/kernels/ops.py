@@ -59,7 +59,7 @@ _SIGNATURES = {
     "psamd_attention_prefill": [_vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _f32,
                                 _i32, _vp, _vp, _i32],
     "psamd_attention_decode": [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32,
-                               _i32, _f32, _i32],
+                               _i32, _f32, _i32, _i32],
     "psamd_sample": [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32],
 }
 
@@ -94,6 +94,7 @@ class HipOps:
         # Set while a step is run for, or under, graph capture: the key length that grids and
         # LDS tables are sized by instead of the step's own, and no product with a workspace.
         self.fixed_kv_len: int | None = None
+        self.fixed_skew = False      # with fixed_kv_len: whether the step's context lengths count as skewed
 
     # ---------------------------------------------------------------- helpers
 
@@ -359,6 +360,11 @@ class HipOps:
                 # merge kernel): 32 requests x 8 kv heads at head size 128: 48 -> 41 us.
                 pairs = ctx.num_decode * hkv
                 nsplit = 1 if pairs >= 256 else max(1, min(64, 512 // pairs, -(-kv_len // 128)))
+                min_run = 128
+                if (self.fixed_skew if self.fixed_kv_len else ctx.decode_skewed) and not win:
+                    # One context far longer than the others: runs of 1,024 keys, as many as the
+                    # longest needs; the short requests use one or two and leave the rest empty.
+                    nsplit, min_run = max(nsplit, min(64, 4096 // ctx.num_decode, -(-kv_len // 1024))), 1024
                 # (requests x splits) is at most 512 / hkv unless there are more requests than
                 # that: asked for at that size, the buffers do not grow from step to step.
                 parts = max(ctx.num_decode * nsplit, 512 // hkv)
@@ -368,7 +374,7 @@ class HipOps:
                     s, qkv.data_ptr(), stride, out.data_ptr(), kv.data_ptr(), part_o.data_ptr(), part_ml.data_ptr(),
                     ctx.dec_items.data_ptr(), ctx.num_decode, ctx.item_start.data_ptr(),
                     ctx.item_end.data_ptr(), g.table_off.data_ptr(), g.block_ids.data_ptr(), hq, hkv, d, nsplit, scale,
-                    win))
+                    win, min_run))
             return
         self._ok(self.lib.psamd_attention_generic(
             s, qkv.data_ptr(), stride, out.data_ptr(), kv.data_ptr(), _code(qkv.dtype), t, ctx.positions.data_ptr(),

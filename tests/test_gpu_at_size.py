@@ -105,7 +105,7 @@ def test_decoding_behind_long_prompts_at_the_benchmarked_layer_sizes(dtype, size
             want = truth[i][1 + k]
             errors.append(float(np.abs(got[i] - want).max() / np.abs(want).max()))
     if runner.use_graphs:
-        assert (3, 3) in runner._graphs
+        assert (3, 3, False) in runner._graphs
     print(name, dtype, f"worst {max(errors):.2e} mean {np.mean(errors):.2e} (plain bf16 {yardstick:.2e})", flush=True)
     assert max(errors) < (2e-5 if dtype == "float32" else TOL_BF16)
     if dtype == "bfloat16":

@@ -432,6 +432,39 @@ def test_decode_attention_of_many_requests(ops, hq, hkv, d, longest, window):
     assert rel(got, want) < 2e-2
 
 
+@pytest.mark.parametrize("hq,hkv,d,short,longest", [
+    (32, 8, 64, 31, 9000),         # many workgroups already: the long request alone gets more runs
+    (16, 8, 128, 7, 12500),        # few requests: runs of 1,024 keys instead of the usual short ones
+    (4, 1, 64, 15, 12000),         # one kv head
+    (6, 3, 96, 40, 11000),         # three kv heads, head size 96
+])
+def test_decode_attention_with_one_long_context_among_short_ones(ops, hq, hkv, d, short, longest):
+    """One request's context is far longer than the others': the step counts as skewed and every
+    request's keys are cut into runs of 1,024 or more, nine or more for the long request, one for
+    the short ones, whose other runs are empty. Slots nobody wrote hold NaN."""
+    rng = np.random.default_rng(longest)
+    old = rng.integers(0, 600, short).tolist()
+    old.insert(short // 2, longest)
+    new = [1] * len(old)
+    pages = sum(-(-(o + 1) // 16) for o in old) + 8
+    seen = {}
+    packed = StepPacker.pack
+
+    def spy(self, items, **kw):
+        ctx = packed(self, items, **kw)
+        seen["skewed"] = ctx.decode_skewed
+        return ctx
+
+    StepPacker.pack = spy
+    try:
+        got, want = paged_case(ops, torch.bfloat16, hq, hkv, d, new, old, seed=11, num_blocks=pages, poison=float("nan"))
+    finally:
+        StepPacker.pack = packed
+    assert seen["skewed"]
+    assert torch.isfinite(got.float()).all()
+    assert rel(got, want) < 2e-2
+
+
 @pytest.mark.parametrize("hq,hkv,d,new,old,window", [
     (32, 8, 64, [2048], [0], None),              # 512 workgroups, nothing cached: grouped, a kv head's tiles on one die
     (24, 8, 128, [2100], [0], None),             # three heads per kv head, an odd number of tiles, a last tile of 20

@@ -121,7 +121,7 @@ def test_graph_replay_equals_eager_decoding(model_dirs):
             if k % 7 == 3:                                           # eager work between replays
                 rp.run_step({"step": 100 + k, "entries": [{"id": "x", "tokens": list(range(5, 40)), "want": [34]}], "end": ["x"]})
         if graphs:
-            assert (3, 3) in runner._graphs
+            assert (3, 3, False) in runner._graphs
         return np.stack(rows)
 
     assert np.array_equal(decode(False, 128), decode(True, 128))
@@ -129,6 +129,50 @@ def test_graph_replay_equals_eager_decoding(model_dirs):
     assert np.array_equal(graph, decode(True, 256))
     apart = np.abs(eager - graph).max(-1) / np.abs(eager).max(-1)
     assert apart.max() < 2.0 ** -8, f"graph and single steps {apart.max():.2e} apart"
+
+
+def test_decoding_with_one_long_context_among_short_ones_through_graphs(tmp_path):
+    """Sixteen requests decode together, one behind 5,700 tokens, the others behind a few dozen:
+    the step counts as skewed, its graph is one of its own (keyed by that), and the attention
+    cuts the long request's keys into runs of 1,024 that the short ones leave empty. Logits of
+    every request against the plain model, and the same steps launched one by one."""
+    from configs import INIT_STD
+    from plain.llama_plain import PlainLlama
+    from prefixserve_amd.weights import write_random_model
+
+    cfg = dict(TINY["A"], max_position_embeddings=8192)
+    write_random_model(tmp_path, cfg, seed=21, std=INIT_STD)
+    plain = PlainLlama(tmp_path)
+    rng = np.random.default_rng(21)
+    lengths, new = [5700] + [20 + 3 * i for i in range(15)], 4
+    seqs = [rng.integers(0, cfg["vocab_size"], n + new).tolist() for n in lengths]
+    truth = [plain.logits_at(s, range(n - 1, n + new)) for s, n in zip(seqs, lengths)]
+    blocks = sum(-(-(n + new) // 16) for n in lengths) + 8
+
+    def decode(graphs):
+        runner = ModelRunner(tmp_path, dtype="bfloat16", device="cuda:0", num_blocks=blocks, max_seq_len=5760,
+                             max_num_seqs=16, use_graphs=graphs)
+        rp = TraceReplayer(runner)
+        rows = []
+        for at in range(0, 5700, 1900):
+            rp.run_step({"step": at, "entries": [{"id": "r0", "tokens": seqs[0][at:at + 1900], "want": []}], "end": []})
+        for i in range(1, 16):
+            rp.run_step({"step": i, "entries": [{"id": f"r{i}", "tokens": seqs[i][:lengths[i]], "want": []}], "end": []})
+        for k in range(new):
+            entries = [{"id": f"r{i}", "tokens": [seqs[i][lengths[i] + k]], "want": [0]} for i in range(16)]
+            rows.append(rp.run_step({"step": 100 + k, "entries": entries, "end": []}))
+        if graphs:
+            assert (16, 16, True) in runner._graphs
+        return np.stack(rows)                       # [new, 16, vocab]
+
+    graph = decode(True)
+    for i in range(16):
+        for k in range(new):
+            want = truth[i][1 + k]
+            err = float(np.abs(graph[k, i] - want).max() / np.abs(want).max())
+            assert err < TOL_BF16, f"request {i}, step {k}: {err:.2e}"
+    apart = np.abs(decode(False) - graph).max(-1) / np.abs(graph).max(-1)
+    assert apart.max() < 2.0 ** -7, f"graph and single steps {apart.max():.2e} apart"
 
 
 def test_graph_replay_with_library_products(model_dirs):
