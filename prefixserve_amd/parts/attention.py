@@ -84,8 +84,9 @@ class PagedAttention(Mixer):
 
     def activation_bytes(self, tokens: int, itemsize: int) -> int:
         # q/k/v, the attention output, the projected output (or its float32 partial sums).
-        # ... and what the attention kernels pass between the workgroups that share a query's keys.
-        split_rows = 32 * (512 // (self.num_kv_heads * -(-(self.num_heads // self.num_kv_heads) // 4)))
+        # ... and what the attention kernels pass between the workgroups that share a query's keys:
+        # the runs of a prompt portion's tiles, and up to 4,096 (request, run) pairs of single tokens.
+        split_rows = 32 * (512 // (self.num_kv_heads * -(-(self.num_heads // self.num_kv_heads) // 4))) + 4096
         return tokens * ((self.q_size + 2 * self.kv_size) + self.q_size) * itemsize + 8 * 64 * self.hidden_size * 4 \
             + tokens * self.hidden_size * itemsize + split_rows * self.num_heads * (self.head_dim + 2) * 4
 
