@@ -298,6 +298,97 @@ __global__ __launch_bounds__(64 * WV) void skinny_mfma_kernel(const bf16_t* __re
   }
 }
 
+// The output matrix over a large vocabulary for up to 8 tokens, as workgroups that stay: each
+// stages the tokens in LDS once (8 rows of K values; in the kernel above every workgroup reads
+// them again from L2 for its one or two row tiles, as many bytes as the rows themselves at two
+// tiles) and then takes groups of RT row tiles in turn, gridDim.x apart. Its eight waves split
+// K as above, a wave's k-steps of all RT tiles in flight together; the partial sums meet in LDS
+// and wave rt finishes tile rt. K must be a multiple of 32.
+template <int RT, int ROWS, typename TO>
+__global__ __launch_bounds__(512) void wide_stream_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                       TO* __restrict__ out, int M, int n_out, int K, int groups) {
+  constexpr int WV = 8, U = 8;
+  extern __shared__ __align__(16) unsigned char wide_smem[];
+  const int XS = K + 8;                                    // elements per token row in LDS (padded: rows on different banks)
+  bf16_t* xs = reinterpret_cast<bf16_t*>(wide_smem);
+  f32x4* red = reinterpret_cast<f32x4*>(wide_smem + static_cast<size_t>(ROWS) * XS * sizeof(bf16_t));   // [WV][RT][64]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  for (int p = threadIdx.x; p < ROWS * (K >> 3); p += blockDim.x) {      // ROWS rows x K / 8 pieces of 16 bytes
+    const int row = p / (K >> 3), c = p - row * (K >> 3);
+    bf16x8 v = zero8();
+    if (row < M) v = load8(x + static_cast<int64_t>(row) * K + 8 * c);
+    *reinterpret_cast<bf16x8*>(xs + row * XS + 8 * c) = v;
+  }
+  __syncthreads();
+  // Lanes 8..15 of a group repeat tokens 0..7: their columns of the result are not stored.
+  const bf16_t* xl = xs + (r % ROWS) * XS + 8 * g;
+  const int steps = K >> 5;
+  for (int grp = blockIdx.x; grp < groups; grp += gridDim.x) {
+    const int tile0 = grp * RT;
+    const bf16_t* wrow[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+      wrow[rt] = w + static_cast<int64_t>(min((tile0 + rt) * 16 + r, n_out - 1)) * K + 8 * g;
+    f32x4 acc[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) acc[rt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int base = wave; base < steps; base += WV * U) {
+      bf16x8 a[RT][U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int st = base + WV * u;
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) a[rt][u] = st < steps ? load8(wrow[rt] + (st << 5)) : zero8();
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int st = min(base + WV * u, steps - 1);      // past the end: the row tiles are zeros
+        const bf16x8 b = *reinterpret_cast<const bf16x8*>(xl + (st << 5));
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[rt][u], b, acc[rt], 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) red[(wave * RT + rt) * 64 + lane] = acc[rt];
+    __syncthreads();
+    if (wave < RT) {
+      const int rt = wave;
+      f32x4 sum = red[rt * 64 + lane];
+#pragma unroll
+      for (int w2 = 1; w2 < WV; ++w2) sum += red[(w2 * RT + rt) * 64 + lane];
+      if (r < M) {
+        TO* dst = out + static_cast<int64_t>(r) * n_out;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const int n = (tile0 + rt) * 16 + 4 * g + v;
+          if (n < n_out) dst[n] = from_float<TO>(sum[v]);
+        }
+      }
+    }
+    __syncthreads();      // the sums are read before the next group's are written
+  }
+}
+
+template <int RT, int ROWS>
+static int launch_wide_stream(hipStream_t s, const void* x, const void* w, void* out, int out_dtype, int M, int n_out,
+                              int K, int workgroups) {
+  const int groups = static_cast<int>(ceil_div(ceil_div(n_out, 16), RT));
+  const size_t smem = static_cast<size_t>(ROWS) * (K + 8) * sizeof(bf16_t) + sizeof(f32x4) * 8 * RT * 64;
+  const int rounds = static_cast<int>(ceil_div(groups, workgroups));
+  const dim3 grid(static_cast<unsigned>(ceil_div(groups, rounds))), block(512);
+  const bf16_t* xp = static_cast<const bf16_t*>(x);
+  const bf16_t* wp = static_cast<const bf16_t*>(w);
+  if (out_dtype == kBF16) {
+    if (smem > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(wide_stream_kernel<RT, ROWS, bf16_t>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem)) != hipSuccess) return -1;
+    wide_stream_kernel<RT, ROWS, bf16_t><<<grid, block, smem, s>>>(xp, wp, static_cast<bf16_t*>(out), M, n_out, K, groups);
+  } else {
+    if (smem > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(wide_stream_kernel<RT, ROWS, float>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem)) != hipSuccess) return -1;
+    wide_stream_kernel<RT, ROWS, float><<<grid, block, smem, s>>>(xp, wp, static_cast<float*>(out), M, n_out, K, groups);
+  }
+  return check_launch("psamd_linear_skinny");
+}
+
 template <int MT, int RT, int WV, bool SWIGLU, bool SPLIT>
 static int launch_skinny2(hipStream_t s, const void* x, const void* w, void* out, int out_dtype, int M, int n_out,
                           int K, int ksplit) {
@@ -339,6 +430,23 @@ static int launch_skinny1(hipStream_t s, const void* x, const void* w, void* out
     // Against four waves with a row tile each over all of K, at 128,256 columns and K = 2,048:
     // 93 -> 84 us at 1 token, 95 -> 87 at 2, 101 -> 96 at 4, 113 -> 111 at 8; the same order at
     // K = 4,096 (193 -> 172 us at 1 token).
+    // From 2 tokens on the workgroups that stay and keep the tokens in LDS are faster (128,256
+    // columns, K = 2,048: 93 -> 92 us at 2 tokens, 102 -> 94 at 4, 112 -> 98 at 8, 125 -> 108
+    // at 16; K = 4,096: 202 -> 175 at 4, 221 -> 181 at 8): two row tiles per group and two
+    // workgroups per compute unit while the tokens are 32 KB, else one and four.
+    if (M >= (K <= 2048 ? 4 : 2) && M <= 16 && ksplit == 1 && ceil_div(n_out, 16) >= 2048 && K % 32 == 0) {
+      const int rows = M <= 8 ? 8 : 16;
+      const bool small = static_cast<int64_t>(rows) * K <= 8 * 2048;
+      const size_t smem = static_cast<size_t>(rows) * (K + 8) * sizeof(bf16_t) + sizeof(f32x4) * 8 * (small ? 2 : 1) * 64;
+      if (smem <= 160 * 1024) {
+        if (rows == 8) {
+          if (small) return launch_wide_stream<2, 8>(s, x, w, out, out_dtype, M, n_out, K, 512);
+          return launch_wide_stream<1, 8>(s, x, w, out, out_dtype, M, n_out, K, 1024);
+        }
+        if (small) return launch_wide_stream<2, 16>(s, x, w, out, out_dtype, M, n_out, K, 512);
+        return launch_wide_stream<1, 16>(s, x, w, out, out_dtype, M, n_out, K, 1024);
+      }
+    }
     if (M <= 8 && ksplit == 1 && ceil_div(n_out, 16) >= 2048) {
       const bf16_t* xp = static_cast<const bf16_t*>(x);
       const bf16_t* wp = static_cast<const bf16_t*>(w);

@@ -222,13 +222,16 @@ def test_linear_bf16_small_m(ops, m, n, k, out_dtype):
 
 
 @pytest.mark.parametrize("m", [1, 3, 5, 8, 9, 16, 31, 48, 64])
-@pytest.mark.parametrize("n,k", [(65536 + 40, 72), (32768 + 24, 2048)])
+@pytest.mark.parametrize("n,k", [(65536 + 40, 72), (32768 + 24, 2048), (32768 + 200, 96), (32768 + 16, 1024), (32768 + 32, 4096)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 def test_linear_bf16_very_many_columns(ops, m, n, k, out_dtype):
     """The forms the output matrix takes: up to 8 tokens one or two row tiles per workgroup of
-    eight waves that split K, from 9 tokens on more row tiles per wave; row counts that are no
-    multiple of the largest group of tiles (an odd number of tiles among them), a K with a
-    partial last step and a K that gives every wave eight steps."""
+    eight waves that split K, from 9 tokens on more row tiles per wave; where K is a multiple of
+    32, from 2 or 4 to 16 tokens, workgroups that keep the tokens in LDS (8 or 16 rows, one or
+    two row tiles per group, a K so small that some waves have no step, a K of two rounds of
+    steps per wave). Row counts that are no multiple of the largest group of tiles (an odd
+    number of tiles among them), a K with a partial last step and a K that gives every wave
+    eight steps."""
     x, w = rnd(m, k, dtype=torch.bfloat16, seed=1), rnd(n, k, dtype=torch.bfloat16, seed=2, scale=0.1)
     out = torch.full((m + 1, n), 7.0, dtype=out_dtype, device=DEV)
     ops.linear(x, w, out[:m])
