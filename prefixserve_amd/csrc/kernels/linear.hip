@@ -11,6 +11,7 @@
 //   epilogue: SwiGLU over a fused [gate; up] matrix, or float32 output for logits.
 
 #include <algorithm>
+#include <string>
 
 #include "api.h"
 #include "common.h"
@@ -298,67 +299,97 @@ __global__ __launch_bounds__(64 * WV) void skinny_mfma_kernel(const bf16_t* __re
   }
 }
 
-// The output matrix over a large vocabulary for up to 8 tokens, as workgroups that stay: each
-// stages the tokens in LDS once (8 rows of K values; in the kernel above every workgroup reads
-// them again from L2 for its one or two row tiles, as many bytes as the rows themselves at two
-// tiles) and then takes groups of RT row tiles in turn, gridDim.x apart. Its eight waves split
-// K as above, a wave's k-steps of all RT tiles in flight together; the partial sums meet in LDS
-// and wave rt finishes tile rt. K must be a multiple of 32.
-template <int RT, int ROWS, typename TO>
-__global__ __launch_bounds__(512) void wide_stream_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-                                                       TO* __restrict__ out, int M, int n_out, int K, int groups) {
-  constexpr int WV = 8, U = 8;
-  extern __shared__ __align__(16) unsigned char wide_smem[];
-  const int XS = K + 8;                                    // elements per token row in LDS (padded: rows on different banks)
-  bf16_t* xs = reinterpret_cast<bf16_t*>(wide_smem);
-  f32x4* red = reinterpret_cast<f32x4*>(wide_smem + static_cast<size_t>(ROWS) * XS * sizeof(bf16_t));   // [WV][RT][64]
+// Up to 16 tokens as workgroups that stay: each stages its tokens in LDS once (ROWS = 8 or 16
+// rows of its slice of K; in the kernel above every workgroup reads them again from L2 for its
+// one or two row tiles, as many bytes as the rows themselves at two tiles) and then takes groups
+// of RT row tiles in turn, gridDim.x apart. Its eight waves split the slice as above, a wave's
+// k-steps of all RT tiles in flight together; the partial sums meet in LDS and wave rt finishes
+// tile rt. gridDim.y slices of K give partial sums out[blockIdx.y][M][n_out], as above. SWIGLU:
+// w is [gate; up] and a group is RT pairs of tiles. K must be a multiple of 32.
+template <int RT, int ROWS, bool SWIGLU, typename TO>
+__global__ __launch_bounds__(512) void stream_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                  TO* __restrict__ out, int M, int n_out, int K, int groups) {
+  constexpr int WV = 8, U = 8, NACC = SWIGLU ? 2 : 1;
+  extern __shared__ __align__(16) unsigned char stream_smem[];
+  const int steps_all = K >> 5;
+  const int per_slice = (steps_all + gridDim.y - 1) / gridDim.y;
+  const int s_begin = blockIdx.y * per_slice;
+  const int steps = max(0, min(per_slice, steps_all - s_begin));   // k-steps of this workgroup's slice (none: it writes zeros)
+  const int XS = per_slice * 32 + 8;                          // elements per token row in LDS (padded: rows on different banks)
+  bf16_t* xs = reinterpret_cast<bf16_t*>(stream_smem);
+  f32x4* red = reinterpret_cast<f32x4*>(stream_smem + static_cast<size_t>(ROWS) * XS * sizeof(bf16_t));   // [WV][RT][NACC][64]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
-  for (int p = threadIdx.x; p < ROWS * (K >> 3); p += blockDim.x) {      // ROWS rows x K / 8 pieces of 16 bytes
-    const int row = p / (K >> 3), c = p - row * (K >> 3);
-    bf16x8 v = zero8();
-    if (row < M) v = load8(x + static_cast<int64_t>(row) * K + 8 * c);
-    *reinterpret_cast<bf16x8*>(xs + row * XS + 8 * c) = v;
+  {
+    const int pieces = steps * 4;                             // 16-byte pieces of a row's slice
+    const bf16_t* x0 = x + (static_cast<int64_t>(s_begin) << 5);
+    for (int p = threadIdx.x; p < ROWS * pieces; p += blockDim.x) {
+      const int row = p / pieces, c = p - row * pieces;
+      bf16x8 v = zero8();
+      if (row < M) v = load8(x0 + static_cast<int64_t>(row) * K + 8 * c);
+      *reinterpret_cast<bf16x8*>(xs + row * XS + 8 * c) = v;
+    }
   }
   __syncthreads();
-  // Lanes 8..15 of a group repeat tokens 0..7: their columns of the result are not stored.
+  // With ROWS = 8, lanes 8..15 of a group repeat tokens 0..7: their columns of the result are not stored.
   const bf16_t* xl = xs + (r % ROWS) * XS + 8 * g;
-  const int steps = K >> 5;
+  const bf16_t* w0 = w + (static_cast<int64_t>(s_begin) << 5) + 8 * g;
   for (int grp = blockIdx.x; grp < groups; grp += gridDim.x) {
     const int tile0 = grp * RT;
     const bf16_t* wrow[RT];
+    const bf16_t* wrow_up[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      const int row = min((tile0 + rt) * 16 + r, n_out - 1);
+      wrow[rt] = w0 + static_cast<int64_t>(row) * K;
+      wrow_up[rt] = SWIGLU ? w0 + static_cast<int64_t>(n_out + row) * K : nullptr;
+    }
+    f32x4 acc[RT][NACC];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt)
-      wrow[rt] = w + static_cast<int64_t>(min((tile0 + rt) * 16 + r, n_out - 1)) * K + 8 * g;
-    f32x4 acc[RT];
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt) acc[rt] = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int i = 0; i < NACC; ++i) acc[rt][i] = f32x4{0.f, 0.f, 0.f, 0.f};
     for (int base = wave; base < steps; base += WV * U) {
-      bf16x8 a[RT][U];
+      bf16x8 a[RT][U], a_up[RT][U];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int st = base + WV * u;
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt) a[rt][u] = st < steps ? load8(wrow[rt] + (st << 5)) : zero8();
+        for (int rt = 0; rt < RT; ++rt) {
+          a[rt][u] = st < steps ? load8(wrow[rt] + (st << 5)) : zero8();
+          if (SWIGLU) a_up[rt][u] = st < steps ? load8(wrow_up[rt] + (st << 5)) : zero8();
+        }
       }
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int st = min(base + WV * u, steps - 1);      // past the end: the row tiles are zeros
         const bf16x8 b = *reinterpret_cast<const bf16x8*>(xl + (st << 5));
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt) acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[rt][u], b, acc[rt], 0, 0, 0);
+        for (int rt = 0; rt < RT; ++rt) {
+          acc[rt][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[rt][u], b, acc[rt][0], 0, 0, 0);
+          if (SWIGLU) acc[rt][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_up[rt][u], b, acc[rt][1], 0, 0, 0);
+        }
       }
     }
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt) red[(wave * RT + rt) * 64 + lane] = acc[rt];
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int i = 0; i < NACC; ++i) red[((wave * RT + rt) * NACC + i) * 64 + lane] = acc[rt][i];
     __syncthreads();
     if (wave < RT) {
       const int rt = wave;
-      f32x4 sum = red[rt * 64 + lane];
+      f32x4 sum = red[(rt * NACC) * 64 + lane];
 #pragma unroll
-      for (int w2 = 1; w2 < WV; ++w2) sum += red[(w2 * RT + rt) * 64 + lane];
+      for (int w2 = 1; w2 < WV; ++w2) sum += red[((w2 * RT + rt) * NACC) * 64 + lane];
+      if (SWIGLU) {
+        f32x4 up = red[(rt * NACC + 1) * 64 + lane];
+#pragma unroll
+        for (int w2 = 1; w2 < WV; ++w2) up += red[((w2 * RT + rt) * NACC + 1) * 64 + lane];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) sum[v] = silu_f(sum[v]) * up[v];
+      }
       if (r < M) {
-        TO* dst = out + static_cast<int64_t>(r) * n_out;
+        TO* dst = out + (static_cast<int64_t>(blockIdx.y) * M + r) * n_out;
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
           const int n = (tile0 + rt) * 16 + 4 * g + v;
@@ -370,23 +401,33 @@ __global__ __launch_bounds__(512) void wide_stream_kernel(const bf16_t* __restri
   }
 }
 
-template <int RT, int ROWS>
-static int launch_wide_stream(hipStream_t s, const void* x, const void* w, void* out, int out_dtype, int M, int n_out,
-                              int K, int workgroups) {
+// Bytes of LDS stream_kernel needs.
+static size_t stream_smem_bytes(int rt, int rows, bool swiglu, int K, int ksplit) {
+  const int per_slice = static_cast<int>(ceil_div(K >> 5, ksplit));
+  return static_cast<size_t>(rows) * (per_slice * 32 + 8) * sizeof(bf16_t) + sizeof(f32x4) * 8 * rt * (swiglu ? 2 : 1) * 64;
+}
+
+// workgroups: how many may stay per K-slice; the groups are dealt out evenly over them.
+template <int RT, int ROWS, bool SWIGLU>
+static int launch_stream(hipStream_t s, const void* x, const void* w, void* out, int out_dtype, int M, int n_out, int K,
+                         int ksplit, int workgroups) {
   const int groups = static_cast<int>(ceil_div(ceil_div(n_out, 16), RT));
-  const size_t smem = static_cast<size_t>(ROWS) * (K + 8) * sizeof(bf16_t) + sizeof(f32x4) * 8 * RT * 64;
+  const size_t smem = stream_smem_bytes(RT, ROWS, SWIGLU, K, ksplit);
   const int rounds = static_cast<int>(ceil_div(groups, workgroups));
-  const dim3 grid(static_cast<unsigned>(ceil_div(groups, rounds))), block(512);
+  const dim3 grid(static_cast<unsigned>(ceil_div(groups, rounds)), static_cast<unsigned>(ksplit)), block(512);
   const bf16_t* xp = static_cast<const bf16_t*>(x);
   const bf16_t* wp = static_cast<const bf16_t*>(w);
-  if (out_dtype == kBF16) {
-    if (smem > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(wide_stream_kernel<RT, ROWS, bf16_t>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem)) != hipSuccess) return -1;
-    wide_stream_kernel<RT, ROWS, bf16_t><<<grid, block, smem, s>>>(xp, wp, static_cast<bf16_t*>(out), M, n_out, K, groups);
-  } else {
-    if (smem > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(wide_stream_kernel<RT, ROWS, float>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem)) != hipSuccess) return -1;
-    wide_stream_kernel<RT, ROWS, float><<<grid, block, smem, s>>>(xp, wp, static_cast<float*>(out), M, n_out, K, groups);
-  }
-  return check_launch("psamd_linear_skinny");
+  auto run = [&](auto kernel, auto* dst) {
+    if (smem > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                static_cast<int>(smem)) != hipSuccess) {
+      set_error("psamd_linear_skinny: " + std::to_string(smem) + " bytes of LDS were refused");
+      return -1;
+    }
+    kernel<<<grid, block, smem, s>>>(xp, wp, dst, M, n_out, K, groups);
+    return check_launch("psamd_linear_skinny");
+  };
+  if (SWIGLU || out_dtype == kBF16) return run(stream_kernel<RT, ROWS, SWIGLU, bf16_t>, static_cast<bf16_t*>(out));
+  return run(stream_kernel<RT, ROWS, false, float>, static_cast<float*>(out));
 }
 
 template <int MT, int RT, int WV, bool SWIGLU, bool SPLIT>
@@ -437,14 +478,13 @@ static int launch_skinny1(hipStream_t s, const void* x, const void* w, void* out
     if (M >= (K <= 2048 ? 4 : 2) && M <= 16 && ksplit == 1 && ceil_div(n_out, 16) >= 2048 && K % 32 == 0) {
       const int rows = M <= 8 ? 8 : 16;
       const bool small = static_cast<int64_t>(rows) * K <= 8 * 2048;
-      const size_t smem = static_cast<size_t>(rows) * (K + 8) * sizeof(bf16_t) + sizeof(f32x4) * 8 * (small ? 2 : 1) * 64;
-      if (smem <= 160 * 1024) {
+      if (stream_smem_bytes(small ? 2 : 1, rows, false, K, 1) <= 160 * 1024) {
         if (rows == 8) {
-          if (small) return launch_wide_stream<2, 8>(s, x, w, out, out_dtype, M, n_out, K, 512);
-          return launch_wide_stream<1, 8>(s, x, w, out, out_dtype, M, n_out, K, 1024);
+          if (small) return launch_stream<2, 8, false>(s, x, w, out, out_dtype, M, n_out, K, 1, 512);
+          return launch_stream<1, 8, false>(s, x, w, out, out_dtype, M, n_out, K, 1, 1024);
         }
-        if (small) return launch_wide_stream<2, 16>(s, x, w, out, out_dtype, M, n_out, K, 512);
-        return launch_wide_stream<1, 16>(s, x, w, out, out_dtype, M, n_out, K, 1024);
+        if (small) return launch_stream<2, 16, false>(s, x, w, out, out_dtype, M, n_out, K, 1, 512);
+        return launch_stream<1, 16, false>(s, x, w, out, out_dtype, M, n_out, K, 1, 1024);
       }
     }
     if (M <= 8 && ksplit == 1 && ceil_div(n_out, 16) >= 2048) {
@@ -496,6 +536,29 @@ static int launch_skinny1(hipStream_t s, const void* x, const void* w, void* out
         skinny_mfma_kernel<1, 2, 8, true, true, bf16_t, 1><<<grid, block, 0, s>>>(
             static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), M, n_out, K);
         return check_launch("psamd_linear_skinny");
+      }
+    }
+  }
+  if constexpr (MT == 1) {
+    // Workgroups that stay (stream_kernel) pay where each has two or more groups of tiles to go
+    // through with the tokens it staged, us per product at 8 / 16 tokens:
+    //  * products whose K is split over workgroups (o, down), 512 workgroups in all: down of the
+    //    1B shape (2,048 x 8,192) 9.6 -> 9.0 / 12.1 -> 10.3, of the 3B shape 14.6 -> 11.9 /
+    //    17.0 -> 13.9, of the 8B shape (4,096 x 14,336) 30.5 -> 24.5 / 36.4 -> 26.8; o of the 8B
+    //    shape 9.5 -> 9.0 / 11.7 -> 10.1. With one group each (o of the smaller shapes) they lose.
+    //  * gate/up with K from 4,096 on, 256 workgroups: 8B shape 54.8 -> 51.8 at 8 tokens; at
+    //    K = 2,048 or 3,072 the workgroups that come and go are faster (17.7 vs 19.7).
+    const int64_t groups = ceil_div(n_out, 16);
+    if (M >= 4 && K % 32 == 0) {
+      if constexpr (!SWIGLU) {
+        const int wgs = ksplit > 1 ? 512 / ksplit : 0;
+        if (wgs > 0 && groups >= 2 * wgs && stream_smem_bytes(1, 16, false, K, ksplit) <= 160 * 1024) {
+          if (M <= 8) return launch_stream<1, 8, false>(s, x, w, out, out_dtype, M, n_out, K, ksplit, wgs);
+          return launch_stream<1, 16, false>(s, x, w, out, out_dtype, M, n_out, K, ksplit, wgs);
+        }
+      } else {
+        if (M <= 8 && ksplit == 1 && K >= 4096 && groups >= 768 && stream_smem_bytes(1, 8, true, K, 1) <= 160 * 1024)
+          return launch_stream<1, 8, true>(s, x, w, out, out_dtype, M, n_out, K, 1, 256);
       }
     }
   }

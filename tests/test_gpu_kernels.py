@@ -255,6 +255,32 @@ def test_linear_to_residual_splits_k(ops, m, n, k):
     assert small.dim() == 2 and small.dtype == torch.bfloat16                      # too little K to split
 
 
+@pytest.mark.parametrize("m", [3, 4, 5, 8, 9, 13, 16, 17])
+@pytest.mark.parametrize("n,k", [(2048, 8192), (2064, 4128), (3080, 8192), (4096, 4096), (1024 + 8, 9024)])
+def test_linear_to_residual_by_workgroups_that_stay(ops, m, n, k):
+    """From 4 to 16 tokens, a K-split product with two or more groups of row tiles per workgroup
+    goes to workgroups that keep their slice of the tokens in LDS (8 or 16 rows) and walk through
+    their groups: K-slices of unequal length, a row count that is no multiple of 16, and token
+    counts on either side of that form's range."""
+    x, w = rnd(m, k, dtype=torch.bfloat16, seed=3), rnd(n, k, dtype=torch.bfloat16, seed=4, scale=0.05)
+    out = ops.linear_to_residual(x, w, "test.delta3")
+    assert out.dim() == 3 and out.dtype == torch.float32
+    assert torch.isfinite(out).all()
+    assert rel(out.sum(0), x.double() @ w.double().T) < 1e-5
+
+
+@pytest.mark.parametrize("m", [3, 4, 7, 8, 9])
+@pytest.mark.parametrize("inter,k", [(12288 + 40, 4096), (12288, 4128)])
+def test_linear_swiglu_by_workgroups_that_stay(ops, m, inter, k):
+    """Gate/up with K from 4,096 on and 768 or more pairs of tiles, 4 to 8 tokens."""
+    x, w = rnd(m, k, dtype=torch.bfloat16, seed=1), rnd(2 * inter, k, dtype=torch.bfloat16, seed=2, scale=0.03)
+    out = torch.full((m + 1, inter), 7.0, dtype=torch.bfloat16, device=DEV)
+    ops.linear_swiglu(x, w, out[:m])
+    gu = x.double() @ w.double().T
+    want = torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:]
+    assert rel(out[:m], want) < 1e-2 and torch.all(out[m] == 7.0)
+
+
 @pytest.mark.parametrize("m,n,k", [(65, 300, 96), (200, 64, 2048), (3, 50, 70)])
 def test_linear_bf16_other_paths(ops, m, n, k):
     x, w = rnd(m, k, dtype=torch.bfloat16, seed=1), rnd(n, k, dtype=torch.bfloat16, seed=2, scale=0.1)
