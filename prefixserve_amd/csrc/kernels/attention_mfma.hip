@@ -1051,6 +1051,9 @@ static int prefill_nsplit(int n_tiles, int max_kv_len, int hq, int hkv, int head
   const int at_once = head_dim <= 64 ? 512 : 256;
   if (2 * workgroups > at_once) return 1;
   if (grouped_smem(head_dim, 1, 1, static_cast<int>(ceil_div(max_kv_len, kPage))) > 160 * 1024) return 1;
+  // 65 to 128 workgroups on 2,048 to 4,095 keys: two runs (512 tokens on 2,560 cached at head size
+  // 64 / 128: 43 -> 36 / 70 -> 54 us; on 1,536 cached 30 -> 28 / 44 -> 41).
+  if (workgroups > 64 && workgroups <= 128 && max_kv_len >= 2048 && max_kv_len < 4096) return 2;
   const int nsplit = static_cast<int>(std::min<int64_t>({at_once / workgroups, max_kv_len / kMinSplitKeys, kMaxPrefillSplit}));
   const bool per_head_else = workgroups <= (head_dim <= 64 ? 128 : 80);
   if (per_head_else) {

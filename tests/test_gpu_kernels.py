@@ -500,7 +500,8 @@ def test_decode_attention_with_one_long_context_among_short_ones(ops, hq, hkv, d
     (16, 8, 128, [1100], [0], None),             # two heads per kv head at head size 128: grouped, half its waves spare
     (16, 8, 128, [500], [600], None),            # the same with few workgroups: the per-head kernel
     (16, 4, 64, [2048, 2100], [0, 0], None),     # two prompts from position 0 in one step, 4 workgroups per tile
-    (32, 8, 64, [512], [1536], None),            # 128 workgroups on a prefix: the per-head kernel at this head size
+    (32, 8, 64, [512], [1536], None),            # 128 workgroups on 2,048 keys: grouped, two runs
+    (32, 8, 64, [512], [1000], None),            # 128 workgroups on fewer keys: the per-head kernel at this head size
     (32, 8, 64, [512], [7680], None),            # a portion of a long prompt: each tile's keys in four runs
     (32, 8, 128, [40], [16000], None),           # a short tail behind a long context: sixteen workgroups, fifteen runs each
     (24, 8, 128, [20, 300], [9000, 100], None),  # runs that a short request leaves empty, beside a long one; a spare wave
@@ -609,7 +610,8 @@ def test_attention_finds_one_far_key_among_hundreds(ops, act):
 @pytest.mark.parametrize("hq,hkv,d,new,old,window", [
     (32, 8, 64, 100, 1948, None),       # few tiles: grouped, four runs of 512 keys
     (32, 8, 64, 100, 600, None),        # few tiles on few keys: the per-head kernel, keys split over its four waves
-    (32, 8, 64, 512, 1536, None),       # the per-head kernel on a cached prefix, 128 workgroups' worth
+    (32, 8, 64, 512, 1536, None),       # grouped on a cached prefix, two runs of 1,024 keys
+    (32, 8, 64, 512, 1000, None),       # the per-head kernel on a cached prefix, 128 workgroups' worth
     (32, 8, 64, 512, 7680, None),       # four runs of 2,048 keys
     (32, 8, 128, 40, 8000, None),       # head size 128, seven runs of 1,152 keys
     (16, 4, 64, 64, 5000, 1500),        # runs inside a window
