@@ -34,8 +34,6 @@ def _add_engine_options(p: argparse.ArgumentParser) -> None:
                    help="decode steps a batch of decoding requests runs before the host looks at the tokens")
     p.add_argument("--warm-up", action="store_true",
                    help="size buffers and capture the decode graphs before the first request (not timed)")
-    p.add_argument("--tune-products", action="store_true",
-                   help="with --warm-up: let the product library time its algorithms for a full portion and keep the fastest")
 
 
 def _generate(args: argparse.Namespace) -> int:
@@ -47,7 +45,7 @@ def _generate(args: argparse.Namespace) -> int:
     cfg = EngineConfig(model_path=Path(args.model), dtype=args.dtype, max_num_seqs=args.max_running_requests,
                        max_prefill_tokens=args.chunked_prefill_size, max_seq_len=args.max_seq_len,
                        num_blocks=args.num_blocks, use_graphs=not args.no_graphs, sample_seed=args.sample_seed,
-                       decode_steps=args.decode_steps, tune_products=args.tune_products)
+                       decode_steps=args.decode_steps)
     engine = Engine(cfg)
     if args.warm_up:
         engine.warm_up()

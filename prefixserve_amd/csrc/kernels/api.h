@@ -45,14 +45,6 @@ int psamd_linear(void* stream, const void* x, int x_dtype, const void* w, int w_
 int psamd_gemm_lt_available();
 int psamd_gemm_lt(void* stream, const void* x, const void* w, void* out, int out_dtype, int64_t M, int N, int K,
                   int use_workspace);
-// Times every algorithm the library has for the shape on the given buffers (the n_ws matrices of
-// that shape in turn, so that each call reads its matrix from memory) and keeps the fastest
-// for it (and for row counts within a quarter of it) if it beats the heuristic's choice by 3%;
-// out and ref_out receive the product by the kept and by the heuristic's algorithm. For warm-up:
-// takes a second or two and waits for the stream. 2: library or its extension interface missing.
-int psamd_gemm_lt_tune(void* stream, const void* x, const void* const* ws, int n_ws, void* out, void* ref_out, int out_dtype,
-                       int64_t M, int N, int K, float* us_before, float* us_after);
-int psamd_gemm_lt_untune(int out_dtype, int64_t M, int N, int K);
 
 
 // bfloat16 product for M <= 64 on the matrix cores. epilogue 1: w = [gate; up], out = silu(gate) * up.
@@ -79,11 +71,20 @@ int psamd_attention_mfma_supports(int hq, int hkv, int head_dim);
 // part_o [32 * n_tiles * hq * nsplit * head_dim] and part_ml [32 * n_tiles * hq * nsplit * 2] carry
 // to a merge kernel.
 int psamd_attention_prefill_nsplit(int n_tiles, int max_kv_len, int hq, int hkv, int head_dim);
+// The most rows (32 * n_tiles * nsplit) of part_o / part_ml any step of this shape needs.
+int psamd_attention_prefill_part_rows(int hq, int hkv, int head_dim);
 int psamd_attention_prefill(void* stream, const void* qkv, int q_stride, void* out, const void* kv,
                             const int32_t* pf_tiles, int n_tiles, int max_kv_len,
                             const int32_t* item_start, const int32_t* item_pos0,
                             const int32_t* table_off, const int32_t* block_ids, int hq, int hkv, int head_dim,
                             float scale, int window, float* part_o, float* part_ml, int nsplit);
+
+// The plan for a decode step's keys: whether its context lengths count as skewed (one far longer
+// than the rest), into how many runs of at least how many keys each request's keys are cut, and
+// the most (requests x runs) any plan gives (part_o: that many x hq x head_dim floats).
+int psamd_attention_decode_skewed(int n_dec, int longest, int64_t total);
+int psamd_attention_decode_plan(int n_dec, int kv_len, int skewed, int hkv, int window, int* nsplit, int* min_run);
+int psamd_attention_decode_max_parts(int max_requests);
 
 int psamd_attention_decode(void* stream, const void* qkv, int q_stride, void* out, const void* kv, float* part_o,
                            float* part_ml, const int32_t* dec_items, int n_dec, const int32_t* item_start,
@@ -102,7 +103,9 @@ int psamd_sample(void* stream, const float* logits, const float* temperature, co
 // error. The call allocates nothing and calls no library routine that does; the caller passes
 // inputs and outputs as for psamd_sample, with the stream's device current. All calls on one GPU
 // share the array: two calls that overlap there (different streams, or two threads) race, and
-// the caller has to order them. Same kernels and the same result as psamd_sample.
+// the caller has to order them. Same kernels and the same result as psamd_sample. The first
+// call on a device asks the runtime for the array's address there (hipGetSymbolAddress, under
+// a mutex): make it once at set-up, outside any graph capture; later calls only launch.
 int psamd_sample_static_max_rows(void);
 int psamd_sample_static(void* stream, const float* logits, const float* temperature, const float* uniform,
                         int32_t* out, int rows, int vocab);

@@ -1159,6 +1159,18 @@ int psamd_attention_prefill_nsplit(int n_tiles, int max_kv_len, int hq, int hkv,
   return prefill_nsplit(n_tiles, max_kv_len, hq, hkv, head_dim);
 }
 
+// Rows of part_o / part_ml (32 * n_tiles * nsplit) that no step of this shape exceeds while
+// nsplit > 1: the runs are dealt out so that the workgroups fill the chip once, which bounds
+// (tiles x runs) whatever the step. A caller that keeps the buffers at this size never grows them.
+int psamd_attention_prefill_part_rows(int hq, int hkv, int head_dim) {
+  if (!psamd_attention_mfma_supports(hq, hkv, head_dim)) return 0;
+  const int group = hq / hkv;
+  // grouped kernel: tiles * runs * hkv * ceil(group / 4) <= 512 (256 above head size 64; two runs
+  // for up to 128 workgroups stay below it too); per-head kernel: tiles * runs * hq <= 256.
+  const int tiles_times_runs = group <= 2 ? std::max(1, 256 / hq) : std::max(1, 512 / (hkv * ((group + 3) / 4)));
+  return 32 * tiles_times_runs;
+}
+
 // max_kv_len: the longest request of the step after it (sizes the block table staged in LDS).
 // nsplit: 1, or what psamd_attention_prefill_nsplit gave for these sizes (or less); part_o then
 // has room for 32 * n_tiles * hq * nsplit * head_dim floats and part_ml for 32 * n_tiles * hq * nsplit * 2.
@@ -1189,6 +1201,40 @@ int psamd_attention_prefill(void* stream, const void* qkv, int q_stride, void* o
   }
 #undef PSAMD_PF
 }
+
+// Whether the single-token items of a step have one context far longer than the rest: more than
+// four times their mean and 4,096 tokens beyond that. The keys are then cut into runs of 1,024 or
+// more, as many as the longest request needs, instead of as many as fill the chip with requests of
+// equal length; a long request among short ones is otherwise read by a few workgroups while the
+// rest of the chip waits (31 requests of 1,024 tokens and one of 60,000: 429 -> 55 us a layer at
+// head size 64). Steps of equal lengths pay 10 to 25 us a layer for the extra runs, so it is
+// decided step by step. Tuned on 256 compute units.
+int psamd_attention_decode_skewed(int n_dec, int longest, int64_t total) {
+  return n_dec > 1 && static_cast<int64_t>(longest) * n_dec > 4 * total + 4096LL * n_dec;
+}
+
+// How psamd_attention_decode should cut the keys of a step of n_dec single-token items whose
+// longest context is kv_len (for a captured step: the longest there can be): *nsplit runs per
+// request, none shorter than *min_run keys. Two workgroups per compute unit; from one per compute
+// unit on, no split and no merge kernel (32 requests x 8 kv heads at head size 128: 48 -> 41 us).
+int psamd_attention_decode_plan(int n_dec, int kv_len, int skewed, int hkv, int window, int* nsplit, int* min_run) {
+  PSAMD_REQUIRE(n_dec >= 1 && kv_len >= 1 && hkv >= 1 && nsplit != nullptr && min_run != nullptr, "decode plan: bad sizes");
+  if (window > 0) kv_len = std::min(kv_len, window);
+  const int64_t pairs = static_cast<int64_t>(n_dec) * hkv;
+  int n = pairs >= 256 ? 1 : static_cast<int>(std::max<int64_t>(1, std::min<int64_t>({64, 512 / pairs, ceil_div(kv_len, 128)})));
+  int run = 128;
+  if (skewed && window <= 0) {
+    n = std::max(n, static_cast<int>(std::min<int64_t>({64, 4096 / n_dec, ceil_div(kv_len, 1024)})));
+    run = 1024;
+  }
+  *nsplit = std::max(n, 1);
+  *min_run = run;
+  return 0;
+}
+
+// (requests x runs) of any plan for up to max_requests single-token items: room for the partial
+// results of every decode step, so that the buffers never grow.
+int psamd_attention_decode_max_parts(int max_requests) { return std::max({4096, 512, max_requests}); }
 
 // part_o needs n_dec * hq * nsplit * head_dim floats, part_ml n_dec * hq * nsplit * 2.
 // min_split_keys: a request's keys are cut into runs no shorter than this (a multiple of 32), so

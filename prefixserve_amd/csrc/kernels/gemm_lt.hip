@@ -15,22 +15,10 @@
 // the system's): nothing links against it, and if it or one of its entry points is missing
 // psamd_gemm_lt_available() says so and the caller keeps using torch.mm.
 //
-// The library's heuristic picks an algorithm without running anything. psamd_gemm_lt_tune() times
-// every algorithm that supports a shape on the caller's buffers and keeps the fastest for that
-// shape and, where they support them, for row counts within a quarter of it. What it finds depends
-// on the copy of the library in the process: the one that ships with torch here has 4,626
-// algorithms for bfloat16, 230 of them for the products of the Llama 3.2 1B sizes, and its
-// heuristic already returns the fastest of them (one shape of eight gained 5%); ROCm 7.2's own copy
-// has 20,141 (2,084), and its heuristic's first choice is 6 to 30% slower than its best (2,048 rows:
-// q/k/v 30 -> 26 us, o 31 -> 21, gate/up 114 -> 102, down 84 -> 66), which is about where the other
-// copy's heuristic is. So the tuning is off unless asked for. It is meant for warm-up: it takes a
-// quarter of a second per shape and waits for the stream.
-//
 // No kernels in this file.
 
 #include <dlfcn.h>
 #include <hipblaslt/hipblaslt.h>
-#include <hipblaslt/hipblaslt-ext.hpp>
 
 #include <algorithm>
 #include <cstdlib>
@@ -62,10 +50,6 @@ struct Api {
   decltype(&hipblasLtMatmulPreferenceSetAttribute) pref_set = nullptr;
   decltype(&hipblasLtMatmulAlgoGetHeuristic) heuristic = nullptr;
   decltype(&hipblasLtMatmul) matmul = nullptr;
-  // The extension interface (C++ entry points of the same library), for tuning only.
-  bool ext = false;
-  decltype(&hipblaslt_ext::getAllAlgos) all_algos = nullptr;
-  decltype(&hipblaslt_ext::matmulIsAlgoSupported) is_supported = nullptr;
 };
 
 template <typename F>
@@ -90,14 +74,6 @@ const Api& api() {
            bind(lib, "hipblasLtMatmulPreferenceDestroy", a.pref_destroy) &&
            bind(lib, "hipblasLtMatmulPreferenceSetAttribute", a.pref_set) &&
            bind(lib, "hipblasLtMatmulAlgoGetHeuristic", a.heuristic) && bind(lib, "hipblasLtMatmul", a.matmul);
-    a.ext = bind(lib,
-                 "_ZN13hipblaslt_ext11getAllAlgosEPvNS_8GemmTypeE18hipblasOperation_tS2_11hipDataTypeS3_S3_S3_"
-                 "20hipblasComputeType_tRSt6vectorI33_hipblasLtMatmulHeuristicResult_tSaIS6_EE",
-                 a.all_algos) &&
-            bind(lib,
-                 "_ZN13hipblaslt_ext21matmulIsAlgoSupportedEPvP27hipblasLtMatmulDescOpaque_tPKvP29hipblasLtMatrixLayoutOpaque_t"
-                 "S6_S4_S6_S6_R22_hipblasLtMatmulAlgo_tRm",
-                 a.is_supported);
     return a;
   }();
   return loaded;
@@ -110,21 +86,10 @@ struct Plan {
   size_t workspace = 0;
 };
 
-struct Tuned {            // the fastest algorithm found for [M, K] x [N, K]^T by timing
-  int64_t M;
-  int N, K;
-  bool float_out;
-  hipblasLtMatmulAlgo_t algo;
-  size_t workspace;
-};
-
 struct Device {
   hipblasLtHandle_t handle = nullptr;
   void* workspace = nullptr;
   std::map<std::tuple<int64_t, int, int, bool, bool>, Plan> plans;
-  std::vector<Tuned> tuned;
-  std::vector<hipblasLtMatmulHeuristicResult_t> all[2];     // every algorithm for bfloat16 / float32 output
-  bool all_asked[2] = {false, false};
 };
 
 std::mutex g_lock;
@@ -164,24 +129,6 @@ int make_plan(const Api& a, Device& dev, int64_t M, int N, int K, bool use_works
   }
   p.algo = found.algo;
   p.workspace = found.workspaceSize;
-  if (use_workspace && a.ext) {
-    // A tuned algorithm of the nearest row count within a quarter, if it supports this one.
-    const Tuned* best = nullptr;
-    for (const Tuned& t : dev.tuned) {
-      if (t.N != N || t.K != K || t.float_out != float_out || 4 * t.M > 5 * M || 4 * M > 5 * t.M) continue;
-      if (best == nullptr || std::llabs(t.M - M) < std::llabs(best->M - M)) best = &t;
-    }
-    if (best != nullptr) {
-      const float one = 1.f, zero = 0.f;
-      hipblasLtMatmulAlgo_t algo = best->algo;
-      size_t need = 0;
-      if (a.is_supported(dev.handle, p.desc, &one, p.w, p.x, &zero, p.out, p.out, algo, need) == HIPBLAS_STATUS_SUCCESS &&
-          need <= kWorkspaceBytes) {
-        p.algo = algo;
-        p.workspace = need;
-      }
-    }
-  }
   return 0;
 }
 
@@ -240,168 +187,6 @@ int psamd_gemm_lt(void* stream, const void* x, const void* w, void* out, int out
                                       roomy ? dev.workspace : nullptr, roomy ? kWorkspaceBytes : 0,
                                       static_cast<hipStream_t>(stream));
   if (st != HIPBLAS_STATUS_SUCCESS) return fail("psamd_gemm_lt: hipblasLtMatmul returned " + std::to_string(st));
-  return 0;
-}
-
-// Times every algorithm of the library that supports out[M, N] = x[M, K] * w[N, K]^T (with a
-// workspace) on the given buffers, w being each of the n_ws matrices of that shape in turn, and keeps the fastest for this shape from now on, if it beats
-// the heuristic's choice by 3% or more. out receives the product by the kept algorithm and
-// ref_out by the heuristic's, for the caller to compare; us_before and us_after their times.
-// Waits for the stream. Returns 0, 1 for an error, 2 if the library or its extension interface
-// is not there (nothing changes then).
-int psamd_gemm_lt_tune(void* stream, const void* x, const void* const* ws, int n_ws, void* out, void* ref_out, int out_dtype,
-                       int64_t M, int N, int K, float* us_before, float* us_after) {
-  PSAMD_REQUIRE(M > 0 && N > 0 && K > 0 && M <= INT32_MAX, "bad sizes");
-  PSAMD_REQUIRE(out_dtype == kBF16 || out_dtype == kF32, "the output is bfloat16 or float32");
-  PSAMD_REQUIRE(us_before != nullptr && us_after != nullptr && out != nullptr && ref_out != nullptr, "missing outputs");
-  PSAMD_REQUIRE(ws != nullptr && n_ws >= 1, "at least one matrix");
-  const bool float_out = out_dtype == kF32;
-  const Api& a = api();
-  int id = 0;
-  if (!a.ok || !a.ext || hipGetDevice(&id) != hipSuccess || id < 0 || id >= kMaxDevices) return 2;
-  std::lock_guard<std::mutex> guard(g_lock);
-  Device& dev = g_devices[id];
-  PSAMD_REQUIRE(dev.handle != nullptr, "call psamd_gemm_lt_available() on this device first");
-  hipStream_t s = static_cast<hipStream_t>(stream);
-
-  // The plan of the heuristic's choice, made anew so that an earlier tuning does not count as "before".
-  const auto key = std::make_tuple(M, N, K, true, float_out);
-  auto it = dev.plans.find(key);
-  if (it != dev.plans.end()) {
-    drop(a, it->second);
-    dev.plans.erase(it);
-  }
-  dev.tuned.erase(std::remove_if(dev.tuned.begin(), dev.tuned.end(),
-                                 [&](const Tuned& t) { return t.M == M && t.N == N && t.K == K && t.float_out == float_out; }),
-                  dev.tuned.end());
-  Plan p;
-  {
-    std::vector<Tuned> none;
-    none.swap(dev.tuned);                                   // no borrowing from neighbours either
-    const int rc = make_plan(a, dev, M, N, K, true, float_out, p);
-    none.swap(dev.tuned);
-    if (rc != 0) return 2;
-  }
-  const hipblasLtMatmulAlgo_t first = p.algo;
-
-  const int which = float_out ? 1 : 0;
-  if (!dev.all_asked[which]) {
-    dev.all_asked[which] = true;
-    const hipDataType out_type = float_out ? HIP_R_32F : HIP_R_16BF;
-    if (a.all_algos(dev.handle, hipblaslt_ext::GemmType::HIPBLASLT_GEMM, HIPBLAS_OP_T, HIPBLAS_OP_N, HIP_R_16BF, HIP_R_16BF,
-                    out_type, out_type, HIPBLAS_COMPUTE_32F, dev.all[which]) != HIPBLAS_STATUS_SUCCESS)
-      dev.all[which].clear();
-  }
-
-  hipEvent_t e0 = nullptr, e1 = nullptr;
-  if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) {
-    drop(a, p);
-    return fail("psamd_gemm_lt_tune: no events");
-  }
-  const float one = 1.f, zero = 0.f;
-  // Microseconds per call over `reps` calls into `dst`, or a negative number if the call fails.
-  // The matrices are taken in turn (a model's layers): each call then reads its matrix from
-  // memory, as a step does, not from the caches the call before it left warm.
-  int turn = 0;
-  auto timed = [&](hipblasLtMatmulAlgo_t& algo, void* dst, int reps) -> float {
-    if (a.matmul(dev.handle, p.desc, &one, ws[0], p.w, x, p.x, &zero, dst, p.out, dst, p.out, &algo, dev.workspace,
-                 kWorkspaceBytes, s) != HIPBLAS_STATUS_SUCCESS)
-      return -1.f;
-    if (hipEventRecord(e0, s) != hipSuccess) return -1.f;
-    for (int i = 0; i < reps; ++i) {
-      turn = (turn + 1) % n_ws;
-      if (a.matmul(dev.handle, p.desc, &one, ws[turn], p.w, x, p.x, &zero, dst, p.out, dst, p.out, &algo, dev.workspace,
-                   kWorkspaceBytes, s) != HIPBLAS_STATUS_SUCCESS)
-        return -1.f;
-    }
-    if (hipEventRecord(e1, s) != hipSuccess || hipEventSynchronize(e1) != hipSuccess) return -1.f;
-    float ms = 0.f;
-    if (hipEventElapsedTime(&ms, e0, e1) != hipSuccess) return -1.f;
-    return ms * 1000.f / static_cast<float>(reps);
-  };
-
-  // A first pass over all that support the shape, three calls each; the leaders again, with the
-  // heuristic's choice among them, in three rounds of ten (the lowest round counts).
-  std::vector<std::pair<float, size_t>> screened;
-  for (size_t i = 0; i < dev.all[which].size(); ++i) {
-    hipblasLtMatmulAlgo_t algo = dev.all[which][i].algo;
-    size_t need = 0;
-    if (a.is_supported(dev.handle, p.desc, &one, p.w, p.x, &zero, p.out, p.out, algo, need) != HIPBLAS_STATUS_SUCCESS ||
-        need > kWorkspaceBytes)
-      continue;
-    const float us = timed(algo, out, 3);
-    if (us > 0.f) screened.push_back({us, i});
-  }
-  std::sort(screened.begin(), screened.end());
-  if (screened.size() > 12) screened.resize(12);
-  std::vector<hipblasLtMatmulAlgo_t> finalists{first};
-  for (const auto& sc : screened) finalists.push_back(dev.all[which][sc.second].algo);
-  std::vector<float> best(finalists.size(), 1e30f);
-  for (int round = 0; round < 3; ++round)
-    for (size_t i = 0; i < finalists.size(); ++i) {
-      const float us = timed(finalists[i], out, 10);
-      if (us > 0.f) best[i] = std::min(best[i], us);
-    }
-  size_t winner = 0;
-  for (size_t i = 1; i < finalists.size(); ++i)
-    if (best[i] < best[winner]) winner = i;
-  if (best[winner] > 0.97f * best[0]) winner = 0;
-  *us_before = best[0];
-  *us_after = best[winner];
-
-  hipblasLtMatmulAlgo_t ref_algo = first;
-  n_ws = 1;                                              // both products by the first matrix
-  const bool ran = timed(ref_algo, ref_out, 1) > 0.f && timed(finalists[winner], out, 1) > 0.f;
-  (void)hipEventDestroy(e0);
-  (void)hipEventDestroy(e1);
-  if (!ran) {
-    drop(a, p);
-    return fail("psamd_gemm_lt_tune: the product failed");
-  }
-  if (winner != 0) {
-    size_t need = 0;
-    hipblasLtMatmulAlgo_t algo = finalists[winner];
-    (void)a.is_supported(dev.handle, p.desc, &one, p.w, p.x, &zero, p.out, p.out, algo, need);
-    p.algo = algo;
-    p.workspace = need;
-    dev.tuned.push_back(Tuned{M, N, K, float_out, algo, need});
-    // Plans of neighbouring row counts made before now may borrow it: they are made again when next asked for.
-    for (auto pit = dev.plans.begin(); pit != dev.plans.end();) {
-      const auto& k = pit->first;
-      const int64_t m2 = std::get<0>(k);
-      if (std::get<1>(k) == N && std::get<2>(k) == K && std::get<3>(k) && std::get<4>(k) == float_out && 4 * m2 <= 5 * M &&
-          4 * M <= 5 * m2) {
-        drop(a, pit->second);
-        pit = dev.plans.erase(pit);
-      } else {
-        ++pit;
-      }
-    }
-  }
-  dev.plans.emplace(key, p);
-  return 0;
-}
-
-// Forgets what psamd_gemm_lt_tune() kept for a shape (a caller that found its result wrong).
-int psamd_gemm_lt_untune(int out_dtype, int64_t M, int N, int K) {
-  const bool float_out = out_dtype == kF32;
-  const Api& a = api();
-  int id = 0;
-  if (!a.ok || hipGetDevice(&id) != hipSuccess || id < 0 || id >= kMaxDevices) return 2;
-  std::lock_guard<std::mutex> guard(g_lock);
-  Device& dev = g_devices[id];
-  dev.tuned.erase(std::remove_if(dev.tuned.begin(), dev.tuned.end(),
-                                 [&](const Tuned& t) { return t.M == M && t.N == N && t.K == K && t.float_out == float_out; }),
-                  dev.tuned.end());
-  for (auto pit = dev.plans.begin(); pit != dev.plans.end();) {
-    const auto& k = pit->first;
-    if (std::get<1>(k) == N && std::get<2>(k) == K && std::get<3>(k) && std::get<4>(k) == float_out) {
-      drop(a, pit->second);
-      pit = dev.plans.erase(pit);
-    } else {
-      ++pit;
-    }
-  }
   return 0;
 }
 

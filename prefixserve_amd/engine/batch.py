@@ -22,17 +22,6 @@ from ..build import ensure_core
 PAGE = 16  # tokens per page; equals the cache core's BLOCK_SIZE
 
 
-def decode_is_skewed(count: int, longest: int, total: int) -> bool:
-    """Whether the single-token items of a step have one context far longer than the rest: more
-    than four times their mean and 4,096 tokens beyond that. The decode attention then cuts every
-    request's keys into runs of 1,024 or more, as many as the longest request needs, instead of
-    as many as fill the chip with requests of equal length; a long request among short ones is
-    otherwise read by a few workgroups while the rest of the chip waits (31 requests of 1,024 tokens
-    and one of 60,000: 429 -> 55 us a layer at head size 64). Steps of equal lengths pay 10 to 25 us
-    a layer for the extra runs, so it is decided step by step; a captured graph is keyed by it."""
-    return count > 1 and longest * count > 4 * total + 4096 * count
-
-
 class EngineError(RuntimeError):
     """The engine was given a batch it cannot run: a configuration or scheduler bug."""
 
@@ -74,7 +63,7 @@ class StepContext:
     num_decode: int            # items with exactly one token (served by the decode kernel)
     num_prefill_tiles: int
     max_kv_len: int
-    decode_skewed: bool        # one single-token item's context is far longer than the others'
+    decode_skewed: bool        # the kernels' verdict on the single-token items' context lengths (one far longer than the rest)
     token_ids: torch.Tensor    # [T]
     positions: torch.Tensor    # [T] absolute
     tok_item: torch.Tensor     # [T] item of each token
@@ -96,11 +85,15 @@ class StepPacker:
     before the previous step's kernels were enqueued; it waits for the previous copy itself."""
 
     def __init__(self, device: torch.device, groups: Sequence[GroupMeta], vocab_size: int, max_position: int,
-                 num_slots: int, prefill_tile: int, capacity: int = 1 << 16) -> None:
+                 num_slots: int, prefill_tile: int, capacity: int = 1 << 16, skew_rule: Any = None) -> None:
+        """``skew_rule(count, longest, total) -> bool``: the kernel library's rule for when the
+        context lengths of a step's single-token items count as skewed (it cuts their keys
+        another way then, and a captured step is keyed by it); without one, never."""
         self.device = torch.device(device)
         self.groups = list(groups)
         self.vocab_size, self.max_position, self.num_slots = int(vocab_size), int(max_position), int(num_slots)
         self.prefill_tile = int(prefill_tile)
+        self._skew_rule = skew_rule
         self.on_gpu = self.device.type == "cuda"
         self._copied = torch.cuda.Event() if self.on_gpu else None
         self._pack_step = ensure_core().pack_step
@@ -156,7 +149,8 @@ class StepPacker:
         _, on_dev, host, groups = self._views
         return StepContext(
             num_tokens=t_n, num_items=b, num_logit_rows=s_n, num_decode=n_dec, num_prefill_tiles=n_tiles,
-            max_kv_len=max_kv_len, decode_skewed=decode_is_skewed(n_dec, dec_max_kv, dec_sum_kv), groups=groups,
+            max_kv_len=max_kv_len, decode_skewed=bool(self._skew_rule(n_dec, dec_max_kv, dec_sum_kv)) if self._skew_rule and n_dec > 1 else False,
+            groups=groups,
             keys=[it.key for it in items],
             want_counts=[len(it.want) for it in items], host=host, **on_dev,
         )

@@ -38,11 +38,6 @@ class EngineConfig:
     # meets a stop token in between has computed up to decode_steps - 1 tokens for nothing, and
     # a request that arrives waits until the running batch has finished its steps.
     decode_steps: int = 1
-    # warm_up() lets the product library time its algorithms for a step of max_prefill_tokens
-    # tokens and keep the fastest (a quarter of a second per matrix shape of the model). Off by
-    # default: the library that comes with torch already picks its fastest; a copy with a weaker
-    # heuristic gains 10 to 30% on the products of a prompt.
-    tune_products: bool = False
 
 
 class Engine:
@@ -122,29 +117,17 @@ class Engine:
         sizes = [n for n in (1, 2, 4, 8) if n <= top] + list(range(16, top + 1, 8))
         return sizes if sizes and sizes[-1] == top else sizes + [top]
 
-    def warm_up(self, tune_tokens: tuple[int, ...] | None = None) -> None:
+    def warm_up(self) -> None:
         """Does before the first request what the first requests would otherwise pay for: the
         largest step there can be (it sizes the buffers that steps share; a buffer that grows
         later drops the captured graphs, which hold its address) and, if steps are replayed as
         graphs, a capture of the decode step at every size batches are filled up to. The steps run on
         token 0 and write into the first pages of every pool, which hold nothing anybody reads
-        before writing it. Before that, if the configuration asks for it, the product library
-        times its algorithms for steps of ``tune_tokens`` tokens (default: a full portion) and
-        keeps the fastest. Call it before any request is running."""
+        before writing it. Call it before any request is running."""
         r = self.runner
-        groups = r.num_blocks_per_group
-        n = min(self.cfg.max_prefill_tokens, self.cfg.max_seq_len, PAGE * min(groups))
-        if self.cfg.tune_products:
-            r.tune_products(tune_tokens if tune_tokens is not None else (n,))
-        one_page = [[0] for _ in groups]
-        # The largest step a scheduler can ask for: a portion of the whole budget beside
-        # decoding requests in all other places, every item wanting its logits.
-        items = [StepItem(key="warm-up", tokens=np.zeros(n, dtype=np.int32), start=0,
-                          block_tables=[list(range(-(-n // PAGE))) for _ in groups], slot=0, want=(n - 1,))]
-        items += [StepItem(key=f"warm-up-{i}", tokens=(0,), start=0, block_tables=one_page, slot=0, want=(0,))
-                  for i in range(self.cfg.max_num_seqs - 1)]
-        r.step(items)
+        r.step(r.largest_step())
         if r.use_graphs:
+            one_page = [[0] for _ in r.num_blocks_per_group]
             for size in reversed(self._batch_sizes()):
                 items = [StepItem(key=f"warm-up-{i}", tokens=(0,), start=0, block_tables=one_page, slot=0, want=(0,))
                          for i in range(size)]

@@ -12,6 +12,7 @@ import logging
 from pathlib import Path
 from typing import Any, Sequence
 
+import numpy as np
 import torch
 
 import prefixserve_amd.models  # noqa: F401  (fills the architecture registry)
@@ -65,6 +66,16 @@ class ModelRunner:
         self.layer_groups = plan_groups(self.model.cache_needs())
         itemsize = torch.empty((), dtype=self.dtype).element_size()
         self.bytes_per_block = [g.bytes_per_block(itemsize) for g in self.layer_groups]
+        state_needs = self.model.state_needs()
+        self.states = make_states(state_needs, self.max_num_seqs, self.device)
+        self.state_bytes_per_slot = sum(
+            int(torch.empty((), dtype=n.dtype).element_size()) * int(torch.Size(n.shape).numel())
+            for n in state_needs.values())
+        # A model whose mixers keep state of their own runs eagerly: capturing a step runs it
+        # once before and once after the capture, which pages of keys and values do not mind
+        # and a state that is added to does.
+        self.use_graphs = bool(use_graphs) and self.device.type == "cuda" and not state_needs
+        self._graphs: dict[Any, Any] = {}
         if num_blocks is None:
             blocks = self._size_pools(reserve_bytes)
         elif isinstance(num_blocks, int):
@@ -73,23 +84,19 @@ class ModelRunner:
             blocks = [int(n) for n in num_blocks]
         if len(blocks) != len(self.layer_groups):
             raise ValueError(f"{len(blocks)} pool sizes for {len(self.layer_groups)} layer groups")
-        self.num_blocks_per_group = blocks
-        self.pools = KVPools(self.layer_groups, blocks, self.dtype, self.device)
-        state_needs = self.model.state_needs()
-        self.states = make_states(state_needs, self.max_num_seqs, self.device)
-        self.state_bytes_per_slot = sum(
-            int(torch.empty((), dtype=n.dtype).element_size()) * int(torch.Size(n.shape).numel())
-            for n in state_needs.values())
+        self._install_pools(blocks)
+        logger.info("KV pools: %s blocks (%.2f GB)", blocks, self.pools.nbytes() / 1e9)
+
+    def _install_pools(self, blocks: Sequence[int]) -> None:
+        """Page pools of the given sizes, attached to the model, and the packer that checks page
+        ids against them."""
+        self.num_blocks_per_group = list(blocks)
+        self.pools = KVPools(self.layer_groups, self.num_blocks_per_group, self.dtype, self.device)
         self.model.attach(self.pools.layer_caches(), self.states)
         self.packer = StepPacker(
             self.device, [GroupMeta(nb, g.need.window) for g, nb in zip(self.layer_groups, blocks)],
-            self.spec.vocab_size, self.max_seq_len, self.max_num_seqs, self.ops.PREFILL_TILE_Q)
-        # A model whose mixers keep state of their own runs eagerly: capturing a step runs it
-        # once before and once after the capture, which pages of keys and values do not mind
-        # and a state that is added to does.
-        self.use_graphs = bool(use_graphs) and self.device.type == "cuda" and not self.model.state_needs()
-        self._graphs: dict[Any, Any] = {}
-        logger.info("KV pools: %s blocks (%.2f GB)", blocks, self.pools.nbytes() / 1e9)
+            self.spec.vocab_size, self.max_seq_len, self.max_num_seqs, self.ops.PREFILL_TILE_Q,
+            skew_rule=getattr(self.ops, "decode_is_skewed", None))
 
     # ------------------------------------------------------------ properties
 
@@ -112,33 +119,53 @@ class ModelRunner:
 
     # ---------------------------------------------------------------- sizing
 
+    def largest_step(self) -> list[StepItem]:
+        """The largest step a scheduler can ask this runner for: a portion of the whole prefill
+        budget beside decoding requests in all other places, every item wanting its logits. On
+        token 0, in the first pages of every pool and in slot 0: for sizing buffers before any
+        request runs (nothing anybody reads before writing it is touched)."""
+        groups = self.num_blocks_per_group
+        n = min(self.max_prefill_tokens, self.max_seq_len, PAGE * min(groups))
+        one_page = [[0] for _ in groups]
+        items = [StepItem(key="largest", tokens=np.zeros(n, dtype=np.int32), start=0,
+                          block_tables=[list(range(-(-n // PAGE))) for _ in groups], slot=0, want=(n - 1,))]
+        items += [StepItem(key=f"largest-{i}", tokens=(0,), start=0, block_tables=one_page, slot=0, want=(0,))
+                  for i in range(self.max_num_seqs - 1)]
+        return items
+
     def _size_pools(self, reserve_bytes: int) -> list[int]:
-        """Pages that fit in what is free after the weights, the buffers of a worst-case
-        step and a reserve (prefixserve/llama_engine.py:231-267 sizes its pool the same way:
-        sizing from free memory alone would leave nothing for activations)."""
+        """Pages that fit in what is free after the weights, after everything the largest step
+        really takes, and a reserve. The step is run once on a throwaway pool of a few pages: its
+        buffers stay (the workspace keeps them for every later step), so what the device reports
+        free afterwards is what is left for pages (prefixserve/llama_engine.py:231-267,304-320
+        measures a dummy step on a dummy pool the same way; sizing from free memory alone would
+        leave nothing for activations, and an estimate would have to know every part's buffers)."""
         if self.device.type != "cuda":
             raise ValueError("num_blocks must be given when not on a GPU")
-        t = self.max_prefill_tokens + self.max_num_seqs
-        act = self._activation_bytes(t)
+        probe = -(-min(self.max_prefill_tokens, self.max_seq_len) // PAGE) + 1
+        self._install_pools([probe] * len(self.layer_groups))
+        graphs, self.use_graphs = self.use_graphs, False
+        try:
+            self.step(self.largest_step())
+            torch.cuda.synchronize(self.device)
+        finally:
+            self.use_graphs = graphs
+        for state in self.states.values():
+            state.zero_()
+        self.pools = None
+        self.model.attach({}, self.states)
+        torch.cuda.empty_cache()             # the throwaway pool goes back to the device; the step's buffers are in use
         free, _total = torch.cuda.mem_get_info(self.device)
-        usable = free - act - reserve_bytes
-        per_token_page = sum(self.bytes_per_block)
-        n = int(usable // per_token_page)
+        usable = free - reserve_bytes
+        n = int(usable // sum(self.bytes_per_block))
+        n = min(n, (1 << 27) - 1)            # a token's place, page * 16 + offset, is a 32-bit integer
         need = -(-self.max_seq_len // PAGE)
         if n < need:
-            raise EngineError(f"only {n} KV blocks fit ({usable / 1e9:.2f} GB usable); one request of "
-                              f"max_seq_len needs {need}")
+            raise EngineError(f"only {n} KV blocks fit ({usable / 1e9:.2f} GB usable after a largest step's buffers "
+                              f"and a reserve of {reserve_bytes / 1e9:.2f} GB); one request of max_seq_len needs {need}")
+        logger.info("pools sized after a measured largest step: %.2f GB of buffers, %.2f GB for pages",
+                    self.workspace.nbytes() / 1e9, usable / 1e9)
         return [n] * len(self.layer_groups)
-
-    def _activation_bytes(self, tokens: int) -> int:
-        """Device memory the buffers of a step of ``tokens`` tokens take: what the parts say they
-        ask for (buffers are shared between layers by name, so the largest layer counts), the
-        float32 residual stream, the logits of every request and a margin."""
-        s = self.spec
-        itemsize = torch.empty((), dtype=self.dtype).element_size()
-        widest = max((sum(p.activation_bytes(tokens, itemsize) for p in blk.parts()) for blk in self.model.blocks),
-                     default=0)
-        return widest + tokens * s.hidden_size * 4 + self.max_num_seqs * s.vocab_size * 4 + (256 << 20)
 
     # ------------------------------------------------------------------ step
 
@@ -152,6 +179,8 @@ class ModelRunner:
         ``token_feed``: int32 ``[T]`` on the device, taken for the step's token ids instead of
         the items' own (which must still be valid ids): the tokens an earlier step sampled and
         the host has not seen yet."""
+        if self.states:
+            self._clear_new_slots(items)
         if self.use_graphs and all(len(it.tokens) == 1 for it in items):
             from prefixserve_amd.engine.graphs import graphed_decode_step
 
@@ -163,29 +192,19 @@ class ModelRunner:
             ctx.token_ids.copy_(token_feed)
         return self.model.step(ctx)
 
+    def _clear_new_slots(self, items: Sequence[StepItem]) -> None:
+        """Zeroes the state slots of the items that start at position 0, in stream order before
+        the step: a slot comes from the allocator with its last owner's contents, and a request
+        (new, or sent back and starting over) begins from nothing. Mixers never clear slots."""
+        fresh = sorted({int(it.slot) for it in items if it.start == 0})
+        if not fresh:
+            return
+        for s in fresh:
+            if not 0 <= s < self.max_num_seqs:
+                raise EngineError(f"state slot {s} outside [0, {self.max_num_seqs})")
+        index = torch.tensor(fresh, dtype=torch.int64).to(self.device, non_blocking=True)
+        for state in self.states.values():
+            state.index_fill_(0, index, 0)
+
     def pack(self, items: Sequence[StepItem]) -> StepContext:
         return self.packer.pack(items)
-
-    def tune_products(self, token_counts: Sequence[int]) -> list[tuple[int, tuple[int, int], float, float]]:
-        """Lets the product library time its algorithms for steps of the given token counts,
-        once per distinct matrix shape of the model's parts, and keep the fastest: the library's
-        own choice is made without running anything. The same product of every layer shares a
-        shape; its matrices are timed in turn, so that each call reads its matrix from memory as
-        a step does. Returns (tokens, (out, in), microseconds before, after) per tuned product.
-        For warm-up: a second or so per shape."""
-        tune = getattr(self.ops, "tune_linear", None)
-        done: list[tuple[int, tuple[int, int], float, float]] = []
-        if tune is None or self.dtype != torch.bfloat16:
-            return done
-        by_shape: dict[tuple[int, int], list[torch.Tensor]] = {}
-        for blk in self.model.blocks:
-            for part in blk.parts():
-                for w in part.product_weights():
-                    by_shape.setdefault((int(w.shape[0]), int(w.shape[1])), []).append(w)
-        for shape, weights in by_shape.items():
-            for t in dict.fromkeys(int(t) for t in token_counts):
-                res = tune(t, weights)
-                if res is not None:
-                    done.append((t, shape, res[0], res[1]))
-                    logger.info("product of %d tokens by [%d, %d]: %.1f -> %.1f us", t, shape[0], shape[1], *res)
-        return done

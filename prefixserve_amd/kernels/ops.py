@@ -48,14 +48,16 @@ _SIGNATURES = {
     "psamd_rope_kv_append": [_vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp, _vp, _vp, _vp],
     "psamd_linear": [_vp, _vp, _i32, _vp, _i32, _vp, _i32, _i64, _i32, _i32],
     "psamd_gemm_lt": [_vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32],
-    "psamd_gemm_lt_tune": [_vp, _vp, _vp, _i32, _vp, _vp, _i32, _i64, _i32, _i32, _vp, _vp],
-    "psamd_gemm_lt_untune": [_i32, _i64, _i32, _i32],
     "psamd_linear_skinny": [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32],
     "psamd_linear_skinny_ksplit": [_i32, _i32, _i32],
     "psamd_qkv_rope_append": [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp],
     "psamd_attention_generic": [_vp, _vp, _i32, _vp, _vp, _i32, _i64, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _f32, _i32],
     "psamd_attention_mfma_supports": [_i32, _i32, _i32],
     "psamd_attention_prefill_nsplit": [_i32, _i32, _i32, _i32, _i32],
+    "psamd_attention_prefill_part_rows": [_i32, _i32, _i32],
+    "psamd_attention_decode_skewed": [_i32, _i32, _i64],
+    "psamd_attention_decode_plan": [_i32, _i32, _i32, _i32, _i32, _vp, _vp],
+    "psamd_attention_decode_max_parts": [_i32],
     "psamd_attention_prefill": [_vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _f32,
                                 _i32, _vp, _vp, _i32],
     "psamd_attention_decode": [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32,
@@ -85,6 +87,7 @@ class HipOps:
         self.ws = workspace
         self._sample_scratch: torch.Tensor | None = None
         self._step_stream: int | None = None
+        self._plans: dict[tuple, tuple[int, int]] = {}
         self._slice_views: dict[tuple, tuple] = {}      # (name, slices, rows) -> (buffer, its [slices, rows, N] view)
         # The library for large bfloat16 products, called directly if it can be (it sets itself up
         # here, outside any capture); through torch.mm otherwise.
@@ -241,44 +244,6 @@ class HipOps:
         self._ok(self.lib.psamd_linear(self._stream(), x.data_ptr(), _code(x.dtype), w.data_ptr(), _code(w.dtype),
                                        out.data_ptr(), _code(out.dtype), m, n, k))
 
-    def tune_linear(self, rows: int, weights: Sequence[torch.Tensor],
-                    out_dtype: torch.dtype | None = None) -> tuple[float, float] | None:
-        """Lets the library time its algorithms for ``rows`` tokens times each of ``weights`` in turn
-        (matrices of one shape [N, K], bfloat16: the layers of a model, so that a call reads its
-        matrix from memory as a step does) and keep the fastest for that shape and for row
-        counts within a quarter of it. Returns
-        (microseconds with the heuristic's choice, microseconds with what is kept now), or None
-        where the library product does not apply. The kept algorithm's product is compared with
-        the heuristic's here, and dropped again if they differ by more than rounding. Takes a
-        second or two and waits for the device: for warm-up, outside any capture."""
-        w = weights[0]
-        if not (self._direct_library and rows > self.SKINNY_MAX_ROWS and all(
-                v.dtype == torch.bfloat16 and v.shape == w.shape and v.dim() == 2 and v.is_contiguous() for v in weights)):
-            return None
-        n, k = w.shape
-        pointers = (ctypes.c_void_p * len(weights))(*[v.data_ptr() for v in weights])
-        out_dtype = out_dtype or torch.bfloat16
-        gen = torch.Generator(device=self.device).manual_seed(rows + n)
-        x = torch.randn(rows, k, device=self.device, generator=gen).to(torch.bfloat16)
-        got = torch.empty(rows, n, dtype=out_dtype, device=self.device)
-        ref = torch.empty_like(got)
-        before, after = ctypes.c_float(0.0), ctypes.c_float(0.0)
-        rc = self.lib.psamd_gemm_lt_tune(self._stream(), x.data_ptr(), pointers, len(weights), got.data_ptr(), ref.data_ptr(),
-                                         _code(out_dtype), rows, n, k, ctypes.byref(before), ctypes.byref(after))
-        if rc == 2:
-            return None
-        self._ok(rc)
-        torch.cuda.synchronize(self.device)
-        # Two correct algorithms differ by the order of their sums: a few units of bfloat16's last place.
-        scale = float(ref.float().abs().max())
-        apart = float((got.float() - ref.float()).abs().max())
-        if not apart <= 2.0 ** -6 * max(scale, 1e-30):
-            self.lib.psamd_gemm_lt_untune(_code(out_dtype), rows, n, k)
-            logger.warning("tuned product for %d x [%d, %d] differs from the heuristic's by %.3g of %.3g: not kept",
-                           rows, n, k, apart, scale)
-            return before.value, before.value
-        return before.value, after.value
-
     def linear_to_residual(self, x, w, name: str) -> torch.Tensor:
         """x @ w^T for a consumer that adds it to the residual stream (the fused add+norm).
         Returns [T, N] in the activation dtype or, for a small bfloat16 step whose product has
@@ -320,6 +285,24 @@ class HipOps:
 
     # --------------------------------------------------------------- attention
 
+    def decode_is_skewed(self, count: int, longest: int, total: int) -> bool:
+        """The library's rule for when the single-token items of a step have one context far
+        longer than the rest (it then cuts every request's keys into long runs, as many as the
+        longest needs). A captured decode step is keyed by it."""
+        return bool(self.lib.psamd_attention_decode_skewed(int(count), int(longest), int(total)))
+
+    def decode_plan(self, count: int, kv_len: int, skewed: bool, hkv: int, window: int) -> tuple[int, int]:
+        """(runs per request, shortest run in keys) for a step of ``count`` single-token items."""
+        plan = self._plans.get((count, kv_len, skewed, hkv, window))
+        if plan is None:
+            nsplit, min_run = ctypes.c_int(0), ctypes.c_int(0)
+            self._ok(self.lib.psamd_attention_decode_plan(count, kv_len, int(skewed), hkv, window, ctypes.byref(nsplit),
+                                                          ctypes.byref(min_run)))
+            if len(self._plans) > 4096:
+                self._plans.clear()
+            plan = self._plans[(count, kv_len, skewed, hkv, window)] = (nsplit.value, min_run.value)
+        return plan
+
     def mfma_attention_supported(self, hq: int, hkv: int, d: int) -> bool:
         return bool(self.lib.psamd_attention_mfma_supports(hq, hkv, d))
 
@@ -338,36 +321,28 @@ class HipOps:
             if ctx.num_prefill_tiles:
                 kv_len = self.fixed_kv_len or ctx.max_kv_len
                 # Few query tiles on a long context: the kernel deals their keys out to several
-                # workgroups, whose partial results pass through these buffers. They are asked
-                # for at the largest size such a step can need, so they never grow.
+                # workgroups, whose partial results pass through these buffers. They are kept at
+                # the most rows any step of this shape can need (the library says how many), so
+                # they never grow.
                 nsplit = self.lib.psamd_attention_prefill_nsplit(ctx.num_prefill_tiles, kv_len, hq, hkv, d)
-                part_o = part_ml = None
+                rows = self.lib.psamd_attention_prefill_part_rows(hq, hkv, d)
+                part_o = self.ws.get("attn.prefill_part_o", (rows * hq * d,), torch.float32)
+                part_ml = self.ws.get("attn.prefill_part_ml", (rows * hq * 2,), torch.float32)
                 if nsplit > 1:
-                    rows = 32 * (512 // (hkv * (-(-(hq // hkv) // 4))))
                     self._need(32 * ctx.num_prefill_tiles * nsplit <= rows, "attention: more split tiles than planned for")
-                    part_o = self.ws.get("attn.prefill_part_o", (rows * hq * d,), torch.float32).data_ptr()
-                    part_ml = self.ws.get("attn.prefill_part_ml", (rows * hq * 2,), torch.float32).data_ptr()
                 self._ok(self.lib.psamd_attention_prefill(
                     s, qkv.data_ptr(), stride, out.data_ptr(), kv.data_ptr(), ctx.pf_tiles.data_ptr(),
                     ctx.num_prefill_tiles, kv_len,
                     ctx.item_start.data_ptr(), ctx.item_pos0.data_ptr(),
-                    g.table_off.data_ptr(), g.block_ids.data_ptr(), hq, hkv, d, scale, win, part_o, part_ml, nsplit))
+                    g.table_off.data_ptr(), g.block_ids.data_ptr(), hq, hkv, d, scale, win,
+                    part_o.data_ptr() if nsplit > 1 else None, part_ml.data_ptr() if nsplit > 1 else None, nsplit))
             if ctx.num_decode:
                 kv_len = self.fixed_kv_len or ctx.max_kv_len
-                if win:
-                    kv_len = min(kv_len, win)
-                # Two workgroups per compute unit; from one per compute unit on, no split (and no
-                # merge kernel): 32 requests x 8 kv heads at head size 128: 48 -> 41 us.
-                pairs = ctx.num_decode * hkv
-                nsplit = 1 if pairs >= 256 else max(1, min(64, 512 // pairs, -(-kv_len // 128)))
-                min_run = 128
-                if (self.fixed_skew if self.fixed_kv_len else ctx.decode_skewed) and not win:
-                    # One context far longer than the others: runs of 1,024 keys, as many as the
-                    # longest needs; the short requests use one or two and leave the rest empty.
-                    nsplit, min_run = max(nsplit, min(64, 4096 // ctx.num_decode, -(-kv_len // 1024))), 1024
-                # (requests x splits) is at most 512 / hkv unless there are more requests than
-                # that: asked for at that size, the buffers do not grow from step to step.
-                parts = max(ctx.num_decode * nsplit, 512 // hkv)
+                skewed = self.fixed_skew if self.fixed_kv_len else ctx.decode_skewed
+                nsplit, min_run = self.decode_plan(ctx.num_decode, kv_len, skewed, hkv, win)
+                # Room for the (request, run) pairs of any plan: asked for once, never grown.
+                parts = self.lib.psamd_attention_decode_max_parts(ctx.num_decode)
+                self._need(ctx.num_decode * nsplit <= parts, "attention: more (request, run) pairs than planned for")
                 part_o = self.ws.get("attn.part_o", (parts * hq * d,), torch.float32)
                 part_ml = self.ws.get("attn.part_ml", (parts * hq * 2,), torch.float32)
                 self._ok(self.lib.psamd_attention_decode(

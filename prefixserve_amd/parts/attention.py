@@ -79,17 +79,6 @@ class PagedAttention(Mixer):
     def weight_bytes(self) -> int:
         return sum(w.numel() * w.element_size() for w in (self.w_qkv, self.w_o))
 
-    def product_weights(self) -> list[torch.Tensor]:
-        return [self.w_qkv, self.w_o]
-
-    def activation_bytes(self, tokens: int, itemsize: int) -> int:
-        # q/k/v, the attention output, the projected output (or its float32 partial sums).
-        # ... and what the attention kernels pass between the workgroups that share a query's keys:
-        # the runs of a prompt portion's tiles, and up to 4,096 (request, run) pairs of single tokens.
-        split_rows = 32 * (512 // (self.num_kv_heads * -(-(self.num_heads // self.num_kv_heads) // 4))) + 4096
-        return tokens * ((self.q_size + 2 * self.kv_size) + self.q_size) * itemsize + 8 * 64 * self.hidden_size * 4 \
-            + tokens * self.hidden_size * itemsize + split_rows * self.num_heads * (self.head_dim + 2) * 4
-
     def forward(self, x: torch.Tensor, ctx: "StepContext", cache: Any, state: torch.Tensor | None,
                 writes_cache: bool) -> torch.Tensor:
         rt, ops, ws = self.rt, self.rt.ops, self.rt.workspace

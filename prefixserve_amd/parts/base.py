@@ -119,17 +119,6 @@ class Part:
         """Bytes of weights a step reads from this part (for roofline accounting)."""
         return 0
 
-    def product_weights(self) -> list[torch.Tensor]:
-        """The [out, in] matrices this part multiplies every token of a step by (for a runner
-        that lets the product library time its algorithms for them before the first request)."""
-        return []
-
-    def activation_bytes(self, tokens: int, itemsize: int) -> int:
-        """Bytes of buffers this part asks the workspace for in a step of ``tokens`` tokens with
-        activations of ``itemsize`` bytes. The cache pools are sized from what is free after the
-        largest step's buffers; a part that keeps large buffers and does not say so here may
-        leave too little for them."""
-        return 0
 
 
 class Norm(Part):
@@ -178,7 +167,13 @@ class Mixer(Part):
         """x [T, hidden] (activation dtype) -> what is to be added to the residual: [T, hidden]
         in the activation dtype, or [S, T, hidden] float32 slices whose sum it is (what
         ``ops.linear_to_residual`` returns). ``cache`` is this run's ``LayerCache`` (pages of its group) or None; ``state`` is
-        ``[num_slots, *shape]`` or None, indexed by ``ctx.slots``."""
+        ``[num_slots, *shape]`` or None, indexed by ``ctx.slots``.
+
+        Who clears a slot: the runner does. Before a step runs, every state tensor's rows for
+        the items that start at position 0 are set to zero on the stream, so a request (new, or
+        sent back by the scheduler and starting over) always meets zeros, whoever held the slot
+        before. A mixer only reads and updates its rows; a state whose neutral value is not
+        zero must be stored as the difference from it."""
         raise NotImplementedError
 
 

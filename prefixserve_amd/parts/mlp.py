@@ -38,13 +38,6 @@ class SwiGLU(FeedForward):
     def weight_bytes(self) -> int:
         return sum(w.numel() * w.element_size() for w in (self.w_gate_up, self.w_down))
 
-    def product_weights(self) -> list[torch.Tensor]:
-        return [self.w_gate_up, self.w_down]
-
-    def activation_bytes(self, tokens: int, itemsize: int) -> int:
-        # gate and up side by side (large steps), their product, the projected output.
-        return tokens * (3 * self.intermediate_size + self.hidden_size) * itemsize + 8 * 64 * self.hidden_size * 4
-
     def forward(self, x: torch.Tensor, ctx: "StepContext") -> torch.Tensor:
         rt, ops, ws = self.rt, self.rt.ops, self.rt.workspace
         t = x.shape[0]

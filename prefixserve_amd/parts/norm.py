@@ -32,9 +32,6 @@ class RMSNorm(Norm):
     def weight_bytes(self) -> int:
         return self.weight.numel() * self.weight.element_size()
 
-    def activation_bytes(self, tokens: int, itemsize: int) -> int:
-        return tokens * self.hidden_size * itemsize
-
     def add_norm(self, residual: torch.Tensor, delta: torch.Tensor | None, out_name: str) -> torch.Tensor:
         rt = self.rt
         out = rt.workspace.get(out_name, (residual.shape[0], self.hidden_size), rt.dtype)

@@ -36,11 +36,13 @@ class CacheWriteWatch:
         engine.runner.step = step
 
 
-def logit_errors(trace, prompts, outs, plain) -> list[float]:
+def logit_errors(trace, prompts, outs, plain, traced_rows_only: bool = False) -> list[float]:
     """Every row of an engine's ``logit_trace`` against the plain model run over the tokens the
     engine itself produced (so each row is judged given the same tokens before it, whatever
     the engine sampled): per row, max |difference| / max |truth|. Requests are "req-<index>".
-    Rows a round of decode steps computed past a request's last token are skipped."""
+    Rows a round of decode steps computed past a request's last token are skipped.
+    ``traced_rows_only``: the plain model's logits at the traced positions only (a large
+    vocabulary times every position of a long prompt is most of the work otherwise)."""
     import numpy as np
 
     truth = {}
@@ -48,9 +50,38 @@ def logit_errors(trace, prompts, outs, plain) -> list[float]:
     for rid, pos, row in trace:
         i = int(rid.split("-")[1])
         if i not in truth:
-            truth[i] = plain.logits(list(prompts[i]) + list(outs[i].tokens[:-1]))
-        if pos >= len(truth[i]):
+            seq = list(prompts[i]) + list(outs[i].tokens[:-1])
+            if traced_rows_only:
+                places = sorted({p for r, p, _ in trace if r == rid and p < len(seq)})
+                truth[i] = dict(zip(places, plain.logits_at(seq, places)))
+            else:
+                truth[i] = dict(enumerate(plain.logits(seq)))
+        if pos not in truth[i]:
             continue
         want = truth[i][pos]
         errors.append(float(np.abs(row.numpy() - want).max() / np.abs(want).max()))
     return errors
+
+
+def plain_bf16_bars(model_dir, plain, reqs=None, truth=None, vocab=None) -> tuple[float, float]:
+    """(mean row error, bar for a single row) of bfloat16 logits for the model in ``model_dir``:
+    a plain run of it with every result rounded to bfloat16 against ``plain`` (the same model in
+    float64), over ``reqs`` (whose float64 logits may be given as ``truth``) or over four random
+    sequences of 130 tokens. The bar for a row is BF16_ROW_FACTOR x that run's worst row: how far
+    8-bit rounding moves a row is the model's property, and the engine may do no worse than a
+    plain implementation does."""
+    import numpy as np
+
+    from configs import BF16_ROW_FACTOR
+    from plain.llama_plain import PlainLlama
+
+    rough = PlainLlama(model_dir, bf16=True, weights=plain.w)
+    if reqs is None:
+        rng = np.random.default_rng(77)
+        reqs = [rng.integers(0, vocab, 130).tolist() for _ in range(4)]
+    rows = []
+    for i, toks in enumerate(reqs):
+        want = truth[i] if truth is not None else plain.logits(toks)
+        rows.append(np.abs(rough.logits(toks) - want).max(-1) / np.abs(want).max(-1))
+    rows = np.concatenate(rows)
+    return float(rows.mean()), BF16_ROW_FACTOR * float(rows.max())

@@ -32,4 +32,9 @@ TINY = {
 
 # Relative to max|logit| of the compared rows.
 TOL_F32 = 1e-4      # the reference's bar for its exact tier (tests/test_llama_exact.py:42)
-TOL_BF16 = 4e-2     # bfloat16 keeps 8 bits: 2^-8 per rounding, a few tens of roundings deep
+# bfloat16 keeps 8 bits: 2^-8 per rounding, a few tens of roundings deep. How far that moves a
+# row of logits is a property of the model, so a row is held to BF16_ROW_FACTOR x the worst row
+# of a plain bfloat16 run of the same model over the same or as many tokens (conftest's
+# bf16_row_bar and checks.plain_bf16_bars; the worst rows of plain models of random
+# configurations lie between 2.5e-2 and 7.5e-2), and the mean to that run's mean.
+BF16_ROW_FACTOR = 1.5

@@ -243,17 +243,32 @@ def test_a_state_keeping_mixer_through_the_scheduler(tmp_path):
         assert np.argmax(rows, -1).tolist() == o.tokens, f"request {i}"
 
 
-def test_activation_bytes_come_from_the_parts(model_dirs, tmp_path):
-    """The pool is sized from what the parts say their buffers take, not from parameter
-    names: a part with other names is counted too."""
+def test_a_state_slot_is_cleared_by_the_runner_not_by_the_mixer(tmp_path):
+    """The toy mixer never resets its state. Every slot is filled with junk, as a slot's last
+    owner leaves it; a request that starts at position 0 must still give its whole-sequence
+    logits, first in a fresh slot and then in the slot another request has just given back."""
     from toy_parts import write_toy_mean_model
 
-    runner = make_runner(model_dirs["A"])
-    cfg = TINY["A"]
-    per_layer = runner._activation_bytes(1000) - runner._activation_bytes(0)
-    assert per_layer >= 1000 * 4 * (3 * cfg["intermediate_size"] + 4 * cfg["hidden_size"])
-    toy = make_runner(write_toy_mean_model(tmp_path))
-    assert toy._activation_bytes(1000) - toy._activation_bytes(0) >= 1000 * 4 * (3 * 96 + 4 * 64)
+    runner = make_runner(write_toy_mean_model(tmp_path), num_blocks=32, max_seq_len=128)
+    rng = np.random.default_rng(6)
+    a, b = rng.integers(0, 100, 40).tolist(), rng.integers(0, 100, 25).tolist()
+    clean = TraceReplayer(make_runner(tmp_path, num_blocks=32, max_seq_len=128))
+    want_a = clean.run_step({"step": 0, "entries": [{"id": "a", "tokens": a, "want": list(range(40))}], "end": ["a"]})
+    want_b = TraceReplayer(make_runner(tmp_path, num_blocks=32, max_seq_len=128)).run_step(
+        {"step": 0, "entries": [{"id": "b", "tokens": b, "want": list(range(25))}], "end": ["b"]})
+    for state in runner.states.values():
+        state.fill_(123.0)
+    rp = TraceReplayer(runner)
+    got_a = np.concatenate([
+        rp.run_step({"step": 0, "entries": [{"id": "a", "tokens": a[:13], "want": list(range(13))}], "end": []}),
+        rp.run_step({"step": 1, "entries": [{"id": "a", "tokens": a[13:], "want": list(range(27))}], "end": ["a"]})])
+    slot_a = 0 if not rp.live else None
+    got_b = rp.run_step({"step": 2, "entries": [{"id": "b", "tokens": b, "want": list(range(25))}], "end": ["b"]})
+    assert slot_a == 0 and rp.cache.slots.num_free == 8
+    assert np.abs(got_a - want_a).max() <= 1e-5 * np.abs(want_a).max()
+    assert np.abs(got_b - want_b).max() <= 1e-5 * np.abs(want_b).max()
+    # the slots nobody started in still hold the junk
+    assert sum(float(s[-1].abs().max()) == 123.0 for s in runner.states.values()) == len(runner.states)
 
 
 # ------------------------------------------------------------- faults switched on

@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 
 from checks import CacheWriteWatch, logit_errors
-from configs import TINY, TOL_BF16
+from configs import TINY
 
 pytestmark = pytest.mark.gpu
 ROOT = Path(__file__).resolve().parent.parent
@@ -48,7 +48,7 @@ def test_greedy_generation_equals_plain_in_float32(name, model_dirs, plain_model
 
 
 @pytest.mark.parametrize("name", ["A", "B", "C"])
-def test_bfloat16_through_the_scheduler_under_pressure(name, model_dirs, plain_models, plain_bf16_error):
+def test_bfloat16_through_the_scheduler_under_pressure(name, model_dirs, plain_models, plain_bf16_error, bf16_row_bar):
     """The same schedule in bfloat16: portions under a budget of 24, a shared prefix found in
     the cache, eviction, requests sent back and recomputed. Judged by the logits of every
     sampling step, given the tokens the engine produced: each row within the bfloat16 bar and
@@ -69,12 +69,12 @@ def test_bfloat16_through_the_scheduler_under_pressure(name, model_dirs, plain_m
     assert all(len(o.tokens) == 16 for o in outs)
     errors = logit_errors(eng.logit_trace, prompts, outs, plain_models[name])
     assert len(errors) >= 4 * 16
-    assert max(errors) < TOL_BF16 and np.mean(errors) <= plain_bf16_error[name], (max(errors), np.mean(errors))
+    assert max(errors) < bf16_row_bar[name] and np.mean(errors) <= plain_bf16_error[name], (max(errors), np.mean(errors))
     assert sched.cache.num_free(0) + sched.stats().cached_blocks == 11
 
 
 @pytest.mark.parametrize("name", ["B", "C"])
-def test_bfloat16_decode_rounds_through_graphs_after_warm_up(name, model_dirs, plain_models, plain_bf16_error):
+def test_bfloat16_decode_rounds_through_graphs_after_warm_up(name, model_dirs, plain_models, plain_bf16_error, bf16_row_bar):
     """The path the benchmark times: bfloat16, warm_up, eight decode steps per scheduler round
     replayed as graphs with the sampled token fed on the device, batches filled up to the
     captured sizes. Judged by the logits of every step."""
@@ -92,10 +92,10 @@ def test_bfloat16_decode_rounds_through_graphs_after_warm_up(name, model_dirs, p
     assert set(eng.runner._graphs) == captured and all(len(o.tokens) == 40 for o in outs)
     errors = logit_errors(eng.logit_trace, prompts, outs, plain_models[name])
     assert len(errors) >= 7 * 40
-    assert max(errors) < TOL_BF16 and np.mean(errors) <= plain_bf16_error[name], (max(errors), np.mean(errors))
+    assert max(errors) < bf16_row_bar[name] and np.mean(errors) <= plain_bf16_error[name], (max(errors), np.mean(errors))
 
 
-def test_greedy_generation_in_bfloat16_is_close_at_every_step(model_dirs, plain_models, plain_bf16_error):
+def test_greedy_generation_in_bfloat16_is_close_at_every_step(model_dirs, plain_models, plain_bf16_error, bf16_row_bar):
     """Free-running bfloat16 may choose another token than the plain model at a near-tie, so
     the run is judged by its logits: every row the engine sampled from against the plain
     model given the same tokens, and a token that differs from the plain model's choice only
@@ -109,11 +109,11 @@ def test_greedy_generation_in_bfloat16_is_close_at_every_step(model_dirs, plain_
     eng.logit_trace = []
     outs, _ = generate(eng, prompts, 16, ignore_eos=True)
     errors = logit_errors(eng.logit_trace, prompts, outs, plain_models[name])
-    assert len(errors) == 32 and max(errors) < TOL_BF16 and np.mean(errors) <= plain_bf16_error[name]
+    assert len(errors) == 32 and max(errors) < bf16_row_bar[name] and np.mean(errors) <= plain_bf16_error[name]
     for p, o in zip(prompts, outs):
         truth = plain_models[name].logits(p + o.tokens[:-1])[len(p) - 1:]
         for row, tok in zip(truth, o.tokens):
-            assert row.max() - row[tok] < 2 * TOL_BF16 * np.abs(row).max(), "left the plain model at a clear margin"
+            assert row.max() - row[tok] < 2 * bf16_row_bar[name] * np.abs(row).max(), "left the plain model at a clear margin"
 
 
 def test_temperature_sampling_survives_preemption(model_dirs):
@@ -152,12 +152,21 @@ def test_command_line(model_dirs, plain_models, tmp_path):
 def test_pool_is_sized_from_free_memory(model_dirs):
     from prefixserve_amd import Engine, EngineConfig
 
+    import gc
+
+    import torch
+
     eng = Engine(EngineConfig(model_path=model_dirs["A"], dtype="bfloat16", max_seq_len=512, reserve_bytes=200 << 30))
     assert eng.num_blocks > 10_000
+    free = torch.cuda.mem_get_info("cuda:0")[0]
+    assert (200 << 30) - (64 << 20) <= free <= (200 << 30) + (64 << 20), "the reserve is what stays free"
+    del eng
+    gc.collect()
+    torch.cuda.empty_cache()
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_a_hundred_requests_decode_together(dtype, model_dirs, plain_models, plain_bf16_error):
+def test_a_hundred_requests_decode_together(dtype, model_dirs, plain_models, plain_bf16_error, bf16_row_bar):
     """More decoding requests in one step than the small-step kernels take (64): the step falls
     back to the general product and the decode attention runs over 100 block tables."""
     from prefixserve_amd import Engine, EngineConfig, generate
@@ -184,7 +193,7 @@ def test_a_hundred_requests_decode_together(dtype, model_dirs, plain_models, pla
         for p, o in list(zip(prompts, outs))[::7]:
             assert o.tokens == plain_models[name].greedy(p, 10)[0]
     else:
-        assert max(errors) < TOL_BF16 and np.mean(errors) <= plain_bf16_error[name], (max(errors), np.mean(errors))
+        assert max(errors) < bf16_row_bar[name] and np.mean(errors) <= plain_bf16_error[name], (max(errors), np.mean(errors))
 
 
 def test_several_decode_steps_before_the_host_reads(model_dirs, plain_models):

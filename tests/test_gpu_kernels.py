@@ -290,32 +290,6 @@ def test_linear_bf16_other_paths(ops, m, n, k):
         assert rel(out, x.double() @ w.double().T) < (2e-5 if out_dtype == torch.float32 else 5e-3)
 
 
-def test_library_product_with_a_timed_algorithm(ops):
-    """The library times its algorithms for a shape (three matrices in turn) and keeps the
-    fastest, also for row counts within a quarter of the timed one: the products by what it
-    kept agree with float64, and what it kept is no slower than what it started from."""
-    assert ops._direct_library, "hipBLASLt was not found in the process"
-    n, k = 1000, 520
-    ws = [rnd(n, k, dtype=torch.bfloat16, seed=5 + i, scale=0.1) for i in range(3)]
-    res = ops.tune_linear(300, ws)
-    if res is None:
-        pytest.skip("this copy of hipBLASLt has no extension interface")
-    before, after = res
-    assert 0 < after <= before
-    for m in (300, 330, 250, 100):                    # the timed count, two neighbours, one too far to borrow
-        x = rnd(m, k, dtype=torch.bfloat16, seed=m)
-        for w in ws[:2]:
-            out = torch.full((m + 1, n), 7.0, dtype=torch.bfloat16, device=DEV)
-            ops.linear(x, w, out[:m])
-            assert rel(out[:m], x.double() @ w.double().T) < 5e-3 and torch.all(out[m] == 7.0)
-    assert ops.tune_linear(32, ws) is None            # small steps do not go to the library
-    assert ops.lib.psamd_gemm_lt_untune(1, 300, n, k) == 0
-    x = rnd(300, k, dtype=torch.bfloat16, seed=1)
-    out = torch.empty(300, n, dtype=torch.bfloat16, device=DEV)
-    ops.linear(x, ws[0], out)
-    assert rel(out, x.double() @ ws[0].double().T) < 5e-3
-
-
 def test_library_product_called_directly_and_through_torch(ops):
     """Large bfloat16 products go to hipBLASLt through the kernel library's own call (plans kept
     per shape); torch.mm is what remains if the library cannot be found. Both against float64,
@@ -381,7 +355,8 @@ def paged_case(ops, act, hq, hkv, d, lens_new, lens_old, window=None, seed=0, nu
     which stands in for them in the packed table, belongs to nobody and holds ``poison`` too."""
     rng = np.random.default_rng(seed)
     perm = [b for b in rng.permutation(num_blocks).tolist() if not (give_back and b == 0)]
-    pk = StepPacker(torch.device(DEV), [GroupMeta(num_blocks, window)], 10, 100000, 8, ops.PREFILL_TILE_Q)
+    pk = StepPacker(torch.device(DEV), [GroupMeta(num_blocks, window)], 10, 100000, 8, ops.PREFILL_TILE_Q,
+                    skew_rule=ops.decode_is_skewed)
     kv = torch.full((num_blocks, 2, hkv, 16 * d), poison, dtype=act, device=DEV)
     items, full = [], []
     for i, (n, old) in enumerate(zip(lens_new, lens_old)):
@@ -470,7 +445,9 @@ def test_decode_attention_of_many_requests(ops, hq, hkv, d, longest, window):
 def test_decode_attention_with_one_long_context_among_short_ones(ops, hq, hkv, d, short, longest):
     """One request's context is far longer than the others': the step counts as skewed and every
     request's keys are cut into runs of 1,024 or more, nine or more for the long request, one for
-    the short ones, whose other runs are empty. Slots nobody wrote hold NaN."""
+    the short ones, whose other runs are empty. Slots nobody wrote hold NaN. Every request is
+    judged by its own rows: the long request's output, an average over thousands of random
+    values, is a hundred times smaller than the short ones', and a common scale would hide it."""
     rng = np.random.default_rng(longest)
     old = rng.integers(0, 600, short).tolist()
     old.insert(short // 2, longest)
@@ -491,7 +468,75 @@ def test_decode_attention_with_one_long_context_among_short_ones(ops, hq, hkv, d
         StepPacker.pack = packed
     assert seen["skewed"]
     assert torch.isfinite(got.float()).all()
-    assert rel(got, want) < 2e-2
+    for i in range(len(old)):
+        assert rel(got[i], want[i]) < 2e-2, f"request {i} of {old[i]} keys"
+
+
+@pytest.mark.parametrize("hq,hkv,d,short,longest", [
+    (32, 8, 64, 31, 9000),
+    (16, 8, 128, 7, 12500),
+    (4, 1, 64, 15, 12000),
+])
+def test_skewed_decode_attention_finds_one_planted_key(ops, hq, hkv, d, short, longest):
+    """The long request of a skewed step, with one key made to match its query so strongly that
+    the output is that key's value: at the first and last key of the runs of 1,024 (or more)
+    that different workgroups take, at the very first and the very last key. A run that is
+    dropped, read twice or merged with the wrong weight cannot pass; the short requests, whose
+    later runs are empty, are compared one by one with their references."""
+    act = torch.bfloat16
+    group = hq // hkv
+    rng = np.random.default_rng(longest + 1)
+    old = rng.integers(0, 600, short).tolist()
+    long_at = short // 2
+    old.insert(long_at, longest)
+    n_req = len(old)
+    num_blocks = sum(-(-(o + 1) // 16) for o in old) + 8
+    perm = rng.permutation(num_blocks).tolist()
+    tables = [[perm.pop() for _ in range(-(-(o + 1) // 16))] for o in old]
+    ks = [rnd(o + 1, hkv, d, dtype=act, seed=100 + i, scale=0.05) for i, o in enumerate(old)]
+    vs = [rnd(o + 1, hkv, d, dtype=act, seed=200 + i) for i, o in enumerate(old)]
+    qkv = rnd(n_req, (hq + 2 * hkv) * d, dtype=act, seed=3, scale=0.05)
+    pk = StepPacker(torch.device(DEV), [GroupMeta(num_blocks)], 10, 100000, 64, ops.PREFILL_TILE_Q,
+                    skew_rule=ops.decode_is_skewed)
+    items = [StepItem(i, [1], o, [t], slot=i) for i, (o, t) in enumerate(zip(old, tables))]
+    nsplit, min_run = ops.decode_plan(n_req, longest + 1, True, hkv, 0)
+    assert min_run == 1024 and nsplit >= 9
+    run = -(-(-(-(longest + 1) // 32)) // nsplit) * 32            # keys per run: whole 32-key tiles
+    run = max(run, min_run)
+    plants = sorted({0, 1023, 1024, 2047, 2048, longest, longest - 1} |
+                    {p + e for p in range(run, longest, run) for e in (-1, 0)})
+    kv = torch.full((num_blocks, 2, hkv, 16 * d), float("nan"), dtype=act, device=DEV)
+    kp, vp = kv[:, 0].view(num_blocks, hkv, 16, d), kv[:, 1].view(num_blocks, hkv, d, 16)
+    for i, (o, t) in enumerate(zip(old, tables)):
+        pos = torch.arange(o + 1)
+        pg = torch.tensor(t)[pos // 16].to(DEV)
+        kp[pg, :, (pos % 16).to(DEV), :] = ks[i]
+        vp[pg, :, :, (pos % 16).to(DEV)] = vs[i]
+    scale = 50.0
+    want_short = {}
+    for i in range(n_req):
+        if i == long_at:
+            continue
+        q = qkv[i, : hq * d].view(hq, d).double()
+        sc = torch.einsum("hd,mhd->hm", q, ks[i].double().repeat_interleave(group, 1)) * scale
+        want_short[i] = torch.einsum("hm,mhd->hd", torch.softmax(sc, -1), vs[i].double().repeat_interleave(group, 1))
+    for far in plants:
+        page, off = tables[long_at][far // 16], far % 16
+        kept = kp[page, :, off, :].clone()
+        for h in range(hkv):
+            q = qkv[long_at, h * group * d: h * group * d + d]
+            kp[page, h, off, :] = 40.0 * q / q.float().norm()
+        ctx = pk.pack(items)
+        assert ctx.decode_skewed
+        out = torch.empty(n_req, hq * d, dtype=act, device=DEV)
+        ops.paged_attention(qkv, out, kv, ctx, 0, hq, hkv, d, scale, None)
+        kp[page, :, off, :] = kept
+        got = out.view(n_req, hq, d)
+        assert torch.isfinite(got.float()).all()
+        for h in range(hkv):
+            assert rel(got[long_at, h * group], vs[long_at][far, h]) < 2e-2, f"planted key {far} of {longest}, kv head {h}: not found"
+        for i, want in want_short.items():
+            assert rel(got[i], want) < 2e-2, f"short request {i} ({old[i]} keys) beside planted key {far}"
 
 
 @pytest.mark.parametrize("hq,hkv,d,new,old,window", [

@@ -16,13 +16,20 @@ import numpy as np
 import pytest
 
 import traces
-from configs import TINY, TOL_BF16, TOL_F32
+from checks import plain_bf16_bars
+from configs import TINY, TOL_F32
 from prefixserve_amd.engine.replay import TraceReplayer
 from prefixserve_amd.engine.runner import ModelRunner
 
 pytestmark = pytest.mark.gpu
 ROOT = Path(__file__).resolve().parent.parent
-TOL = {"float32": TOL_F32, "bfloat16": TOL_BF16}
+
+
+def tol(dtype, bf16_bar):
+    """The bar for one row: the reference's 1e-4 in 32-bit; in bfloat16 the model's own
+    (1.5 x the worst row of a plain bfloat16 run of it)."""
+    return TOL_F32 if dtype == "float32" else bf16_bar
+
 LENGTHS = [70, 33, 120, 97, 64, 18, 130, 45, 101, 77, 128, 90]
 
 
@@ -38,20 +45,21 @@ def runner_for(model_dir, dtype, num_blocks, graphs=True, max_seq_len=256):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B", "C"])
-def test_every_cutting_matches_the_plain_model(name, dtype, model_dirs, plain_models, plain_bf16_error):
+def test_every_cutting_matches_the_plain_model(name, dtype, model_dirs, plain_models, plain_bf16_error, bf16_row_bar):
     reqs = requests_for(name)
     truth = [plain_models[name].logits(t) for t in reqs]
     runner = runner_for(model_dirs[name], dtype, 64)
     worst, errors = {}, []
     for build in (traces.whole, traces.decode_tail, traces.portions):
         steps, expect = build(reqs)
-        worst[build.__name__] = traces.compare(TraceReplayer(runner).run_step, steps, expect, truth, TOL[dtype], errors)
+        worst[build.__name__] = traces.compare(TraceReplayer(runner).run_step, steps, expect, truth,
+                                               tol(dtype, bf16_row_bar[name]), errors)
     steps, expect, peak = traces.mixed(reqs, seed=3)
     assert sum(len(r) for r in reqs) > 1.5 * peak
     small = runner_for(model_dirs[name], dtype, peak // 16)
     small.pools.tensors[0].fill_(1e30)                              # a reused page never holds zeros
     rp = TraceReplayer(small)
-    worst["mixed"] = traces.compare(rp.run_step, steps, expect, truth, TOL[dtype], errors)
+    worst["mixed"] = traces.compare(rp.run_step, steps, expect, truth, tol(dtype, bf16_row_bar[name]), errors)
     assert rp.cache.num_free(0) == peak // 16
     print(name, dtype, {k: f"{v:.2e}" for k, v in worst.items()}, f"mean {np.mean(errors):.2e}")
     if dtype == "float32":
@@ -62,7 +70,7 @@ def test_every_cutting_matches_the_plain_model(name, dtype, model_dirs, plain_mo
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_cuttings_agree_with_each_other(dtype, model_dirs, plain_bf16_error):
+def test_cuttings_agree_with_each_other(dtype, model_dirs, plain_bf16_error, bf16_row_bar):
     """Whatever the distance to the plain model, the engine must agree with itself: the same
     position's logits from a whole prompt, from a decode step and from a mixed batch differ
     by rounding only, and in 32-bit not at all."""
@@ -78,10 +86,10 @@ def test_cuttings_agree_with_each_other(dtype, model_dirs, plain_bf16_error):
             for row, key in zip(out if out is not None else [], ex):
                 got[key] = row
         rows[build.__name__] = got
-    # Each cutting is within TOL of the plain model, so two cuttings are within 2 * TOL of each
+    # Each cutting is within the row bar of the plain model, so two cuttings are within twice that of each
     # other: the only bound that follows for the worst row. The typical row must agree at
     # least as well as a plain bfloat16 run agrees with the truth.
-    worst_tol = 1e-5 if dtype == "float32" else 2 * TOL_BF16
+    worst_tol = 1e-5 if dtype == "float32" else 2 * bf16_row_bar["C"]
     median_tol = 2e-6 if dtype == "float32" else plain_bf16_error["C"]
     errs = []
     for key, ref in rows["whole"].items():
@@ -165,17 +173,18 @@ def test_decoding_with_one_long_context_among_short_ones_through_graphs(tmp_path
             assert (16, 16, True) in runner._graphs
         return np.stack(rows)                       # [new, 16, vocab]
 
+    _mean, row_bar = plain_bf16_bars(tmp_path, plain, vocab=cfg["vocab_size"])
     graph = decode(True)
     for i in range(16):
         for k in range(new):
             want = truth[i][1 + k]
             err = float(np.abs(graph[k, i] - want).max() / np.abs(want).max())
-            assert err < TOL_BF16, f"request {i}, step {k}: {err:.2e}"
+            assert err < row_bar, f"request {i}, step {k}: {err:.2e}"
     apart = np.abs(decode(False) - graph).max(-1) / np.abs(graph).max(-1)
     assert apart.max() < 2.0 ** -7, f"graph and single steps {apart.max():.2e} apart"
 
 
-def test_graph_replay_with_library_products(model_dirs):
+def test_graph_replay_with_library_products(model_dirs, bf16_row_bar):
     """Seventy requests decoding together: more than 64 rows, so the products of the captured
     step are the library's (asked for algorithms without a workspace, which clear nothing with
     memset nodes). Every replay against the same step launched one by one, with other work
@@ -201,11 +210,11 @@ def test_graph_replay_with_library_products(model_dirs):
             assert any(shape[0] == n_req for shape in runner._graphs)
     scale = np.abs(out[False]).max(axis=-1)
     err = np.abs(out[False] - out[True]).max(axis=-1) / scale           # [steps, requests]
-    assert err.max() < TOL_BF16 and np.median(err) < 5e-3, f"worst {err.max():.3e} at step {int(err.max(axis=1).argmax())}"
+    assert err.max() < bf16_row_bar["C"] and np.median(err) < 5e-3, f"worst {err.max():.3e} at step {int(err.max(axis=1).argmax())}"
     assert err[-1].max() < 1.5 * max(err[0].max(), 1e-3)                 # replays do not drift apart
 
 
-def test_first_tokens_of_a_sequence(model_dirs, plain_models):
+def test_first_tokens_of_a_sequence(model_dirs, plain_models, bf16_row_bar):
     """Positions 0, 1, 2: a single key, no rotation at position 0."""
     for dtype in ("float32", "bfloat16"):
         runner = runner_for(model_dirs["B"], dtype, 8)
@@ -214,10 +223,10 @@ def test_first_tokens_of_a_sequence(model_dirs, plain_models):
         truth = plain_models["B"].logits(toks)
         for p in range(3):
             got = rp.run_step({"step": p, "entries": [{"id": "a", "tokens": [toks[p]], "want": [0]}], "end": []})
-            assert np.abs(got[0] - truth[p]).max() / np.abs(truth[p]).max() < TOL[dtype]
+            assert np.abs(got[0] - truth[p]).max() / np.abs(truth[p]).max() < tol(dtype, bf16_row_bar["B"])
 
 
-def test_long_decoding(model_dirs, plain_models):
+def test_long_decoding(model_dirs, plain_models, bf16_row_bar):
     """Three hundred tokens one by one after a short prompt, crossing many pages, with the
     graph path; compared at every position."""
     toks = requests_for("A", [330], seed=12)[0]
@@ -230,11 +239,11 @@ def test_long_decoding(model_dirs, plain_models):
         for p in range(10, 330):
             got = rp.run_step({"step": p, "entries": [{"id": "a", "tokens": [toks[p]], "want": [0]}], "end": []})
             worst = max(worst, float(np.abs(got[0] - truth[p]).max() / np.abs(truth[p]).max()))
-        assert worst < TOL[dtype], f"{dtype}: {worst:.3e}"
+        assert worst < tol(dtype, bf16_row_bar["A"]), f"{dtype}: {worst:.3e}"
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_trace_run_program(dtype, model_dirs, plain_models, tmp_path):
+def test_trace_run_program(dtype, model_dirs, plain_models, tmp_path, bf16_row_bar):
     """bin/trace_run as a user runs it: JSON lines in, <step>.f32 files and 'done <step>' out."""
     name = "B"
     reqs = requests_for(name, LENGTHS[:8])
@@ -256,7 +265,7 @@ def test_trace_run_program(dtype, model_dirs, plain_models, tmp_path):
                 got = np.fromfile(path, dtype="<f4").reshape(len(ex), -1)
                 for row, (i, p) in zip(got, ex):
                     err = np.abs(row - truth[i][p]).max() / np.abs(truth[i][p]).max()
-                    assert err < TOL[dtype], f"step {st['step']} request {i} position {p}: {err:.3e}"
+                    assert err < tol(dtype, bf16_row_bar[name]), f"step {st['step']} request {i} position {p}: {err:.3e}"
             else:
                 assert not path.exists()
         proc.stdin.close()
@@ -264,6 +273,33 @@ def test_trace_run_program(dtype, model_dirs, plain_models, tmp_path):
     finally:
         if proc.poll() is None:
             proc.kill()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_gpu_comparisons_catch_a_fault_that_is_switched_on(dtype, model_dirs, plain_models, bf16_row_bar):
+    """What the comparisons on this page are worth on the compiled kernels: the reference's own
+    switchable fault (prefixserve/llama_engine.py:192, ``rope_relative``: positions restart at 0
+    in every portion; checked there by tests/test_llama_exact.py:227-241) is switched on in the
+    step's integers on the device. Whole prompts are still right; every cutting must fail."""
+    name = "B"
+    reqs = requests_for(name, [70, 33, 97])
+    truth = [plain_models[name].logits(t) for t in reqs]
+    runner = runner_for(model_dirs[name], dtype, 64)
+    inner = runner.packer.pack
+
+    def pack(items, **kw):
+        ctx = inner(items, **kw)
+        ctx.positions -= ctx.item_pos0[ctx.tok_item.long()]
+        return ctx
+
+    runner.packer.pack = pack
+    bar = tol(dtype, bf16_row_bar[name])
+    steps, expect = traces.whole(reqs)
+    traces.compare(TraceReplayer(runner).run_step, steps, expect, truth, bar)
+    for build in (traces.decode_tail, traces.portions):
+        steps, expect = build(reqs)
+        with pytest.raises(AssertionError, match="relative error"):
+            traces.compare(TraceReplayer(runner).run_step, steps, expect, truth, bar)
 
 
 def _random_config(rng):
@@ -298,11 +334,15 @@ WIDE = dict(architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=6
             rms_norm_eps=1e-5, rope_theta=500000.0, max_position_embeddings=512, tie_word_embeddings=True)
 
 
-@pytest.mark.parametrize("seed", [0, 1, 2, 3, 4, 5, 6, 7, "awkward", "wide"])
+@pytest.mark.parametrize("seed", [0, 1, 2, 3, 4, 5, 6, 7, "awkward", "wide", "deep-309", "deep-311"])
 def test_random_configurations_in_both_dtypes(seed, tmp_path):
     """``awkward``: a width and an inner width that are no multiples of 8 (no 16-byte rows: the
     vectorized kernels and the small-step products must refuse and the general ones run), a
-    head size without a matrix-core kernel, an odd vocabulary. ``wide``: see above."""
+    head size without a matrix-core kernel, an odd vocabulary. ``wide``: see above. ``deep-N``:
+    two drawn configurations whose plain bfloat16 run has rows 7e-2 off (three layers, logits
+    that nearly cancel): a fixed bar of 4e-2 for a row failed them by one row in a hundred runs
+    of random configurations while the mean error stayed at 0.6 of the plain run's, which is
+    why a row is held to the plain bfloat16 run's own worst row and not to a constant."""
     from configs import INIT_STD
     from plain.llama_plain import PlainLlama
     from prefixserve_amd.weights import write_random_model
@@ -311,6 +351,10 @@ def test_random_configurations_in_both_dtypes(seed, tmp_path):
         rng, cfg, seed = np.random.default_rng(999), dict(AWKWARD), 99
     elif seed == "wide":
         rng, cfg, seed = np.random.default_rng(998), dict(WIDE), 98
+    elif isinstance(seed, str):
+        seed = int(seed.split("-")[1])
+        rng = np.random.default_rng(5000 + seed)
+        cfg = _random_config(rng)
     else:
         rng = np.random.default_rng(1000 + seed)
         cfg = _random_config(rng)
@@ -318,21 +362,20 @@ def test_random_configurations_in_both_dtypes(seed, tmp_path):
     plain = PlainLlama(tmp_path)
     reqs = [rng.integers(0, cfg["vocab_size"], n).tolist() for n in (75, 40, 97, 18, 66)]
     truth = [plain.logits(t) for t in reqs]
-    rough = PlainLlama(tmp_path, bf16=True).logits(reqs[0])
-    yardstick = float(np.mean(np.abs(rough - truth[0]).max(-1) / np.abs(truth[0]).max(-1)))
+    yardstick, row_bar = plain_bf16_bars(tmp_path, plain, reqs, truth)
     for dtype in ("float32", "bfloat16"):
         runner = runner_for(tmp_path, dtype, 32)
         errors = []
         for build in (traces.decode_tail, traces.portions):
             steps, expect = build(reqs)
-            traces.compare(TraceReplayer(runner).run_step, steps, expect, truth, TOL[dtype], errors)
+            traces.compare(TraceReplayer(runner).run_step, steps, expect, truth, tol(dtype, row_bar), errors)
         steps, expect, peak = traces.mixed(reqs, seed=seed)
         small = runner_for(tmp_path, dtype, peak // 16)
         small.pools.tensors[0].fill_(1e30)
-        worst = traces.compare(TraceReplayer(small).run_step, steps, expect, truth, TOL[dtype], errors)
+        worst = traces.compare(TraceReplayer(small).run_step, steps, expect, truth, tol(dtype, row_bar), errors)
         print(seed, dtype, {k: cfg[k] for k in ("hidden_size", "num_attention_heads", "num_key_value_heads", "head_dim")},
-              f"worst {worst:.2e} mean {np.mean(errors):.2e} (plain bf16 {yardstick:.2e})")
+              f"worst {worst:.2e} mean {np.mean(errors):.2e} (plain bf16: mean {yardstick:.2e}, row bar {row_bar:.2e})")
         if dtype == "float32":
             assert max(errors) < 2e-5
         else:
-            assert np.mean(errors) <= 1.5 * yardstick, f"{np.mean(errors):.3e} > 1.5 x {yardstick:.3e}"
+            assert np.mean(errors) <= yardstick, f"{np.mean(errors):.3e} > {yardstick:.3e}"

@@ -299,6 +299,43 @@ def test_norm_weights_matter(plain_models, model_dirs):
     assert np.abs(nw - 1).max() > 0.05
 
 
+def test_the_final_norm_stands_in_front_of_the_output_matrix(plain_models, model_dirs, tmp_path):
+    """logits = head . (norm.weight * h / rms(h)) (prefixserve/model/llama.py:123-126). A model
+    whose final norm weight is zero gives zero logits; doubling the weight doubles them; and a
+    last hidden state scaled by 1,000 gives the same logits, because the norm divides the scale
+    out. A ``logits()`` that skips the norm, applies it after the product or leaves out its
+    weight fails one of the three."""
+    import shutil
+
+    from safetensors.numpy import save_file
+
+    name = "B"
+    toks = np.random.default_rng(3).integers(0, 512, 20).tolist()
+    base = plain_models[name].logits(toks)
+    w = P.read_safetensors(model_dirs[name] / "model.safetensors")
+
+    def variant(folder, **changed):
+        folder.mkdir()
+        shutil.copy(model_dirs[name] / "config.json", folder / "config.json")
+        save_file({k: np.ascontiguousarray(changed.get(k, v), dtype=np.float32) for k, v in w.items()},
+                  str(folder / "model.safetensors"))
+        return P.PlainLlama(folder)
+
+    zero = variant(tmp_path / "zero", **{"model.norm.weight": np.zeros_like(w["model.norm.weight"])})
+    assert np.abs(base).max() > 0.1 and np.array_equal(zero.logits(toks), np.zeros_like(base))
+    twice = variant(tmp_path / "twice", **{"model.norm.weight": 2.0 * w["model.norm.weight"]})
+    assert np.allclose(twice.logits(toks), 2.0 * base, rtol=1e-12, atol=0)
+    # Scale what the last layer adds to the residual stream: its down projection. With a tiny
+    # eps the norm removes almost all of it; a product without the norm would grow with it.
+    plain = plain_models[name]
+    h = plain.hidden(toks)
+    head = plain.w["lm_head.weight"]
+    by_hand = P.rms_norm(h, plain.w["model.norm.weight"], plain.cfg.eps) @ head.T
+    assert np.allclose(base, by_hand, rtol=1e-12, atol=1e-12)
+    assert np.allclose(P.rms_norm(1000.0 * h, plain.w["model.norm.weight"], plain.cfg.eps) @ head.T, base, rtol=1e-6)
+    assert not np.allclose(h @ head.T, base, rtol=0.05, atol=0.05 * np.abs(base).max())
+
+
 def test_bf16_reader_is_exact():
     from safetensors.torch import save_file
     import tempfile, os

@@ -19,7 +19,8 @@ TOY_MEAN_CONFIG = {"architectures": ["ToyMeanForCausalLM"], "hidden_size": 64, "
 
 
 class RunningMean(Mixer):
-    """out_t = W . mean(x_0..x_t); the state is (sum [hidden], count [1]) per request."""
+    """out_t = W . mean(x_0..x_t); the state is (sum [hidden], count [1]) per request. It never
+    clears its slot: the runner hands a request that starts at position 0 a zeroed one."""
 
     def __init__(self, hidden_size, positions, name):
         self.h, self.name = hidden_size, name
@@ -34,17 +35,12 @@ class RunningMean(Mixer):
         super().bind(tensors, rt)
         self.w = rt.ops.prepare_matrix(tensors[self.name], rt)
 
-    def activation_bytes(self, tokens, itemsize):
-        return 2 * tokens * self.h * itemsize
-
     def forward(self, x, ctx, cache, state, writes_cache):
         assert cache is None and state is not None
         out = self.rt.workspace.get("toy.mean", tuple(x.shape), x.dtype)
         starts = ctx.host["item_start"].tolist()
         for i in range(ctx.num_items):
             slot = int(ctx.host["slots"][i])
-            if int(ctx.host["item_pos0"][i]) == 0:
-                state[slot].zero_()                               # a new request starts from nothing
             seg = x[starts[i]:starts[i + 1]].float()
             sums = state[slot, : self.h] + torch.cumsum(seg, 0)
             counts = state[slot, self.h] + torch.arange(1, seg.shape[0] + 1, device=x.device)
