@@ -8,6 +8,7 @@ and trace replay (prefixserve/llama_engine.py:75-150 of the reference is the cou
 
 from __future__ import annotations
 
+import gc
 import logging
 from pathlib import Path
 from typing import Any, Sequence
@@ -154,6 +155,7 @@ class ModelRunner:
             state.zero_()
         self.pools = None
         self.model.attach({}, self.states)
+        gc.collect()
         torch.cuda.empty_cache()             # the throwaway pool goes back to the device; the step's buffers are in use
         free, _total = torch.cuda.mem_get_info(self.device)
         usable = free - reserve_bytes
