@@ -59,6 +59,20 @@ int psamd_qkv_rope_append(void* stream, const void* x, const void* w, void* qkv_
                           int head_dim, const int32_t* positions, const float* table, void* kv,
                           const int32_t* write_slot);
 
+// Small steps without a norm kernel and without partial slices to add up (bfloat16, M <= 16):
+// the products that feed the residual stream add into it (psamd_linear_skinny_add: float atomics,
+// K split over workgroups; the order of the additions differs from run to run), and the products
+// that read the normalized stream (q/k/v, gate/up, the output matrix) take rows of the float32
+// residual and apply the RMS norm themselves (weight norm_w, bfloat16 or float32; statistics in
+// 32-bit, eps inside the root). psamd_normed_supports: whether they take M tokens of width K.
+int psamd_normed_supports(int M, int K);
+int psamd_linear_skinny_add(void* stream, const void* x, const void* w, float* out, int M, int n_out, int K);
+int psamd_linear_normed(void* stream, const float* resid, const int32_t* rows, const void* norm_w, int norm_w_dtype,
+                        float eps, const void* w, void* out, int out_dtype, int M, int n_out, int K, int epilogue);
+int psamd_qkv_rope_append_normed(void* stream, const float* resid, const void* norm_w, int norm_w_dtype, float eps,
+                                 const void* w, void* qkv_out, int M, int K, int hq, int hkv, int head_dim,
+                                 const int32_t* positions, const float* table, void* kv, const int32_t* write_slot);
+
 int psamd_attention_generic(void* stream, const void* qkv, int q_stride, void* out, const void* kv, int act_dtype,
                             int64_t tokens, const int32_t* positions, const int32_t* tok_item,
                             const int32_t* table_off, const int32_t* block_ids, int hq, int hkv, int head_dim,

@@ -143,6 +143,12 @@ __device__ __forceinline__ bf16x8 zero8() {
 
 __device__ __forceinline__ float silu_f(float g) { return g / (1.f + __expf(-g)); }
 
+// *p += v, done by the memory side, nothing returned: the way K-slices of different workgroups,
+// on any die, add into one float32 sum.
+__device__ __forceinline__ void add_to(float* p, float v) { (void)unsafeAtomicAdd(p, v); }
+template <typename T>
+__device__ __forceinline__ void add_to(T*, float) {}
+
 // Streams rows of w through v_mfma_f32_16x16x32_bf16 with the M tokens as the other operand.
 // Two ways to lay the work over a workgroup's 4 waves:
 //  * SPLIT (few output columns): the workgroup owns 16 rows of w and a range of K; its waves
@@ -166,7 +172,11 @@ __device__ __forceinline__ float silu_f(float g) { return g / (1.f + __expf(-g))
 // U = k-steps whose loads are in flight together.
 constexpr int skinny_depth(int mt, int rt) { return mt == 1 ? 8 : (mt * rt <= 2 ? 4 : (mt * rt <= 8 ? 2 : 1)); }
 
-template <int MT, int RT, int WV, bool SWIGLU, bool SPLIT, typename TO, int U = skinny_depth(MT, RT)>
+// ATOMIC (float32 output, plain epilogue): every K-slice adds its partial sums into the one
+// out[M][n_out] with float atomics that return nothing, instead of writing a slice of its own:
+// out is the residual stream, and no kernel has to add the slices up afterwards. The order of
+// the additions, and with it the last bit of the sums, differs from run to run.
+template <int MT, int RT, int WV, bool SWIGLU, bool SPLIT, typename TO, int U = skinny_depth(MT, RT), bool ATOMIC = false>
 __global__ __launch_bounds__(64 * WV) void skinny_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                           TO* __restrict__ out, int M, int n_out, int K) {
   constexpr int NACC = SWIGLU ? 2 * MT : MT;
@@ -261,11 +271,13 @@ __global__ __launch_bounds__(64 * WV) void skinny_mfma_kernel(const bf16_t* __re
     }
     const int m = mt * 16 + r;
     if (m >= M) return;
-    TO* dst = out + (static_cast<int64_t>(blockIdx.y) * M + m) * n_out;
+    TO* dst = out + (static_cast<int64_t>(ATOMIC ? 0 : blockIdx.y) * M + m) * n_out;
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
       const int n = (tile0 + rt) * 16 + 4 * g + v;
-      if (n < n_out) dst[n] = from_float<TO>(sum[v]);
+      if (n >= n_out) continue;
+      if constexpr (ATOMIC) add_to(dst + n, sum[v]);
+      else dst[n] = from_float<TO>(sum[v]);
     }
   };
 
@@ -299,6 +311,87 @@ __global__ __launch_bounds__(64 * WV) void skinny_mfma_kernel(const bf16_t* __re
   }
 }
 
+// Where the tokens of a small step come from: bfloat16 rows x[M][K], or (x == nullptr) rows of the
+// float32 residual stream that the kernel normalizes itself on the way in (RMS norm: statistics
+// in 32-bit, eps inside the root, times the norm's weight), row rows[m] for token m (rows ==
+// nullptr: row m). A kernel that reads its tokens this way needs no norm kernel in front of it.
+struct Tokens {
+  const bf16_t* x;
+  const float* resid;
+  const void* norm_w;
+  const int32_t* rows;
+  float eps;
+  int norm_w_bf16;      // the norm's weight is bfloat16 (else float32)
+};
+
+// Stages the M <= ROWS tokens of a small step in LDS for a workgroup of WV waves, from rows of
+// the float32 residual stream: xs[row][k] = bfloat16(resid[row][k] * norm_w[k]), and the rows'
+// sums of squares, from which stage_scale() gives 1 / sqrt(mean(resid[row]^2) + eps) once a
+// barrier has passed. The caller multiplies its sums by that (the product is linear in the tokens,
+// so a row's scale may wait until the end). With few tokens a row is dealt out to several waves
+// (8 for one token, 4 for two, 2 up to four), so that a single token's row is not one wave's
+// work while seven wait; each leaves its part of the row's sum in ss[row][part]. Rows from M on
+// are zeros. K must be a multiple of 8.
+template <int WV>
+__device__ __forceinline__ int stage_waves_per_row(int M) {
+  return M <= 1 ? WV : (M <= 2 ? WV / 2 : (M <= 4 ? WV / 4 : 1));
+}
+
+template <int ROWS, int WV>
+__device__ __forceinline__ void stage_normed(const Tokens& tk, bf16_t* xs, int XS, float* ss, int M, int K, int wave,
+                                             int lane) {
+  const int wpr = stage_waves_per_row<WV>(M);
+  const int pieces = K >> 3;                               // 8 elements each
+  for (int i = threadIdx.x; i < (ROWS - M) * pieces; i += 64 * WV) {
+    const int row = M + i / pieces, c = i - (row - M) * pieces;
+    *reinterpret_cast<bf16x8*>(xs + row * XS + 8 * c) = zero8();
+  }
+  const int per_part = (pieces + wpr - 1) / wpr;
+  for (int job = wave; job < ROWS * wpr; job += WV) {
+    const int row = job / wpr, part = job - row * wpr;
+    if (row >= M) break;
+    bf16_t* dst = xs + row * XS;
+    const float* src = tk.resid + static_cast<int64_t>(tk.rows != nullptr ? tk.rows[row] : row) * K;
+    const int c_end = min(pieces, (part + 1) * per_part);
+    float sum = 0.f;
+#pragma unroll 4
+    for (int c = part * per_part + lane; c < c_end; c += 64) {
+      const float4 a = *reinterpret_cast<const float4*>(src + 8 * c);
+      const float4 b = *reinterpret_cast<const float4*>(src + 8 * c + 4);
+      float wn[8];
+      if (tk.norm_w_bf16) {
+        const bf16x8 wv = load8(static_cast<const bf16_t*>(tk.norm_w) + 8 * c);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) wn[i] = static_cast<float>(wv[i]);
+      } else {
+        const float4 w0 = *reinterpret_cast<const float4*>(static_cast<const float*>(tk.norm_w) + 8 * c);
+        const float4 w1 = *reinterpret_cast<const float4*>(static_cast<const float*>(tk.norm_w) + 8 * c + 4);
+        wn[0] = w0.x, wn[1] = w0.y, wn[2] = w0.z, wn[3] = w0.w, wn[4] = w1.x, wn[5] = w1.y, wn[6] = w1.z, wn[7] = w1.w;
+      }
+      const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+      bf16x8 o;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        sum = fmaf(v[i], v[i], sum);
+        o[i] = static_cast<__bf16>(v[i] * wn[i]);
+      }
+      *reinterpret_cast<bf16x8*>(dst + 8 * c) = o;
+    }
+    sum = wave_sum(sum);
+    if (lane == 0) ss[row * WV + part] = sum;
+  }
+}
+
+// The scale of token `row` (after the barrier behind stage_normed).
+template <int WV>
+__device__ __forceinline__ float stage_scale(const Tokens& tk, const float* ss, int row, int M, int K) {
+  if (row >= M) return 0.f;
+  const int wpr = stage_waves_per_row<WV>(M);
+  float sum = 0.f;
+  for (int p = 0; p < wpr; ++p) sum += ss[row * WV + p];
+  return rsqrtf(sum / static_cast<float>(K) + tk.eps);
+}
+
 // Up to 16 tokens as workgroups that stay: each stages its tokens in LDS once (ROWS = 8 or 16
 // rows of its slice of K; in the kernel above every workgroup reads them again from L2 for its
 // one or two row tiles, as many bytes as the rows themselves at two tiles) and then takes groups
@@ -306,8 +399,11 @@ __global__ __launch_bounds__(64 * WV) void skinny_mfma_kernel(const bf16_t* __re
 // k-steps of all RT tiles in flight together; the partial sums meet in LDS and wave rt finishes
 // tile rt. gridDim.y slices of K give partial sums out[blockIdx.y][M][n_out], as above. SWIGLU:
 // w is [gate; up] and a group is RT pairs of tiles. K must be a multiple of 32.
-template <int RT, int ROWS, bool SWIGLU, typename TO>
-__global__ __launch_bounds__(512) void stream_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+// NORMED: the tokens are rows of the float32 residual stream, normalized while they are staged
+// (gridDim.y must be 1: a row's statistics need the whole row). ATOMIC: the K-slices add into one
+// out[M][n_out] (see skinny_mfma_kernel).
+template <int RT, int ROWS, bool SWIGLU, typename TO, bool NORMED = false, bool ATOMIC = false>
+__global__ __launch_bounds__(512) void stream_kernel(Tokens tk, const bf16_t* __restrict__ w,
                                                   TO* __restrict__ out, int M, int n_out, int K, int groups) {
   constexpr int WV = 8, U = 8, NACC = SWIGLU ? 2 : 1;
   extern __shared__ __align__(16) unsigned char stream_smem[];
@@ -318,11 +414,16 @@ __global__ __launch_bounds__(512) void stream_kernel(const bf16_t* __restrict__ 
   const int XS = per_slice * 32 + 8;                          // elements per token row in LDS (padded: rows on different banks)
   bf16_t* xs = reinterpret_cast<bf16_t*>(stream_smem);
   f32x4* red = reinterpret_cast<f32x4*>(stream_smem + static_cast<size_t>(ROWS) * XS * sizeof(bf16_t));   // [WV][RT][NACC][64]
+  float* ss = reinterpret_cast<float*>(red + WV * RT * NACC * 64);                                         // [ROWS][WV] (NORMED)
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
-  {
+  // (Asking for the first group's rows of w before or while the tokens are staged was measured
+  // and lost: the registers that hold them cost the second workgroup of a compute unit, or spill.)
+  if constexpr (NORMED) {
+    stage_normed<ROWS, WV>(tk, xs, XS, ss, M, K, wave, lane);
+  } else {
     const int pieces = steps * 4;                             // 16-byte pieces of a row's slice
-    const bf16_t* x0 = x + (static_cast<int64_t>(s_begin) << 5);
+    const bf16_t* x0 = tk.x + (static_cast<int64_t>(s_begin) << 5);
     for (int p = threadIdx.x; p < ROWS * pieces; p += blockDim.x) {
       const int row = p / pieces, c = p - row * pieces;
       bf16x8 v = zero8();
@@ -334,6 +435,7 @@ __global__ __launch_bounds__(512) void stream_kernel(const bf16_t* __restrict__ 
   // With ROWS = 8, lanes 8..15 of a group repeat tokens 0..7: their columns of the result are not stored.
   const bf16_t* xl = xs + (r % ROWS) * XS + 8 * g;
   const bf16_t* w0 = w + (static_cast<int64_t>(s_begin) << 5) + 8 * g;
+  const float row_scale = NORMED ? stage_scale<WV>(tk, ss, r % ROWS, M, K) : 1.f;
   for (int grp = blockIdx.x; grp < groups; grp += gridDim.x) {
     const int tile0 = grp * RT;
     const bf16_t* wrow[RT];
@@ -381,19 +483,23 @@ __global__ __launch_bounds__(512) void stream_kernel(const bf16_t* __restrict__ 
       f32x4 sum = red[(rt * NACC) * 64 + lane];
 #pragma unroll
       for (int w2 = 1; w2 < WV; ++w2) sum += red[((w2 * RT + rt) * NACC) * 64 + lane];
+      if (NORMED) sum *= row_scale;
       if (SWIGLU) {
         f32x4 up = red[(rt * NACC + 1) * 64 + lane];
 #pragma unroll
         for (int w2 = 1; w2 < WV; ++w2) up += red[((w2 * RT + rt) * NACC + 1) * 64 + lane];
+        if (NORMED) up *= row_scale;
 #pragma unroll
         for (int v = 0; v < 4; ++v) sum[v] = silu_f(sum[v]) * up[v];
       }
       if (r < M) {
-        TO* dst = out + (static_cast<int64_t>(blockIdx.y) * M + r) * n_out;
+        TO* dst = out + (static_cast<int64_t>(ATOMIC ? 0 : blockIdx.y) * M + r) * n_out;
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
           const int n = (tile0 + rt) * 16 + 4 * g + v;
-          if (n < n_out) dst[n] = from_float<TO>(sum[v]);
+          if (n >= n_out) continue;
+          if constexpr (ATOMIC) add_to(dst + n, sum[v]);
+          else dst[n] = from_float<TO>(sum[v]);
         }
       }
     }
@@ -404,18 +510,20 @@ __global__ __launch_bounds__(512) void stream_kernel(const bf16_t* __restrict__ 
 // Bytes of LDS stream_kernel needs.
 static size_t stream_smem_bytes(int rt, int rows, bool swiglu, int K, int ksplit) {
   const int per_slice = static_cast<int>(ceil_div(K >> 5, ksplit));
-  return static_cast<size_t>(rows) * (per_slice * 32 + 8) * sizeof(bf16_t) + sizeof(f32x4) * 8 * rt * (swiglu ? 2 : 1) * 64;
+  return static_cast<size_t>(rows) * (per_slice * 32 + 8) * sizeof(bf16_t) + sizeof(f32x4) * 8 * rt * (swiglu ? 2 : 1) * 64 +
+         sizeof(float) * rows * 8;
 }
 
+static Tokens plain_tokens(const void* x) { return Tokens{static_cast<const bf16_t*>(x), nullptr, nullptr, nullptr, 0.f, 0}; }
+
 // workgroups: how many may stay per K-slice; the groups are dealt out evenly over them.
-template <int RT, int ROWS, bool SWIGLU>
-static int launch_stream(hipStream_t s, const void* x, const void* w, void* out, int out_dtype, int M, int n_out, int K,
+template <int RT, int ROWS, bool SWIGLU, bool NORMED = false, bool ATOMIC = false>
+static int launch_stream(hipStream_t s, const Tokens& tk, const void* w, void* out, int out_dtype, int M, int n_out, int K,
                          int ksplit, int workgroups) {
   const int groups = static_cast<int>(ceil_div(ceil_div(n_out, 16), RT));
   const size_t smem = stream_smem_bytes(RT, ROWS, SWIGLU, K, ksplit);
   const int rounds = static_cast<int>(ceil_div(groups, workgroups));
   const dim3 grid(static_cast<unsigned>(ceil_div(groups, rounds)), static_cast<unsigned>(ksplit)), block(512);
-  const bf16_t* xp = static_cast<const bf16_t*>(x);
   const bf16_t* wp = static_cast<const bf16_t*>(w);
   auto run = [&](auto kernel, auto* dst) {
     if (smem > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -423,11 +531,15 @@ static int launch_stream(hipStream_t s, const void* x, const void* w, void* out,
       set_error("psamd_linear_skinny: " + std::to_string(smem) + " bytes of LDS were refused");
       return -1;
     }
-    kernel<<<grid, block, smem, s>>>(xp, wp, dst, M, n_out, K, groups);
+    kernel<<<grid, block, smem, s>>>(tk, wp, dst, M, n_out, K, groups);
     return check_launch("psamd_linear_skinny");
   };
-  if (SWIGLU || out_dtype == kBF16) return run(stream_kernel<RT, ROWS, SWIGLU, bf16_t>, static_cast<bf16_t*>(out));
-  return run(stream_kernel<RT, ROWS, false, float>, static_cast<float*>(out));
+  if constexpr (ATOMIC) {
+    return run(stream_kernel<RT, ROWS, false, float, NORMED, true>, static_cast<float*>(out));
+  } else {
+    if (SWIGLU || out_dtype == kBF16) return run(stream_kernel<RT, ROWS, SWIGLU, bf16_t, NORMED>, static_cast<bf16_t*>(out));
+    return run(stream_kernel<RT, ROWS, false, float, NORMED>, static_cast<float*>(out));
+  }
 }
 
 template <int MT, int RT, int WV, bool SWIGLU, bool SPLIT>
@@ -480,11 +592,11 @@ static int launch_skinny1(hipStream_t s, const void* x, const void* w, void* out
       const bool small = static_cast<int64_t>(rows) * K <= 8 * 2048;
       if (stream_smem_bytes(small ? 2 : 1, rows, false, K, 1) <= 160 * 1024) {
         if (rows == 8) {
-          if (small) return launch_stream<2, 8, false>(s, x, w, out, out_dtype, M, n_out, K, 1, 512);
-          return launch_stream<1, 8, false>(s, x, w, out, out_dtype, M, n_out, K, 1, 1024);
+          if (small) return launch_stream<2, 8, false>(s, plain_tokens(x), w, out, out_dtype, M, n_out, K, 1, 512);
+          return launch_stream<1, 8, false>(s, plain_tokens(x), w, out, out_dtype, M, n_out, K, 1, 1024);
         }
-        if (small) return launch_stream<2, 16, false>(s, x, w, out, out_dtype, M, n_out, K, 1, 512);
-        return launch_stream<1, 16, false>(s, x, w, out, out_dtype, M, n_out, K, 1, 1024);
+        if (small) return launch_stream<2, 16, false>(s, plain_tokens(x), w, out, out_dtype, M, n_out, K, 1, 512);
+        return launch_stream<1, 16, false>(s, plain_tokens(x), w, out, out_dtype, M, n_out, K, 1, 1024);
       }
     }
     if (M <= 8 && ksplit == 1 && ceil_div(n_out, 16) >= 2048) {
@@ -553,12 +665,12 @@ static int launch_skinny1(hipStream_t s, const void* x, const void* w, void* out
       if constexpr (!SWIGLU) {
         const int wgs = ksplit > 1 ? 512 / ksplit : 0;
         if (wgs > 0 && groups >= 2 * wgs && stream_smem_bytes(1, 16, false, K, ksplit) <= 160 * 1024) {
-          if (M <= 8) return launch_stream<1, 8, false>(s, x, w, out, out_dtype, M, n_out, K, ksplit, wgs);
-          return launch_stream<1, 16, false>(s, x, w, out, out_dtype, M, n_out, K, ksplit, wgs);
+          if (M <= 8) return launch_stream<1, 8, false>(s, plain_tokens(x), w, out, out_dtype, M, n_out, K, ksplit, wgs);
+          return launch_stream<1, 16, false>(s, plain_tokens(x), w, out, out_dtype, M, n_out, K, ksplit, wgs);
         }
       } else {
         if (M <= 8 && ksplit == 1 && K >= 4096 && groups >= 768 && stream_smem_bytes(1, 8, true, K, 1) <= 160 * 1024)
-          return launch_stream<1, 8, true>(s, x, w, out, out_dtype, M, n_out, K, 1, 256);
+          return launch_stream<1, 8, true>(s, plain_tokens(x), w, out, out_dtype, M, n_out, K, 1, 256);
       }
     }
   }
@@ -585,12 +697,19 @@ static int launch_skinny(hipStream_t s, const void* x, const void* w, void* out,
 // qkv_out[m] receives the rotated q and k and v (the layout the attention kernels read q
 // from); k and v also go to page slot write_slot[m] when a cache is given.
 // RT such tiles per workgroup and WV waves, as in skinny_mfma_kernel.
-template <int MT, int RT, int WV>
+// ROWS > 0 (MT == 1, K a multiple of 32): the tokens are ROWS rows of the float32 residual stream,
+// normalized and staged in LDS once per workgroup as in stream_kernel; the matrix instructions
+// then read them from there.
+template <int MT, int RT, int WV, int ROWS = 0>
 __global__ __launch_bounds__(64 * WV) void qkv_rope_append_kernel(
-    const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, bf16_t* __restrict__ qkv_out, int M, int K, int hq,
+    Tokens tk, const bf16_t* __restrict__ w, bf16_t* __restrict__ qkv_out, int M, int K, int hq,
     int hkv, int d, const int32_t* __restrict__ positions, const float2* __restrict__ table,
     bf16_t* __restrict__ kv, const int32_t* __restrict__ write_slot) {
+  constexpr bool NORMED = ROWS > 0;
+  static_assert(!NORMED || MT == 1, "staged tokens: one tile of up to 16");
   __shared__ f32x4 red[WV][MT][64];
+  extern __shared__ __align__(16) unsigned char qkv_smem[];     // NORMED: xs[ROWS][K + 8] bfloat16, ss[ROWS][WV]
+  const bf16_t* x = tk.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
   const int half = d >> 1;
@@ -635,16 +754,38 @@ __global__ __launch_bounds__(64 * WV) void qkv_rope_append_kernel(
   }
   const int s_full = K >> 5;
   constexpr int U = MT == 1 ? 8 : (MT * RT <= 2 ? 4 : 2);   // steps whose loads are in flight together
+  const int XS = K + 8;
+  bf16_t* xs = reinterpret_cast<bf16_t*>(qkv_smem);
+  float* ss = reinterpret_cast<float*>(qkv_smem + static_cast<size_t>(NORMED ? ROWS : 0) * XS * sizeof(bf16_t));   // [ROWS][WV]
+  float row_scale = 1.f;
+  bf16x8 pre[RT][U];
+  if constexpr (NORMED) {
+    // The rows of w for the first k-steps are asked for before the tokens are staged: both trips
+    // to memory are then under way together (7.8 against 8.1 us at 8 tokens of the 1B shape).
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) pre[rt][u] = wave + WV * u < s_full ? load8(wrow[rt] + ((wave + WV * u) << 5)) : zero8();
+    stage_normed<ROWS, WV>(tk, xs, XS, ss, M, K, wave, lane);
+    __syncthreads();
+    row_scale = stage_scale<WV>(tk, ss, r % ROWS, M, K);
+  }
+  const bf16_t* xl = xs + (NORMED ? (r % ROWS) * XS + 8 * g : 0);
   for (int base = wave; base < s_full; base += WV * U) {
     bf16x8 a[RT][U], b[MT][U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int s = base + WV * u;
-      if (s < s_full) {
+      if (NORMED && base == wave) {
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) a[rt][u] = pre[rt][u];
+      } else if (s < s_full) {
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) a[rt][u] = load8(wrow[rt] + (s << 5));
+        if constexpr (!NORMED) {
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) b[mt][u] = load8(xrow[mt] + (s << 5));
+          for (int mt = 0; mt < MT; ++mt) b[mt][u] = load8(xrow[mt] + (s << 5));
+        }
       } else {
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) a[rt][u] = zero8();
@@ -653,14 +794,16 @@ __global__ __launch_bounds__(64 * WV) void qkv_rope_append_kernel(
       }
     }
 #pragma unroll
-    for (int u = 0; u < U; ++u)
+    for (int u = 0; u < U; ++u) {
+      if constexpr (NORMED) b[0][u] = *reinterpret_cast<const bf16x8*>(xl + (min(base + WV * u, s_full - 1) << 5));
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
           acc[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[rt][u], b[mt][u], acc[rt][mt], 0, 0, 0);
+    }
   }
-  if ((K & 31) != 0 && (s_full % WV) == wave) {
+  if (!NORMED && (K & 31) != 0 && (s_full % WV) == wave) {
     const int k = s_full << 5;
     const bool in = k + 8 * g < K;
 #pragma unroll
@@ -687,6 +830,7 @@ __global__ __launch_bounds__(64 * WV) void qkv_rope_append_kernel(
     f32x4 own = red[0][mt][lane];
 #pragma unroll
     for (int w2 = 1; w2 < WV; ++w2) own += red[w2][mt][lane];
+    if (NORMED) own *= row_scale;
     const int m = mt * 16 + r;
     const int mc = min(m, M - 1);
     const bool second = g >= 2;
@@ -731,13 +875,39 @@ template <int MT>
 static void launch_qkv(hipStream_t s, const bf16_t* x, const bf16_t* w, bf16_t* out, int M, int K, int hq, int hkv, int d,
                        const int32_t* positions, const float2* table, bf16_t* kv, const int32_t* write_slot) {
   const int n_tiles = (hq + 2 * hkv) * (d / 16);
+  const Tokens tk = plain_tokens(x);
   if (M > 8 && n_tiles >= 320) {
     qkv_rope_append_kernel<MT, 2, 8><<<dim3(static_cast<unsigned>(ceil_div(n_tiles, 2))), dim3(512), 0, s>>>(
-        x, w, out, M, K, hq, hkv, d, positions, table, kv, write_slot);
+        tk, w, out, M, K, hq, hkv, d, positions, table, kv, write_slot);
   } else {
     qkv_rope_append_kernel<MT, 1, 8><<<dim3(static_cast<unsigned>(n_tiles)), dim3(512), 0, s>>>(
-        x, w, out, M, K, hq, hkv, d, positions, table, kv, write_slot);
+        tk, w, out, M, K, hq, hkv, d, positions, table, kv, write_slot);
   }
+}
+
+// LDS the staged form needs beside the kernel's static array.
+static size_t qkv_staged_smem(int rows, int K) { return static_cast<size_t>(rows) * (K + 8) * sizeof(bf16_t) + sizeof(float) * rows * 8; }
+
+// Up to 16 tokens read from the residual stream and normalized in the kernel (K a multiple of 32).
+template <int RT, int ROWS>
+static int launch_qkv_normed(hipStream_t s, const Tokens& tk, const bf16_t* w, bf16_t* out, int M, int K, int hq, int hkv, int d,
+                             const int32_t* positions, const float2* table, bf16_t* kv, const int32_t* write_slot) {
+  const int n_tiles = (hq + 2 * hkv) * (d / 16);
+  const size_t smem = qkv_staged_smem(ROWS, K);
+  auto kernel = qkv_rope_append_kernel<1, RT, 8, ROWS>;
+  if (smem + sizeof(f32x4) * 8 * 64 > 64 * 1024 &&
+      hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                          static_cast<int>(smem)) != hipSuccess)
+    return fail("psamd_qkv_rope_append_normed: " + std::to_string(smem) + " bytes of LDS were refused");
+  kernel<<<dim3(static_cast<unsigned>(ceil_div(n_tiles, RT))), dim3(512), smem, s>>>(tk, w, out, M, K, hq, hkv, d, positions,
+                                                                                   table, kv, write_slot);
+  return check_launch("psamd_qkv_rope_append_normed");
+}
+
+// Whether the kernels that normalize their tokens themselves take a step of M tokens of width K:
+// up to 16 tokens, whole 32-wide k-steps, and the staged tokens fit in LDS beside the partial sums.
+static bool normed_ok(int M, int K) {
+  return M >= 1 && M <= 16 && K >= 32 && K % 32 == 0 && stream_smem_bytes(1, M <= 8 ? 8 : 16, true, K, 1) <= 160 * 1024;
 }
 
 }  // namespace psamd
@@ -832,6 +1002,87 @@ int psamd_qkv_rope_append(void* stream, const void* x, const void* w, void* qkv_
     default: launch_qkv<4>(s, xp, wp, op, M, K, hq, hkv, head_dim, positions, tab, kvp, write_slot); break;
   }
   return check_launch("psamd_qkv_rope_append");
+}
+
+// 1 if psamd_linear_normed and psamd_qkv_rope_append_normed take M tokens of width K.
+int psamd_normed_supports(int M, int K) { return normed_ok(M, K) ? 1 : 0; }
+
+// out[M, n_out] (float32, the residual stream) += x[M, K] * w[n_out, K]^T for M <= 16: K is split
+// over as many workgroups as fill the chip, and every slice adds its partial sums with float
+// atomics that return nothing. The order of the additions is not fixed: results differ in the
+// last bit from run to run.
+int psamd_linear_skinny_add(void* stream, const void* x, const void* w, float* out, int M, int n_out, int K) {
+  PSAMD_REQUIRE(M >= 1 && M <= 16, "M must be in [1, 16]");
+  PSAMD_REQUIRE(n_out > 0 && K > 0 && K % 8 == 0, "K must be a positive multiple of 8");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int ksplit = psamd_linear_skinny_ksplit(M, n_out, K);
+  const int64_t groups = ceil_div(n_out, 16);
+  const int wgs = ksplit > 1 ? 512 / ksplit : 0;
+  if (M >= 4 && K % 32 == 0 && wgs > 0 && groups >= 2 * wgs && stream_smem_bytes(1, 16, false, K, ksplit) <= 160 * 1024) {
+    if (M <= 8) return launch_stream<1, 8, false, false, true>(s, plain_tokens(x), w, out, kF32, M, n_out, K, ksplit, wgs);
+    return launch_stream<1, 16, false, false, true>(s, plain_tokens(x), w, out, kF32, M, n_out, K, ksplit, wgs);
+  }
+  const dim3 grid(static_cast<unsigned>(groups), static_cast<unsigned>(ksplit)), block(64 * 4);
+  skinny_mfma_kernel<1, 1, 4, false, true, float, 8, true><<<grid, block, 0, s>>>(
+      static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), out, M, n_out, K);
+  return check_launch("psamd_linear_skinny_add");
+}
+
+// out[M, n_out] = norm(resid[rows[m]]) * w^T for M <= 16 tokens, where norm is the RMS norm with
+// weight norm_w [K] (bfloat16 or float32) and eps, computed inside the kernel from the float32
+// residual rows (rows == NULL: row m). epilogue 0: out bfloat16 or float32; epilogue 1 (SwiGLU):
+// w = [gate; up] with n_out rows each, out = silu(gate) * up in bfloat16.
+int psamd_linear_normed(void* stream, const float* resid, const int32_t* rows, const void* norm_w, int norm_w_dtype,
+                        float eps, const void* w, void* out, int out_dtype, int M, int n_out, int K, int epilogue) {
+  PSAMD_REQUIRE(normed_ok(M, K), "M must be in [1, 16] and K a multiple of 32 that fits in LDS");
+  PSAMD_REQUIRE(n_out > 0 && (epilogue == 0 || epilogue == 1), "bad sizes");
+  PSAMD_REQUIRE(out_dtype == kBF16 || out_dtype == kF32, "output must be bfloat16 or float32");
+  PSAMD_REQUIRE(epilogue == 0 || out_dtype == kBF16, "the SwiGLU epilogue writes bfloat16");
+  PSAMD_REQUIRE(norm_w_dtype == kBF16 || norm_w_dtype == kF32, "the norm's weight is bfloat16 or float32");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const Tokens tk{nullptr, resid, norm_w, rows, eps, norm_w_dtype == kBF16 ? 1 : 0};
+  const int64_t groups = ceil_div(n_out, 16);
+  const bool eight = M <= 8;
+  if (epilogue == 1) {
+    // One pair of gate/up tiles per group; as many workgroups as give each one or two groups.
+    // 512 pairs of tiles (an intermediate size of 8,192) and up to 8 tokens: a workgroup per pair
+    // (17.9 us at 8 tokens against 19.0 with two pairs each); more tokens (the staged rows then
+    // leave a compute unit room for one workgroup) or more pairs: 256 workgroups that stay for two
+    // or more (16 tokens: 25.4 -> 21.1 us; 896 pairs at K = 4,096, 8 tokens: 56.4 -> 53.0).
+    const int wgs = (eight && groups < 768) ? 512 : 256;
+    if (eight) return launch_stream<1, 8, true, true>(s, tk, w, out, out_dtype, M, n_out, K, 1, wgs);
+    return launch_stream<1, 16, true, true>(s, tk, w, out, out_dtype, M, n_out, K, 1, wgs);
+  }
+  // Two row tiles per group while the staged tokens are small (two workgroups per compute unit).
+  const bool small = static_cast<int64_t>(eight ? 8 : 16) * K <= 8 * 2048 && groups >= 2048;
+  if (eight) {
+    if (small) return launch_stream<2, 8, false, true>(s, tk, w, out, out_dtype, M, n_out, K, 1, 512);
+    return launch_stream<1, 8, false, true>(s, tk, w, out, out_dtype, M, n_out, K, 1, 1024);
+  }
+  if (small) return launch_stream<2, 16, false, true>(s, tk, w, out, out_dtype, M, n_out, K, 1, 512);
+  return launch_stream<1, 16, false, true>(s, tk, w, out, out_dtype, M, n_out, K, 1, 1024);
+}
+
+// psamd_qkv_rope_append with the tokens read from the float32 residual stream and normalized in
+// the kernel (RMS norm with weight norm_w and eps), for M <= 16.
+int psamd_qkv_rope_append_normed(void* stream, const float* resid, const void* norm_w, int norm_w_dtype, float eps,
+                                 const void* w, void* qkv_out, int M, int K, int hq, int hkv, int head_dim,
+                                 const int32_t* positions, const float* table, void* kv, const int32_t* write_slot) {
+  PSAMD_REQUIRE(normed_ok(M, K), "M must be in [1, 16] and K a multiple of 32 that fits in LDS");
+  PSAMD_REQUIRE(hq > 0 && hkv > 0 && head_dim >= 16 && head_dim % 16 == 0, "head_dim must be a multiple of 16");
+  PSAMD_REQUIRE(positions != nullptr, "positions are needed");
+  PSAMD_REQUIRE(kv == nullptr || write_slot != nullptr, "a cache needs write slots");
+  PSAMD_REQUIRE(norm_w_dtype == kBF16 || norm_w_dtype == kF32, "the norm's weight is bfloat16 or float32");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const Tokens tk{nullptr, resid, norm_w, nullptr, eps, norm_w_dtype == kBF16 ? 1 : 0};
+  const bf16_t* wp = static_cast<const bf16_t*>(w);
+  bf16_t* op = static_cast<bf16_t*>(qkv_out);
+  const float2* tab = reinterpret_cast<const float2*>(table);
+  bf16_t* kvp = static_cast<bf16_t*>(kv);
+  const int n_tiles = (hq + 2 * hkv) * (head_dim / 16);
+  if (M <= 8) return launch_qkv_normed<1, 8>(s, tk, wp, op, M, K, hq, hkv, head_dim, positions, tab, kvp, write_slot);
+  if (n_tiles >= 320) return launch_qkv_normed<2, 16>(s, tk, wp, op, M, K, hq, hkv, head_dim, positions, tab, kvp, write_slot);
+  return launch_qkv_normed<1, 16>(s, tk, wp, op, M, K, hq, hkv, head_dim, positions, tab, kvp, write_slot);
 }
 
 }  // extern "C"

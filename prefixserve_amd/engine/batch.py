@@ -78,6 +78,9 @@ class StepContext:
     keys: list[Hashable]
     want_counts: list[int]
     host: dict[str, np.ndarray] = field(default_factory=dict)
+    # The step's residual stream (float32 [T, hidden]), set by the model before the layers run: a
+    # part may add its output into it itself instead of handing back what is to be added.
+    residual: Any = None
 
 
 class StepPacker:

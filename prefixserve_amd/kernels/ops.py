@@ -18,6 +18,7 @@ from typing import Any, Sequence
 import torch
 
 from prefixserve_amd.build import ensure_kernels
+from prefixserve_amd.parts.base import NormedRows
 
 _F32, _BF16 = 0, 1
 _vp, _i32, _i64, _f32 = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_float
@@ -51,6 +52,10 @@ _SIGNATURES = {
     "psamd_linear_skinny": [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32],
     "psamd_linear_skinny_ksplit": [_i32, _i32, _i32],
     "psamd_qkv_rope_append": [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp],
+    "psamd_normed_supports": [_i32, _i32],
+    "psamd_linear_skinny_add": [_vp, _vp, _vp, _vp, _i32, _i32, _i32],
+    "psamd_linear_normed": [_vp, _vp, _vp, _vp, _i32, _f32, _vp, _vp, _i32, _i32, _i32, _i32, _i32],
+    "psamd_qkv_rope_append_normed": [_vp, _vp, _vp, _i32, _f32, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp],
     "psamd_attention_generic": [_vp, _vp, _i32, _vp, _vp, _i32, _i64, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _f32, _i32],
     "psamd_attention_mfma_supports": [_i32, _i32, _i32],
     "psamd_attention_prefill_nsplit": [_i32, _i32, _i32, _i32, _i32],
@@ -88,6 +93,7 @@ class HipOps:
         self._sample_scratch: torch.Tensor | None = None
         self._step_stream: int | None = None
         self._plans: dict[tuple, tuple[int, int]] = {}
+        self._fuses: dict[tuple[int, int], bool] = {}
         self._slice_views: dict[tuple, tuple] = {}      # (name, slices, rows) -> (buffer, its [slices, rows, N] view)
         # The library for large bfloat16 products, called directly if it can be (it sets itself up
         # here, outside any capture); through torch.mm otherwise.
@@ -125,6 +131,38 @@ class HipOps:
     def _need(cond: bool, msg: str) -> None:
         if not cond:
             raise KernelError(msg)
+
+    def fuses_norm(self, count: int, width: int, dtype: torch.dtype) -> bool:
+        """Whether a bfloat16 step of ``count`` tokens of this width runs without norm kernels:
+        the products that read the normalized residual stream normalize its rows themselves
+        (``NormedRows`` for x), and ``linear_to_residual`` adds into the stream."""
+        if dtype != torch.bfloat16:
+            return False
+        key = (int(count), int(width))
+        ok = self._fuses.get(key)
+        if ok is None:
+            ok = self._fuses[key] = bool(self.lib.psamd_normed_supports(*key))
+        return ok
+
+    def normed(self, x: "torch.Tensor | NormedRows", name: str = "normed.x") -> torch.Tensor:
+        """x as a tensor: rows handed over with their norm still to be applied go through the
+        norm kernel now (for a consumer whose kernel does not normalize its tokens itself)."""
+        if not isinstance(x, NormedRows):
+            return x
+        out = self.ws.get(name, x.shape, x.dtype)
+        if x.rows is None:
+            self.add_rmsnorm(x.residual, None, x.weight, x.eps, out)
+        else:
+            self.add_rmsnorm_rows(x.residual, None, x.rows, x.weight, x.eps, out)
+        return out
+
+    def _normed_args(self, x: NormedRows, k: int) -> tuple:
+        self._need(x.residual.dtype == torch.float32 and x.residual.is_contiguous() and x.residual.shape[1] == k,
+                   "rows to normalize must be float32 [T, K]")
+        self._need(x.weight.numel() == k and x.weight.is_contiguous(), "the norm's weight must be [K]")
+        if x.rows is not None:
+            self._need(x.rows.dtype == torch.int32 and x.rows.is_contiguous(), "rows must be int32")
+        return x.residual.data_ptr(), _ptr(x.rows), x.weight.data_ptr(), _code(x.weight.dtype), float(x.eps)
 
     def prepare_matrix(self, w: torch.Tensor, rt: Any) -> torch.Tensor:
         """A weight matrix on the device in the activation dtype (bfloat16 values widen to
@@ -196,6 +234,24 @@ class HipOps:
         """qkv = x @ w_qkv^T, q and k rotated, k and v written to their pages. One kernel for a
         bfloat16 step of at most 64 tokens; otherwise the product followed by ``rope_kv_append``."""
         m, k = x.shape
+        if isinstance(x, NormedRows):
+            if (x.rows is None and d % 16 == 0 and qkv.dtype == torch.bfloat16 and self.fuses_norm(m, k, x.dtype)):
+                resid, _rows, nw, nw_code, eps = self._normed_args(x, k)
+                self._need(w_qkv.shape == ((hq + 2 * hkv) * d, k) and qkv.shape == (m, (hq + 2 * hkv) * d), "qkv: shapes")
+                self._need(w_qkv.is_contiguous() and qkv.is_contiguous() and w_qkv.dtype == torch.bfloat16, "qkv: operands")
+                self._need(positions.dtype == torch.int32 and positions.numel() == m, "qkv: positions")
+                if table is not None:
+                    self._need(table.dtype == torch.float32 and table.shape[1:] == (d // 2, 2) and table.is_contiguous(),
+                               "qkv: table must be float32 [positions, D/2, 2]")
+                if kv is not None:
+                    self._need(kv.dtype == qkv.dtype and kv.shape[1:] == (2, hkv, 16 * d) and kv.is_contiguous(),
+                               "qkv: cache must be [blocks, 2, kv_heads, 16*D] in the activation dtype")
+                    self._need(write_slot.dtype == torch.int32 and write_slot.numel() == m, "qkv: write slots")
+                self._ok(self.lib.psamd_qkv_rope_append_normed(
+                    self._stream(), resid, nw, nw_code, eps, w_qkv.data_ptr(), qkv.data_ptr(), m, k, hq, hkv, d,
+                    positions.data_ptr(), _ptr(table), _ptr(kv), None if kv is None else write_slot.data_ptr()))
+                return
+            x = self.normed(x)
         if (x.dtype == torch.bfloat16 and 0 < m <= self.SKINNY_MAX_ROWS and k % 8 == 0 and d % 16 == 0):
             self._need(w_qkv.shape == ((hq + 2 * hkv) * d, k) and qkv.shape == (m, (hq + 2 * hkv) * d), "qkv: shapes")
             self._need(x.is_contiguous() and w_qkv.is_contiguous() and qkv.is_contiguous(), "qkv: contiguous operands")
@@ -219,6 +275,14 @@ class HipOps:
     def linear(self, x, w, out) -> None:
         m, k = x.shape
         n = w.shape[0]
+        if isinstance(x, NormedRows):
+            if m > 0 and w.dtype == torch.bfloat16 and self.fuses_norm(m, k, x.dtype):
+                resid, rows, nw, nw_code, eps = self._normed_args(x, k)
+                self._need(w.shape[1] == k and out.shape == (m, n) and w.is_contiguous() and out.is_contiguous(), "linear: operands")
+                self._ok(self.lib.psamd_linear_normed(self._stream(), resid, rows, nw, nw_code, eps, w.data_ptr(), out.data_ptr(),
+                                                      _code(out.dtype), m, n, k, 0))
+                return
+            x = self.normed(x)
         self._need(w.shape[1] == k and out.shape == (m, n), f"linear: shapes {tuple(x.shape)} x {tuple(w.shape)}")
         self._need(x.is_contiguous() and w.is_contiguous() and out.is_contiguous(), "linear: contiguous operands")
         self._need(x.dtype == w.dtype, "linear: x and w must have one dtype")
@@ -244,13 +308,21 @@ class HipOps:
         self._ok(self.lib.psamd_linear(self._stream(), x.data_ptr(), _code(x.dtype), w.data_ptr(), _code(w.dtype),
                                        out.data_ptr(), _code(out.dtype), m, n, k))
 
-    def linear_to_residual(self, x, w, name: str) -> torch.Tensor:
+    def linear_to_residual(self, x, w, name: str, residual: torch.Tensor | None = None) -> torch.Tensor | None:
         """x @ w^T for a consumer that adds it to the residual stream (the fused add+norm).
         Returns [T, N] in the activation dtype or, for a small bfloat16 step whose product has
         few output columns, [S, T, N] float32 partial sums of a K-split, which the consumer adds
-        up: splitting K over workgroups is what lets such a product use the whole chip."""
+        up: splitting K over workgroups is what lets such a product use the whole chip. With the
+        stream itself given as ``residual`` (float32 [T, N]), a step small enough to run without
+        norm kernels adds the product into it here, K-slice by K-slice, and returns None."""
         m, k = x.shape
         n = w.shape[0]
+        if (residual is not None and 0 < m and x.dtype == torch.bfloat16 and k % 8 == 0 and residual.shape == (m, n)
+                and self.fuses_norm(m, n, x.dtype)):
+            self._need(residual.dtype == torch.float32 and residual.is_contiguous(), "the residual stream is float32")
+            self._need(w.shape[1] == k and x.is_contiguous() and w.is_contiguous(), "linear_to_residual: operands")
+            self._ok(self.lib.psamd_linear_skinny_add(self._stream(), x.data_ptr(), w.data_ptr(), residual.data_ptr(), m, n, k))
+            return None
         if x.dtype == torch.bfloat16 and k % 8 == 0 and 0 < m <= self.SKINNY_MAX_ROWS:
             ksplit = self.lib.psamd_linear_skinny_ksplit(m, n, k)
             if ksplit > 1:
@@ -275,6 +347,14 @@ class HipOps:
         self._need(w_gate_up.shape == (2 * inter, k) and out.shape[0] == m, "linear_swiglu: shapes")
         if m == 0:
             return
+        if isinstance(x, NormedRows):
+            if w_gate_up.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and self.fuses_norm(m, k, x.dtype):
+                resid, rows, nw, nw_code, eps = self._normed_args(x, k)
+                self._need(w_gate_up.is_contiguous() and out.is_contiguous(), "linear_swiglu: operands")
+                self._ok(self.lib.psamd_linear_normed(self._stream(), resid, rows, nw, nw_code, eps, w_gate_up.data_ptr(),
+                                                      out.data_ptr(), _BF16, m, inter, k, 1))
+                return
+            x = self.normed(x)
         if x.dtype == torch.bfloat16 and k % 8 == 0 and m <= self.SKINNY_MAX_ROWS:
             self._ok(self.lib.psamd_linear_skinny(self._stream(), x.data_ptr(), w_gate_up.data_ptr(), out.data_ptr(),
                                                   _BF16, m, inter, k, 1, 1))

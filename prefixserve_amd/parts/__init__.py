@@ -1,4 +1,4 @@
-from .base import (CacheNeed, FeedForward, Mixer, Norm, Part, PositionEncoding, RotaryTable, Runtime, StateNeed,
+from .base import (CacheNeed, FeedForward, Mixer, Norm, NormedRows, Part, PositionEncoding, RotaryTable, Runtime, StateNeed,
                    WeightWant, Workspace, make, register_block, register_feed_forward, register_mixer, register_norm,
                    register_position)
 from .model import DecoderModel

@@ -35,6 +35,8 @@ class PagedAttention(Mixer):
     q.k / sqrt(head_dim) unless ``scale`` is given; softmax in 32-bit
     (prefixserve/model/llama.py:113-117, prefixserve/model/attention.py:103-120)."""
 
+    takes_normed_rows = True
+
     def __init__(self, hidden_size: int, positions: Mapping[str, PositionEncoding], num_heads: int,
                  num_kv_heads: int, head_dim: int, names: Mapping[str, str], position: str | None = None,
                  window: int | None = None, scale: float | None = None) -> None:
@@ -90,7 +92,7 @@ class PagedAttention(Mixer):
         out = ws.get("attn.out", (t, self.q_size), rt.dtype)
         ops.paged_attention(qkv, out, cache.kv, ctx, cache.group, self.num_heads, self.num_kv_heads,
                             self.head_dim, self.scale, cache.window)
-        return ops.linear_to_residual(out, self.w_o, "attn.delta")
+        return ops.linear_to_residual(out, self.w_o, "attn.delta", getattr(ctx, "residual", None))
 
 
 register_mixer("paged_attention", PagedAttention)

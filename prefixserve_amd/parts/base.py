@@ -93,6 +93,26 @@ class Workspace:
 
 
 @dataclass
+class NormedRows:
+    """Rows of the residual stream with a norm still to be applied: what a norm hands to a
+    consumer whose kernel normalizes its tokens itself while it reads them, instead of a tensor a
+    norm kernel has written. ``rows`` (int32, on the device) selects rows of ``residual``; None
+    means all of them in order. A consumer that cannot take it asks ``ops.normed(x)`` for the
+    tensor."""
+
+    residual: torch.Tensor          # [T, hidden] float32
+    weight: torch.Tensor            # [hidden]
+    eps: float
+    dtype: torch.dtype              # the activation dtype the normalized rows stand for
+    rows: torch.Tensor | None = None
+
+    @property
+    def shape(self) -> tuple[int, int]:
+        n = self.rows.numel() if self.rows is not None else self.residual.shape[0]
+        return (int(n), int(self.residual.shape[1]))
+
+
+@dataclass
 class Runtime:
     """What every part needs to run: the device, the activation dtype (bfloat16 for
     serving, float32 for the exact path), the kernel bindings and the buffer store."""
@@ -124,14 +144,18 @@ class Part:
 class Norm(Part):
     """A normalisation fused with the residual sum that precedes it."""
 
-    def add_norm(self, residual: torch.Tensor, delta: torch.Tensor | None, out_name: str) -> torch.Tensor:
+    def add_norm(self, residual: torch.Tensor, delta: torch.Tensor | None, out_name: str,
+                 lazy: bool = False) -> "torch.Tensor | NormedRows":
         """residual (float32 [T,H], updated in place) += delta; returns norm(residual) in the
-        activation dtype. ``delta`` is [T,H] or [S,T,H] float32 slices to be summed. The sum and
-        the statistics are 32-bit."""
+        activation dtype. ``delta`` is [T,H] or [S,T,H] float32 slices to be summed, or None when
+        there is nothing to add (the first layer, or a sub-layer that added its output into the
+        residual stream itself). The sum and the statistics are 32-bit. ``lazy``: the caller's
+        consumer takes ``NormedRows``; the norm may then return that instead of running a kernel
+        (only when delta is None: a consumer normalizes, it does not add)."""
         raise NotImplementedError
 
     def add_norm_rows(self, residual: torch.Tensor, delta: torch.Tensor | None, rows: torch.Tensor,
-                      out_name: str) -> torch.Tensor:
+                      out_name: str, lazy: bool = False) -> "torch.Tensor | NormedRows":
         """The same for the selected rows only; ``residual`` is left as it is."""
         raise NotImplementedError
 
@@ -162,10 +186,15 @@ class Mixer(Part):
     def state_need(self) -> StateNeed | None:
         return None
 
+    # True: ``forward`` takes ``NormedRows`` for x (it hands x to kernels that normalize their
+    # tokens themselves); the block then lets the norm in front of it be lazy.
+    takes_normed_rows = False
+
     def forward(self, x: torch.Tensor, ctx: "StepContext", cache: Any, state: torch.Tensor | None,
-                writes_cache: bool) -> torch.Tensor:
+                writes_cache: bool) -> torch.Tensor | None:
         """x [T, hidden] (activation dtype) -> what is to be added to the residual: [T, hidden]
-        in the activation dtype, or [S, T, hidden] float32 slices whose sum it is (what
+        in the activation dtype, or [S, T, hidden] float32 slices whose sum it is, or None if the
+        part has added its output into ``ctx.residual`` itself (the three things
         ``ops.linear_to_residual`` returns). ``cache`` is this run's ``LayerCache`` (pages of its group) or None; ``state`` is
         ``[num_slots, *shape]`` or None, indexed by ``ctx.slots``.
 
@@ -180,7 +209,10 @@ class Mixer(Part):
 class FeedForward(Part):
     """Per-position transformation (dense or experts)."""
 
-    def forward(self, x: torch.Tensor, ctx: "StepContext") -> torch.Tensor:
+    takes_normed_rows = False       # as for Mixer
+
+    def forward(self, x: torch.Tensor, ctx: "StepContext") -> torch.Tensor | None:
+        """x [T, hidden] -> what is to be added to the residual, as for ``Mixer.forward``."""
         raise NotImplementedError
 
 

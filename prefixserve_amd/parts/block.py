@@ -17,7 +17,10 @@ class PreNormBlock:
 
     The residual stream is float32. Each sub-layer's output is not added at once: it is
     handed on as ``pending`` and summed into the residual by the next norm's fused
-    add+norm, so the stream is read and written once per sub-layer."""
+    add+norm, so the stream is read and written once per sub-layer. A sub-layer may also add its
+    output into the stream itself and hand on None; and where a sub-layer's kernels normalize
+    their tokens themselves (``takes_normed_rows``), the norm in front of it may hand over the
+    rows of the stream instead of running a kernel."""
 
     def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm, feed_forward_norm: Norm) -> None:
         self.mixer, self.feed_forward = mixer, feed_forward
@@ -28,9 +31,15 @@ class PreNormBlock:
 
     def forward(self, residual: torch.Tensor, pending: torch.Tensor | None, ctx: "StepContext", cache: Any,
                 state: torch.Tensor | None, writes_cache: bool) -> torch.Tensor:
-        x = self.mixer_norm.add_norm(residual, pending, "block.x")
+        if self.mixer.takes_normed_rows:
+            x = self.mixer_norm.add_norm(residual, pending, "block.x", lazy=True)
+        else:
+            x = self.mixer_norm.add_norm(residual, pending, "block.x")
         mixed = self.mixer.forward(x, ctx, cache, state, writes_cache)
-        x = self.feed_forward_norm.add_norm(residual, mixed, "block.x")
+        if self.feed_forward.takes_normed_rows:
+            x = self.feed_forward_norm.add_norm(residual, mixed, "block.x", lazy=True)
+        else:
+            x = self.feed_forward_norm.add_norm(residual, mixed, "block.x")
         return self.feed_forward.forward(x, ctx)
 
 

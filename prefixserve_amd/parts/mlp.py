@@ -17,6 +17,8 @@ class SwiGLU(FeedForward):
     first ``intermediate_size`` columns are the gate (prefixserve/model/llama.py:120-121,
     prefixserve/model/weights.py:120-123)."""
 
+    takes_normed_rows = True
+
     def __init__(self, hidden_size: int, intermediate_size: int, names: Mapping[str, str],
                  activation: str = "silu") -> None:
         if activation != "silu":
@@ -43,7 +45,7 @@ class SwiGLU(FeedForward):
         t = x.shape[0]
         act = ws.get("mlp.act", (t, self.intermediate_size), rt.dtype)
         ops.linear_swiglu(x, self.w_gate_up, act)
-        return ops.linear_to_residual(act, self.w_down, "mlp.delta")
+        return ops.linear_to_residual(act, self.w_down, "mlp.delta", getattr(ctx, "residual", None))
 
 
 register_feed_forward("swiglu", SwiGLU)

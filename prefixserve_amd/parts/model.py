@@ -126,13 +126,14 @@ class DecoderModel:
         with ops.step_scope():
             residual = ws.get("residual", (t, s.hidden_size), torch.float32)
             ops.embed(ctx.token_ids, self.embedding, residual)
+            ctx.residual = residual
             pending = None
             for i, run in enumerate(s.order):
                 pending = self.blocks[run.layer].forward(residual, pending, ctx, self.caches.get(run.cache),
                                                          self.states.get(i), run.writes_cache)
             if ctx.num_logit_rows == 0:
                 return None
-            x = self.final_norm.add_norm_rows(residual, pending, ctx.logit_rows, "final.x")
+            x = self.final_norm.add_norm_rows(residual, pending, ctx.logit_rows, "final.x", lazy=True)
             logits = ws.get("logits", (ctx.num_logit_rows, s.vocab_size), torch.float32)
             ops.linear(x, self.head, logits)
             return logits

@@ -6,7 +6,7 @@ from typing import Mapping
 
 import torch
 
-from .base import Norm, Runtime, WeightWant, register_norm
+from .base import Norm, NormedRows, Runtime, WeightWant, register_norm
 
 
 class RMSNorm(Norm):
@@ -32,15 +32,25 @@ class RMSNorm(Norm):
     def weight_bytes(self) -> int:
         return self.weight.numel() * self.weight.element_size()
 
-    def add_norm(self, residual: torch.Tensor, delta: torch.Tensor | None, out_name: str) -> torch.Tensor:
+    def _lazy(self, count: int) -> bool:
+        """Whether the kernels of this runtime normalize ``count`` rows of this width themselves."""
+        fuses = getattr(self.rt.ops, "fuses_norm", None)
+        return fuses is not None and fuses(count, self.hidden_size, self.rt.dtype)
+
+    def add_norm(self, residual: torch.Tensor, delta: torch.Tensor | None, out_name: str,
+                 lazy: bool = False) -> torch.Tensor | NormedRows:
         rt = self.rt
+        if lazy and delta is None and self._lazy(residual.shape[0]):
+            return NormedRows(residual, self.weight, self.eps, rt.dtype)
         out = rt.workspace.get(out_name, (residual.shape[0], self.hidden_size), rt.dtype)
         rt.ops.add_rmsnorm(residual, delta, self.weight, self.eps, out)
         return out
 
     def add_norm_rows(self, residual: torch.Tensor, delta: torch.Tensor | None, rows: torch.Tensor,
-                      out_name: str) -> torch.Tensor:
+                      out_name: str, lazy: bool = False) -> torch.Tensor | NormedRows:
         rt = self.rt
+        if lazy and delta is None and self._lazy(rows.shape[0]):
+            return NormedRows(residual, self.weight, self.eps, rt.dtype, rows)
         out = rt.workspace.get(out_name, (rows.shape[0], self.hidden_size), rt.dtype)
         rt.ops.add_rmsnorm_rows(residual, delta, rows, self.weight, self.eps, out)
         return out

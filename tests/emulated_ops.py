@@ -48,7 +48,7 @@ class EmulatedOps:
     def linear(self, x, w, out) -> None:
         out.copy_((x.float() @ w.float().T).to(out.dtype))
 
-    def linear_to_residual(self, x, w, name):
+    def linear_to_residual(self, x, w, name, residual=None):
         out = self.ws.get(name, (x.shape[0], w.shape[0]), x.dtype)
         self.linear(x, w, out)
         return out

@@ -269,6 +269,135 @@ def test_linear_to_residual_by_workgroups_that_stay(ops, m, n, k):
     assert rel(out.sum(0), x.double() @ w.double().T) < 1e-5
 
 
+# ---- small steps without norm kernels: products that add into the residual stream, and products
+# ---- that normalize the rows they read
+
+def _rms_rows(resid, weight, eps):
+    x = resid.double()
+    return x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps) * weight.double()
+
+
+@pytest.mark.parametrize("m", [1, 3, 4, 8, 9, 16])
+@pytest.mark.parametrize("n,k", [(2048, 2048), (2048, 8192), (200, 96), (2064, 4128), (4096, 14336), (72, 520), (3072, 8192)])
+def test_linear_to_residual_adds_into_the_stream(ops, m, n, k):
+    """Up to 16 tokens: every K-slice adds its partial sums into the float32 residual itself
+    (float atomics), whatever was there before; twice in a row adds twice. Rows after the last
+    token are not touched."""
+    if not ops.fuses_norm(m, n, torch.bfloat16):
+        pytest.skip("this width is not one the kernels without a norm kernel take")
+    x, w = rnd(m, k, dtype=torch.bfloat16, seed=1), rnd(n, k, dtype=torch.bfloat16, seed=2, scale=0.05)
+    start = rnd(m + 1, n, seed=3)
+    resid = start.clone()
+    assert ops.linear_to_residual(x, w, "test.add", resid[:m]) is None
+    prod = x.double() @ w.double().T
+    assert rel(resid[:m].double() - start[:m].double(), prod) < 1e-5
+    assert ops.linear_to_residual(x, w, "test.add", resid[:m]) is None
+    assert rel(resid[:m].double() - start[:m].double(), 2 * prod) < 1e-5
+    assert torch.equal(resid[m], start[m])
+    # a step too large for it hands back what is to be added, as before
+    big = rnd(17, k, dtype=torch.bfloat16, seed=4)
+    out = ops.linear_to_residual(big, w, "test.add2", torch.zeros(17, n, device=DEV))
+    assert out is not None and rel(out.sum(0) if out.dim() == 3 else out, big.double() @ w.double().T) < 5e-3
+
+
+@pytest.mark.parametrize("m", [1, 2, 5, 8, 9, 16])
+@pytest.mark.parametrize("n,k,epilogue,out_dtype,wdt", [
+    (8192, 2048, 1, torch.bfloat16, torch.bfloat16),      # gate/up of the 1B shape: 512 pairs of tiles
+    (14336, 4096, 1, torch.bfloat16, torch.bfloat16),     # of the 8B shape: 896 pairs, workgroups that stay for several
+    (344, 96, 1, torch.bfloat16, torch.float32),          # a pair count that is no multiple of anything, 32-bit norm weight
+    (66000, 2048, 0, torch.float32, torch.bfloat16),      # the output matrix: two row tiles per group
+    (33000, 4096, 0, torch.float32, torch.float32),       # one row tile per group
+    (1001, 160, 0, torch.bfloat16, torch.bfloat16),       # bfloat16 output, a partial last tile
+    (257, 64, 0, torch.float32, torch.bfloat16),
+])
+def test_products_that_normalize_the_rows_they_read(ops, m, n, k, epilogue, out_dtype, wdt):
+    """x is handed over as rows of the float32 residual stream with their RMS norm still to be
+    applied; the kernel applies it while it stages the rows. Against float64, with rows picked
+    by an index list (as the logits' rows are) and in order, a norm weight in either dtype, an
+    eps that matters (one row is tiny) and a row of zeros."""
+    from prefixserve_amd.parts.base import NormedRows
+
+    t = m + 5
+    resid = rnd(t, k, seed=5, scale=3.0)
+    resid[1] *= 1e-4                                   # eps decides this row's scale
+    resid[2] = 0.0
+    weight = (1.0 + 0.1 * torch.randn(k, generator=torch.Generator().manual_seed(6))).to(wdt).to(DEV)
+    eps = 1e-5
+    rows_list = [int(i) for i in np.random.default_rng(m).permutation(t)[:m]]
+    if m >= 3:
+        rows_list[0], rows_list[1] = 1, 2
+    rows = torch.tensor(rows_list, dtype=torch.int32, device=DEV)
+    w = rnd((2 if epilogue else 1) * n, k, dtype=torch.bfloat16, seed=7, scale=0.05)
+    for idx in (rows, None):
+        src = resid if idx is not None else resid[:m].contiguous()
+        x = NormedRows(src, weight, eps, torch.bfloat16, idx)
+        out = torch.full((m + 1, n), 7.0, dtype=out_dtype, device=DEV)
+        normed = _rms_rows(src[idx.long()] if idx is not None else src, weight, eps)
+        y = normed @ w.double().T
+        if epilogue:
+            ops.linear_swiglu(x, w, out[:m])
+            y = torch.nn.functional.silu(y[:, :n]) * y[:, n:]
+        else:
+            ops.linear(x, w, out[:m])
+        assert torch.all(out[m] == 7.0)
+        # the tokens are rounded to bfloat16 once, as the norm kernel's output is
+        for i in range(m):
+            scale = float(y[i].abs().max())
+            if scale == 0.0:
+                assert float(out[i].abs().max()) == 0.0
+            else:
+                assert float((out[i].double() - y[i]).abs().max()) < 1e-2 * scale, f"row {i}"
+    # and the same through the norm kernel, for a step the fused form does not take
+    x = NormedRows(resid, weight, eps, torch.bfloat16, None)
+    assert ops.normed(x).shape == (t, k) and rel(ops.normed(x), _rms_rows(resid, weight, eps)) < 5e-3
+
+
+@pytest.mark.parametrize("m", [1, 5, 8, 9, 16])
+@pytest.mark.parametrize("hq,hkv,d,k", [(32, 8, 64, 2048), (4, 2, 16, 64), (3, 1, 32, 96), (32, 8, 128, 4096), (50, 1, 128, 64),
+                                        (6, 3, 48, 160)])
+def test_qkv_rope_append_that_normalizes_its_rows(ops, m, hq, hkv, d, k):
+    """q/k/v + rotation + cache write reading the residual stream and normalizing it itself,
+    against float64 and against the norm kernel followed by the kernel that takes tokens."""
+    from prefixserve_amd.parts.base import NormedRows
+    from prefixserve_amd.parts.rope import rope_inv_freq
+
+    blocks = 12
+    resid = rnd(m, k, seed=1, scale=2.0)
+    weight = (1.0 + 0.1 * torch.randn(k, generator=torch.Generator().manual_seed(2))).to(torch.bfloat16).to(DEV)
+    eps = 1e-6
+    w = rnd((hq + 2 * hkv) * d, k, dtype=torch.bfloat16, seed=2, scale=0.1)
+    pos = torch.tensor([(7 * i + 3) % 150 for i in range(m)], dtype=torch.int32, device=DEV)
+    slots = torch.tensor(np.random.default_rng(m).permutation(blocks * 16)[:m].tolist(), dtype=torch.int32, device=DEV)
+    ang = torch.outer(torch.arange(150, dtype=torch.float32), rope_inv_freq(d, 10000.0, None)).double()
+    table = torch.stack((ang.cos(), ang.sin()), -1).float().to(DEV).contiguous()
+    n = (hq + 2 * hkv) * d
+    kv_a = torch.full((blocks, 2, hkv, 16 * d), 3.0, dtype=torch.bfloat16, device=DEV)
+    kv_b = kv_a.clone()
+    fused = torch.full((m + 1, n), 7.0, dtype=torch.bfloat16, device=DEV)
+    assert ops.fuses_norm(m, k, torch.bfloat16)
+    ops.qkv_rope_append(NormedRows(resid, weight, eps, torch.bfloat16), w, fused[:m], hq, hkv, d, pos, table, kv_a, slots)
+    xn = torch.empty(m, k, dtype=torch.bfloat16, device=DEV)
+    ops.add_rmsnorm(resid.clone(), None, weight, eps, xn)
+    plain = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+    ops.qkv_rope_append(xn, w, plain, hq, hkv, d, pos, table, kv_b, slots)
+    y = _rms_rows(resid, weight, eps) @ w.double().T
+    z = y[:, : (hq + hkv) * d].view(m, hq + hkv, d)
+    cs = table[pos.long()].double()
+    cos, sin = cs[..., 0][:, None], cs[..., 1][:, None]
+    z1, z2 = z[..., : d // 2], z[..., d // 2:]
+    want = torch.cat((torch.cat((z1 * cos - z2 * sin, z2 * cos + z1 * sin), -1).reshape(m, -1), y[:, (hq + hkv) * d:]), 1)
+    assert rel(fused[:m], want) < 1e-2 and rel(plain, want) < 1e-2 and torch.all(fused[m] == 7.0)
+    page, off = (slots // 16).long(), (slots % 16).long()
+    kp = kv_a[:, 0].view(blocks, hkv, 16, d)
+    vp = kv_a[:, 1].view(blocks, hkv, d, 16)
+    assert torch.equal(kp[page, :, off, :].reshape(m, -1), fused[:m, hq * d:(hq + hkv) * d])
+    assert torch.equal(vp[page, :, :, off].reshape(m, -1), fused[:m, (hq + hkv) * d:])
+    assert rel(kv_a.float(), kv_b.float()) < 2e-2
+    touched = torch.zeros(blocks, 16, dtype=torch.bool, device=DEV)
+    touched[page, off] = True
+    assert torch.all(kp.permute(0, 2, 1, 3)[~touched] == 3.0) and torch.all(vp.permute(0, 3, 1, 2)[~touched] == 3.0)
+
+
 @pytest.mark.parametrize("m", [3, 4, 7, 8, 9])
 @pytest.mark.parametrize("inter,k", [(12288 + 40, 4096), (12288, 4128)])
 def test_linear_swiglu_by_workgroups_that_stay(ops, m, inter, k):

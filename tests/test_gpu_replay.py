@@ -109,10 +109,14 @@ def test_graph_replay_equals_eager_decoding(model_dirs):
     """Decode steps through a captured graph, replayed many times with other work in between,
     against the same steps launched one by one. A graph is captured for the longest request
     there can be and splits the keys accordingly; a step launched by itself splits them for the
-    requests it has. With a longest request of 128 tokens both use one split and the logits agree
-    bit for bit; with 256 the graph merges two splits (the second of them empty here) where the
-    single step divides by the sum directly, which rounds differently: there the two agree to
-    within one bfloat16 step of the largest logit, and two runs through graphs bit for bit."""
+    requests it has: with a longest request of 256 tokens the graph merges two splits (the second
+    of them empty here) where the single step divides by the sum directly, which rounds
+    differently. And a small bfloat16 step adds the K-slices of its o and down products into the
+    residual stream with float atomics, in whatever order they arrive, so two runs of the same
+    step differ in the last bit of those sums and, where that flips the rounding of an
+    activation to bfloat16, by a little more. Graph and single steps, and two runs through
+    graphs, therefore agree to within one bfloat16 step of the largest logit, not bit for bit
+    (the 32-bit path, which has no atomics, does: test_cuttings_agree_with_each_other)."""
     reqs = requests_for("C", [90, 61, 40], seed=9)
 
     def decode(graphs, max_seq_len):
@@ -132,11 +136,14 @@ def test_graph_replay_equals_eager_decoding(model_dirs):
             assert (3, 3, False) in runner._graphs
         return np.stack(rows)
 
-    assert np.array_equal(decode(False, 128), decode(True, 128))
+    def apart(a, b):
+        return float((np.abs(a - b).max(-1) / np.abs(a).max(-1)).max())
+
+    short = apart(decode(False, 128), decode(True, 128))
     eager, graph = decode(False, 256), decode(True, 256)
-    assert np.array_equal(graph, decode(True, 256))
-    apart = np.abs(eager - graph).max(-1) / np.abs(eager).max(-1)
-    assert apart.max() < 2.0 ** -8, f"graph and single steps {apart.max():.2e} apart"
+    assert short < 2.0 ** -8, f"graph and single steps {short:.2e} apart"
+    assert apart(eager, graph) < 2.0 ** -8, f"graph and single steps {apart(eager, graph):.2e} apart"
+    assert apart(graph, decode(True, 256)) < 2.0 ** -8
 
 
 def test_decoding_with_one_long_context_among_short_ones_through_graphs(tmp_path):
