@@ -13,6 +13,7 @@ uniform-random token ids and seeded random weights; nothing is downloaded.
 from __future__ import annotations
 
 import argparse
+import gc
 import json
 import sys
 import tempfile
@@ -79,6 +80,12 @@ def main() -> int:
                     help="how often the timed region of K steps is run; the line reports the median repeat")
     ap.add_argument("--long-context", type=int, default=16384,
                     help="context of the extra decode point (0: skip it); its prompts fill all but 2,048 tokens of it")
+    ap.add_argument("--longer-context", type=int, default=65536, help="context of a second extra decode point (0: skip it)")
+    ap.add_argument("--skewed-context", type=int, default=30000,
+                    help="extra point: 32 requests decode together, one behind this many tokens, the others behind 200 (0: skip it)")
+    ap.add_argument("--other-shape", choices=sorted(SHAPES) + ["none"], default="llama-3.1-8b",
+                    help="extra point: some layers of this shape decoding at batch 32 in an 8,192 context")
+    ap.add_argument("--other-layers", type=int, default=8, help="how many layers of --other-shape are run")
     ap.add_argument("--no-peaks", action="store_true", help="skip measuring the copy bandwidth and a large library product")
     ap.add_argument("--model", default=None, help="use this model folder instead of writing random weights")
     ap.add_argument("--shape", choices=sorted(SHAPES), default="llama-3.2-1b", help="layer sizes of the random model")
@@ -120,15 +127,17 @@ def main() -> int:
     def sync() -> None:
         torch.cuda.synchronize()
 
-    def decode_run(engine, batch: int, steps: int, warmup: int, prompt_len: int, context: int, repeats: int = 1) -> dict:
+    def decode_run(engine, batch: int, steps: int, warmup: int, prompt_len, context: int, repeats: int = 1) -> dict:
         """``repeats`` timed regions of exactly ``steps`` decode steps each, every one between two
         device synchronisations; the result is the median region. Beside the host clock, the
         device's own time per scheduler round (events on the stream around the round's
         launches) and the host's shares: scheduling, packing the step's integers, commit."""
         runner = engine.runner
+        lens = list(prompt_len) if isinstance(prompt_len, (list, tuple)) else [prompt_len] * batch
+        prompt_len = max(lens)
         sched = engine.make_scheduler(chunk_size=prompt_len, enable_prefix_cache=False)
         for b in range(batch):
-            sched.add_request(f"d{batch}-{b}", rng.integers(0, vocab, prompt_len), context - prompt_len - 1, ignore_eos=True)
+            sched.add_request(f"d{batch}-{b}", rng.integers(0, vocab, lens[b]), context - lens[b] - 1, ignore_eos=True)
         # prompts, untimed: one request's prompt per step
         while any(r.num_computed < len(r.prompt) for r in sched.requests()):
             bt = sched.schedule_step(prompt_len, batch)
@@ -246,18 +255,48 @@ def main() -> int:
 
     peaks = {} if args.no_peaks else measured_peaks()      # last: a long product changes the clocks of what follows
 
-    if not args.no_points and args.long_context > args.context:
-        # The same batch over a long context, where the cache is most of what a step reads.
-        del runner
-        engine = None
+    def fresh_engine(folder, batch: int, prefill_tokens: int, context: int, blocks: int) -> "Engine":
+        """Another engine in place of the current one (its pools go back to the device first)."""
+        nonlocal engine, runner, weight_bytes, kv_bytes_per_token
+        engine = runner = None
+        gc.collect()
         torch.cuda.empty_cache()
-        ctx_len = args.long_context
-        engine = Engine(EngineConfig(model_path=model_dir, dtype=args.dtype, max_num_seqs=args.batch,
-                                     max_prefill_tokens=ctx_len - 2048, max_seq_len=ctx_len,
-                                     num_blocks=args.batch * (ctx_len // 16) + 64, use_graphs=not args.no_graphs))
-        long_run = decode_run(engine, args.batch, max(16, args.steps // 4), max(4, args.warmup // 4), ctx_len - 2048, ctx_len)
+        engine = Engine(EngineConfig(model_path=folder, dtype=args.dtype, max_num_seqs=batch, max_prefill_tokens=prefill_tokens,
+                                     max_seq_len=context, num_blocks=blocks, use_graphs=not args.no_graphs))
+        weight_bytes = engine.runner.model.step_weight_bytes()
+        kv_bytes_per_token = sum(engine.runner.bytes_per_block) // 16
+        return engine
+
+    steps_q, warm_q = max(16, args.steps // 4), max(4, args.warmup // 4)
+    for ctx_len in ([] if args.no_points else [c for c in (args.long_context, args.longer_context) if c > args.context]):
+        # The same batch over a long context, where the cache is most of what a step reads.
+        fresh_engine(model_dir, args.batch, ctx_len - 2048, ctx_len, args.batch * (ctx_len // 16) + 64)
+        long_run = decode_run(engine, args.batch, steps_q, warm_q, ctx_len - 2048, ctx_len)
         points[f"decode_b{args.batch}_context_{ctx_len}"] = long_run["tok_s"]
         points[f"decode_b{args.batch}_context_{ctx_len}_hbm_frac"] = long_run["gbs"] / HBM_PEAK_GBS
+
+    if not args.no_points and args.skewed_context > 0:
+        # Contexts of unequal length in one batch: 31 requests behind 200 tokens and one behind
+        # args.skewed_context, the attention reading the long one with the whole chip.
+        lens = [args.skewed_context] + [200] * 31
+        top = args.skewed_context + 512
+        fresh_engine(model_dir, 32, args.skewed_context, top, sum(-(-(n + 300) // 16) for n in lens) + 64)
+        run = decode_run(engine, 32, steps_q, warm_q, lens, top)
+        points[f"decode_b32_one_context_of_{args.skewed_context}_among_200"] = run["tok_s"]
+        points[f"decode_b32_one_context_of_{args.skewed_context}_among_200_hbm_frac"] = run["gbs"] / HBM_PEAK_GBS
+
+    if not args.no_points and args.other_shape != "none" and args.model is None:
+        # Another width and head size: some of the layers of a larger shape (the name says how
+        # many of how many), decoding at batch 32 behind 4,096-token prompts in an 8,192 context.
+        other = dict(SHAPES[args.other_shape])
+        of = other["num_hidden_layers"]
+        other["num_hidden_layers"] = min(args.other_layers, of)
+        other_dir = write_random_model(Path(tmp.name) / "other", other, seed=1)
+        fresh_engine(other_dir, 32, 4096, 8192, 32 * (8192 // 16) + 64)
+        run = decode_run(engine, 32, steps_q, warm_q, 4096, 8192)
+        name = f"{args.other_shape}_{other['num_hidden_layers']}_of_{of}_layers_decode_b32_context_8192"
+        points[name] = run["tok_s"]
+        points[name + "_hbm_frac"] = run["gbs"] / HBM_PEAK_GBS
 
     line = {
         "metric": "decode_tokens_per_second", "value": main_run["tok_s"], "unit": "tok/s", "n_gpus": 1,
