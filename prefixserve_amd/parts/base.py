@@ -206,6 +206,16 @@ class Mixer(Part):
         raise NotImplementedError
 
 
+class Transform(Part):
+    """Changes a float32 tensor of the step in place: the residual stream ``[T, hidden]`` right
+    behind the token table, or the logits ``[S, vocab]``. ``rows`` are the flat token rows the
+    tensor's rows belong to (all tokens in order for the stream, ``ctx.logit_rows`` for logits),
+    for a transform that depends on the position (``ctx.positions[rows]``)."""
+
+    def apply(self, t: torch.Tensor, ctx: "StepContext", rows: torch.Tensor | None) -> None:
+        raise NotImplementedError
+
+
 class FeedForward(Part):
     """Per-position transformation (dense or experts)."""
 
@@ -221,7 +231,7 @@ class FeedForward(Part):
 Factory = Callable[..., Any]
 
 _REGISTRIES: dict[str, dict[str, Factory]] = {
-    "mixer": {}, "feed_forward": {}, "norm": {}, "position": {}, "block": {},
+    "mixer": {}, "feed_forward": {}, "norm": {}, "position": {}, "block": {}, "transform": {},
 }
 
 
@@ -253,8 +263,13 @@ def register_position(kind: str, factory: Factory) -> None:
 
 
 def register_block(kind: str, factory: Factory) -> None:
-    """factory(mixer=..., feed_forward=..., mixer_norm=..., feed_forward_norm=...) -> Block"""
+    """factory(mixer=..., feed_forward=..., mixer_norm=..., feed_forward_norm=..., **extra_norms) -> Block"""
     _register("block", kind, factory)
+
+
+def register_transform(kind: str, factory: Factory) -> None:
+    """factory(hidden_size=..., vocab_size=..., **params) -> Transform"""
+    _register("transform", kind, factory)
 
 
 def make(family: str, kind: str, **kwargs: Any) -> Any:

@@ -20,7 +20,9 @@ class PreNormBlock:
     add+norm, so the stream is read and written once per sub-layer. A sub-layer may also add its
     output into the stream itself and hand on None; and where a sub-layer's kernels normalize
     their tokens themselves (``takes_normed_rows``), the norm in front of it may hand over the
-    rows of the stream instead of running a kernel."""
+    rows of the stream instead of running a kernel. An arrangement that needs a sub-layer's
+    output itself (to normalize it before it is added, say) sets ``ctx.residual = None`` first:
+    the sub-layers then hand their output back in every step."""
 
     def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm, feed_forward_norm: Norm) -> None:
         self.mixer, self.feed_forward = mixer, feed_forward

@@ -32,9 +32,13 @@ class DecoderModel:
             ff = make("feed_forward", layer.feed_forward.kind, hidden_size=h, **layer.feed_forward.params)
             n1 = make("norm", layer.mixer_norm.kind, hidden_size=h, **layer.mixer_norm.params)
             n2 = make("norm", layer.feed_forward_norm.kind, hidden_size=h, **layer.feed_forward_norm.params)
+            extra = {name: make("norm", ps.kind, hidden_size=h, **ps.params) for name, ps in layer.extra_norms.items()}
             self.blocks.append(make("block", layer.block, mixer=mixer, feed_forward=ff, mixer_norm=n1,
-                                    feed_forward_norm=n2))
+                                    feed_forward_norm=n2, **extra))
         self.final_norm = make("norm", spec.final_norm.kind, hidden_size=spec.hidden_size, **spec.final_norm.params)
+        sizes = dict(hidden_size=spec.hidden_size, vocab_size=spec.vocab_size)
+        self.embedding_transforms = [make("transform", ps.kind, **sizes, **ps.params) for ps in spec.embedding_transforms]
+        self.logit_transforms = [make("transform", ps.kind, **sizes, **ps.params) for ps in spec.logit_transforms]
         self.caches: dict[int, Any] = {}
         self.states: dict[int, torch.Tensor] = {}
         self.rt: Runtime | None = None
@@ -46,6 +50,7 @@ class DecoderModel:
         for layer, blk in zip(self.spec.layers, self.blocks):
             out += [(layer.prefix, p) for p in blk.parts()]
         out.append((self.spec.final_norm_prefix, self.final_norm))
+        out += [("", tr) for tr in self.embedding_transforms + self.logit_transforms]
         return out
 
     def weights(self) -> dict[str, WeightWant]:
@@ -126,6 +131,8 @@ class DecoderModel:
         with ops.step_scope():
             residual = ws.get("residual", (t, s.hidden_size), torch.float32)
             ops.embed(ctx.token_ids, self.embedding, residual)
+            for tr in self.embedding_transforms:
+                tr.apply(residual, ctx, None)
             ctx.residual = residual
             pending = None
             for i, run in enumerate(s.order):
@@ -136,4 +143,6 @@ class DecoderModel:
             x = self.final_norm.add_norm_rows(residual, pending, ctx.logit_rows, "final.x", lazy=True)
             logits = ws.get("logits", (ctx.num_logit_rows, s.vocab_size), torch.float32)
             ops.linear(x, self.head, logits)
+            for tr in self.logit_transforms:
+                tr.apply(logits, ctx, ctx.logit_rows)
             return logits

@@ -31,6 +31,9 @@ class LayerSpec:
     mixer_norm: PartSpec
     feed_forward_norm: PartSpec
     block: str = "prenorm"
+    # Further norms an arrangement other than "prenorm" may want (norms behind the sub-layers,
+    # say): built like the two above and handed to the block's factory by these names.
+    extra_norms: Mapping[str, PartSpec] = field(default_factory=dict)
 
 
 @dataclass(frozen=True)
@@ -62,6 +65,11 @@ class ModelSpec:
     max_position: int
     stop_token_ids: frozenset[int] = frozenset()
     ignored_weights: tuple[str, ...] = ()  # name suffixes a checkpoint may carry and we recompute
+    # Transforms of the residual stream right behind the token table (a scale, an added table by
+    # position) and of the logits (a cap, a scale, a bias), in the order they are applied; their
+    # weight names are taken as they are, without a prefix.
+    embedding_transforms: tuple[PartSpec, ...] = ()
+    logit_transforms: tuple[PartSpec, ...] = ()
 
     def validate(self) -> None:
         writers: dict[int, int] = {}

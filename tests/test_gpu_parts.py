@@ -4,6 +4,7 @@ registered, built into a model and stepped without touching the package's files.
 
 from __future__ import annotations
 
+import math
 
 import numpy as np
 import pytest
@@ -448,3 +449,141 @@ def test_a_toy_position_encoding_and_a_routed_feed_forward(tmp_path):
                 err = np.abs(got - want[p0:p0 + c]).max(-1) / np.abs(want[p0:p0 + c]).max(-1)
                 assert err.max() < tol, f"{dtype} positions {p0}..{p0 + c}: {err.max():.3e}"
                 p0 += c
+
+
+def test_toy_transforms_and_a_block_with_more_norms(tmp_path):
+    """Three more things a model may be made of, defined and registered from this test only: the
+    residual stream scaled and given a learned row per position right behind the token table,
+    the logits capped (cap * tanh(logits / cap)), and a block with a norm behind each sub-layer
+    as well as in front of it (``LayerSpec.extra_norms``). The block wants each sub-layer's
+    output itself, so it keeps the stream to itself (``ctx.residual = None``). Compared with the
+    plain functions whole, in portions and token by token through graphs, in both dtypes."""
+    import json
+
+    from safetensors.torch import save_file
+
+    from prefixserve_amd.config import register_architecture, registered_architectures
+    from prefixserve_amd.engine.replay import TraceReplayer
+    from prefixserve_amd.engine.runner import ModelRunner
+    from prefixserve_amd.parts import (DecoderModel, LayerRun, LayerSpec, ModelSpec, PartSpec, Transform, WeightWant,
+                                       register_block, register_transform)
+    from prefixserve_amd.weights import random_tensors
+
+    H, HQ, HKV, D, INNER, V, CAP, MAXPOS = 64, 4, 2, 16, 96, 110, 3.0, 256
+
+    class Scale(Transform):
+        def __init__(self, hidden_size, vocab_size, factor):
+            self.factor = float(factor)
+
+        def apply(self, t, ctx, rows):
+            t.mul_(self.factor)
+
+    class LearnedPositions(Transform):
+        def __init__(self, hidden_size, vocab_size, name, positions):
+            self.h, self.name, self.n = hidden_size, name, positions
+
+        def weights(self):
+            return {self.name: WeightWant((self.n, self.h))}
+
+        def bind(self, tensors, rt):
+            super().bind(tensors, rt)
+            self.table = tensors[self.name].to(rt.device, torch.float32)
+
+        def apply(self, t, ctx, rows):
+            pos = ctx.positions if rows is None else ctx.positions[rows.long()]
+            t.add_(self.table[pos.long()])
+
+    class SoftCap(Transform):
+        def __init__(self, hidden_size, vocab_size, cap):
+            self.cap = float(cap)
+
+        def apply(self, t, ctx, rows):
+            t.copy_(self.cap * torch.tanh(t / self.cap))
+
+    class Sandwich:
+        def __init__(self, mixer, feed_forward, mixer_norm, feed_forward_norm, post_mixer, post_feed_forward):
+            self.mixer, self.ff, self.n1, self.n2, self.p1, self.p2 = mixer, feed_forward, mixer_norm, feed_forward_norm, post_mixer, post_feed_forward
+
+        def parts(self):
+            return [self.n1, self.mixer, self.p1, self.n2, self.ff, self.p2]
+
+        def _normed(self, norm, delta, name):
+            ws = norm.rt.workspace
+            t = delta.shape[-2]
+            zero = ws.get("sandwich.zero", (t, H), torch.float32)
+            zero.zero_()
+            return norm.add_norm(zero, delta, name)                # norm(0 + delta)
+
+        def forward(self, residual, pending, ctx, cache, state, writes_cache):
+            ctx.residual = None                                    # the sub-layers hand their output back
+            x = self.n1.add_norm(residual, pending, "block.x")
+            y = self._normed(self.p1, self.mixer.forward(x, ctx, cache, state, writes_cache), "sandwich.y1")
+            x = self.n2.add_norm(residual, y, "block.x")
+            return self._normed(self.p2, self.ff.forward(x, ctx), "sandwich.y2")
+
+    class Cfg:
+        def __init__(self, raw):
+            self.raw = raw
+
+        @classmethod
+        def from_dicts(cls, raw, gen=None):
+            return cls(dict(raw))
+
+    def build(cfg):
+        attn = PartSpec("paged_attention", {"num_heads": HQ, "num_kv_heads": HKV, "head_dim": D, "position": "rope",
+                                            "names": {"q": "q.weight", "k": "k.weight", "v": "v.weight", "o": "o.weight"}})
+        ff = PartSpec("swiglu", {"intermediate_size": INNER, "names": {"gate": "g.weight", "up": "u.weight", "down": "d.weight"}})
+        norm = lambda nm: PartSpec("rmsnorm", {"eps": 1e-5, "name": nm})
+        layers = tuple(LayerSpec(prefix=f"l{i}.", mixer=attn, feed_forward=ff, mixer_norm=norm("n1.weight"),
+                                 feed_forward_norm=norm("n2.weight"), block="test_sandwich",
+                                 extra_norms={"post_mixer": norm("p1.weight"), "post_feed_forward": norm("p2.weight")})
+                       for i in range(2))
+        return ModelSpec(vocab_size=V, hidden_size=H, embedding="emb.weight", layers=layers,
+                         order=(LayerRun(0, 0), LayerRun(1, 1)), final_norm=norm("norm.weight"), final_norm_prefix="",
+                         head=None, positions={"rope": PartSpec("rope", {"head_dim": D, "theta": 10000.0})}, max_position=MAXPOS,
+                         embedding_transforms=(PartSpec("test_scale", {"factor": math.sqrt(H)}),
+                                               PartSpec("test_learned_positions", {"name": "pos.weight", "positions": MAXPOS})),
+                         logit_transforms=(PartSpec("test_softcap", {"cap": CAP}),))
+
+    if "ToySandwichForCausalLM" not in registered_architectures():
+        register_transform("test_scale", Scale)
+        register_transform("test_learned_positions", LearnedPositions)
+        register_transform("test_softcap", SoftCap)
+        register_block("test_sandwich", Sandwich)
+        register_architecture("ToySandwichForCausalLM", Cfg, build)
+    raw = {"architectures": ["ToySandwichForCausalLM"]}
+    (tmp_path / "config.json").write_text(json.dumps(raw))
+    tensors = random_tensors(DecoderModel(build(Cfg(raw))).weights(), seed=4, std=0.1)
+    assert "pos.weight" in tensors and "l1.p2.weight" in tensors
+    save_file(tensors, str(tmp_path / "model.safetensors"))
+    w = {k: v.double().numpy() for k, v in tensors.items()}
+
+    toks = np.random.default_rng(5).integers(0, V, 90).tolist()
+    n = len(toks)
+    cos, sin = P.rope_cos_sin(np.arange(n), P.rope_inv_freq(D, 10000.0, None))
+    h = w["emb.weight"][toks] * math.sqrt(H) + w["pos.weight"][:n]
+    for i in range(2):
+        p = f"l{i}."
+        x = P.rms_norm(h, w[p + "n1.weight"], 1e-5)
+        q = P.apply_rope((x @ w[p + "q.weight"].T).reshape(n, HQ, D), cos, sin)
+        k = P.apply_rope((x @ w[p + "k.weight"].T).reshape(n, HKV, D), cos, sin)
+        v = (x @ w[p + "v.weight"].T).reshape(n, HKV, D)
+        h = h + P.rms_norm(P.causal_attention(q, k, v).reshape(n, HQ * D) @ w[p + "o.weight"].T, w[p + "p1.weight"], 1e-5)
+        x = P.rms_norm(h, w[p + "n2.weight"], 1e-5)
+        h = h + P.rms_norm(P.swiglu_mlp(x, w[p + "g.weight"], w[p + "u.weight"], w[p + "d.weight"]), w[p + "p2.weight"], 1e-5)
+    want = CAP * np.tanh(P.rms_norm(h, w["norm.weight"], 1e-5) @ w["emb.weight"].T / CAP)
+    assert np.abs(want).max() > 0.5 * CAP                          # the cap is felt
+
+    for dtype, tol in (("float32", 2e-5), ("bfloat16", 4e-2)):
+        runner = ModelRunner(tmp_path, dtype=dtype, device="cuda:0", num_blocks=16, max_seq_len=128, max_num_seqs=2,
+                             use_graphs=True)
+        for cuts in ([n], [7, 2, 30, 1, 1, 17] + [1] * 32):
+            rp = TraceReplayer(runner)
+            p0 = 0
+            for kk, c in enumerate(cuts):
+                got = rp.run_step({"step": kk, "entries": [{"id": "a", "tokens": toks[p0:p0 + c], "want": list(range(c))}],
+                                   "end": ["a"] if p0 + c == n else []})
+                err = np.abs(got - want[p0:p0 + c]).max(-1) / np.abs(want[p0:p0 + c]).max(-1)
+                assert err.max() < tol, f"{dtype} positions {p0}..{p0 + c}: {err.max():.3e}"
+                p0 += c
+        assert (1, 1, False) in runner._graphs                    # the single tokens went through a captured graph
