@@ -150,10 +150,10 @@ class StepPacker:
                                   buf[o_t:o_t + b + 1], buf[o_b:o_b + p_total]) for o_t, o_w, o_b in group_offs]
             self._views = (sig, on_dev, host, groups)
         _, on_dev, host, groups = self._views
+        skewed = bool(self._skew_rule(n_dec, dec_max_kv, dec_sum_kv)) if self._skew_rule is not None and n_dec > 1 else False
         return StepContext(
             num_tokens=t_n, num_items=b, num_logit_rows=s_n, num_decode=n_dec, num_prefill_tiles=n_tiles,
-            max_kv_len=max_kv_len, decode_skewed=bool(self._skew_rule(n_dec, dec_max_kv, dec_sum_kv)) if self._skew_rule and n_dec > 1 else False,
-            groups=groups,
+            max_kv_len=max_kv_len, decode_skewed=skewed, groups=groups,
             keys=[it.key for it in items],
             want_counts=[len(it.want) for it in items], host=host, **on_dev,
         )

@@ -93,6 +93,7 @@ class HipOps:
         self._sample_scratch: torch.Tensor | None = None
         self._step_stream: int | None = None
         self._plans: dict[tuple, tuple[int, int]] = {}
+        self._bounds: dict[Any, int] = {}                # sizes of the attention's partial-result buffers, from the library
         self._fuses: dict[tuple[int, int], bool] = {}
         self._slice_views: dict[tuple, tuple] = {}      # (name, slices, rows) -> (buffer, its [slices, rows, N] view)
         # The library for large bfloat16 products, called directly if it can be (it sets itself up
@@ -405,7 +406,9 @@ class HipOps:
                 # the most rows any step of this shape can need (the library says how many), so
                 # they never grow.
                 nsplit = self.lib.psamd_attention_prefill_nsplit(ctx.num_prefill_tiles, kv_len, hq, hkv, d)
-                rows = self.lib.psamd_attention_prefill_part_rows(hq, hkv, d)
+                rows = self._bounds.get((hq, hkv, d))
+                if rows is None:
+                    rows = self._bounds[(hq, hkv, d)] = int(self.lib.psamd_attention_prefill_part_rows(hq, hkv, d))
                 part_o = self.ws.get("attn.prefill_part_o", (rows * hq * d,), torch.float32)
                 part_ml = self.ws.get("attn.prefill_part_ml", (rows * hq * 2,), torch.float32)
                 if nsplit > 1:
@@ -421,7 +424,9 @@ class HipOps:
                 skewed = self.fixed_skew if self.fixed_kv_len else ctx.decode_skewed
                 nsplit, min_run = self.decode_plan(ctx.num_decode, kv_len, skewed, hkv, win)
                 # Room for the (request, run) pairs of any plan: asked for once, never grown.
-                parts = self.lib.psamd_attention_decode_max_parts(ctx.num_decode)
+                parts = self._bounds.get(ctx.num_decode)
+                if parts is None:
+                    parts = self._bounds[ctx.num_decode] = int(self.lib.psamd_attention_decode_max_parts(ctx.num_decode))
                 self._need(ctx.num_decode * nsplit <= parts, "attention: more (request, run) pairs than planned for")
                 part_o = self.ws.get("attn.part_o", (parts * hq * d,), torch.float32)
                 part_ml = self.ws.get("attn.part_ml", (parts * hq * 2,), torch.float32)
