@@ -283,11 +283,16 @@ def test_linear_to_residual_adds_into_the_stream(ops, m, n, k):
     """Up to 16 tokens: every K-slice adds its partial sums into the float32 residual itself
     (float atomics), whatever was there before; twice in a row adds twice. Rows after the last
     token are not touched."""
-    if not ops.fuses_norm(m, n, torch.bfloat16):
-        pytest.skip("this width is not one the kernels without a norm kernel take")
     x, w = rnd(m, k, dtype=torch.bfloat16, seed=1), rnd(n, k, dtype=torch.bfloat16, seed=2, scale=0.05)
     start = rnd(m + 1, n, seed=3)
     resid = start.clone()
+    if not ops.fuses_norm(m, n, torch.bfloat16):
+        # a width the kernels that normalize their rows do not take (no whole 32-wide k-steps, or rows
+        # that do not fit LDS): the product is handed back and the stream left alone
+        out = ops.linear_to_residual(x, w, "test.add", resid[:m])
+        assert out is not None and torch.equal(resid, start)
+        assert rel(out.sum(0) if out.dim() == 3 else out, x.double() @ w.double().T) < 5e-3
+        return
     assert ops.linear_to_residual(x, w, "test.add", resid[:m]) is None
     prod = x.double() @ w.double().T
     assert rel(resid[:m].double() - start[:m].double(), prod) < 1e-5
@@ -722,8 +727,6 @@ def test_attention_ignores_what_lies_in_slots_nobody_wrote(ops, act, hq, hkv, d,
     """The rest of a request's last page, and pages a window has given back, may hold what an
     earlier owner left there, NaN and infinities included. Their keys are masked; their values
     must not reach the output either (0 x NaN is NaN)."""
-    if act == torch.float32 and max(new) > 1000:
-        pytest.skip("the 32-bit kernel is one wave per token and head: covered at the small sizes")
     pages = sum(-(-(n + o) // 16) for n, o in zip(new, old)) + 8
     for poison in (float("nan"), float("inf")):
         got, want = paged_case(ops, act, hq, hkv, d, new, old, window=window, seed=7 + d, num_blocks=pages, poison=poison,
