@@ -74,6 +74,7 @@ _SIGNATURES = {
 class HipOps:
     PREFILL_TILE_Q = 32    # queries per workgroup of the prefill attention kernel (its 4 waves split the keys)
     SKINNY_MAX_ROWS = 64
+    FUSED_SWIGLU_MAX_ROWS = 32      # above it (to SKINNY_MAX_ROWS) gate/up goes to the library, where there is one
     name = "hip"
 
     def __init__(self, device: torch.device | str, workspace: Any = None) -> None:
@@ -356,7 +357,19 @@ class HipOps:
                                                       out.data_ptr(), _BF16, m, inter, k, 1))
                 return
             x = self.normed(x)
-        if x.dtype == torch.bfloat16 and k % 8 == 0 and m <= self.SKINNY_MAX_ROWS:
+        self._need(x.is_contiguous() and w_gate_up.is_contiguous() and out.is_contiguous(), "linear_swiglu: contiguous operands")
+        small = x.dtype == torch.bfloat16 and k % 8 == 0 and m <= self.SKINNY_MAX_ROWS
+        if small and m > self.FUSED_SWIGLU_MAX_ROWS and self._direct_library:
+            # Between these row counts the library's product and the activation kernel behind it
+            # take less time than the fused form, which streams the weights with too few rows a wave.
+            gu = self.ws.get("mlp.gate_up", (m, 2 * inter), x.dtype)
+            rc = self.lib.psamd_gemm_lt(self._stream(), x.data_ptr(), w_gate_up.data_ptr(), gu.data_ptr(), _BF16,
+                                        m, 2 * inter, k, 0 if self.fixed_kv_len else 1)
+            if rc != 2:                          # 2: no algorithm for this shape: the fused form below
+                self._ok(rc)
+                self.swiglu(gu, out)
+                return
+        if small:
             self._ok(self.lib.psamd_linear_skinny(self._stream(), x.data_ptr(), w_gate_up.data_ptr(), out.data_ptr(),
                                                   _BF16, m, inter, k, 1, 1))
             return

@@ -472,11 +472,18 @@ def test_linear_swiglu_wide(ops, m, inter):
     the rows of such a group, a K with a partial last step."""
     k = 72
     x, w = rnd(m, k, dtype=torch.bfloat16, seed=1), rnd(2 * inter, k, dtype=torch.bfloat16, seed=2, scale=0.2)
-    out = torch.full((m + 1, inter), 7.0, dtype=torch.bfloat16, device=DEV)
-    ops.linear_swiglu(x, w, out[:m])
     gu = x.double() @ w.double().T
     want = torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:]
-    assert rel(out[:m], want) < 1e-2 and torch.all(out[m] == 7.0)
+    # above 32 tokens the library's product and the activation kernel stand in where the library
+    # is found; the fused form is what remains without it, so both are run
+    for through_library in ((True, False) if m > ops.FUSED_SWIGLU_MAX_ROWS else (True,)):
+        ops._direct_library = through_library
+        try:
+            out = torch.full((m + 1, inter), 7.0, dtype=torch.bfloat16, device=DEV)
+            ops.linear_swiglu(x, w, out[:m])
+        finally:
+            ops._direct_library = True
+        assert rel(out[:m], want) < 1e-2 and torch.all(out[m] == 7.0)
 
 
 # -------------------------------------------------------------------- attention
