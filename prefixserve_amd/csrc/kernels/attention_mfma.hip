@@ -1156,8 +1156,8 @@ extern "C" {
 int psamd_attention_mfma_supports(int hq, int hkv, int head_dim) {
   if (hq <= 0 || hkv <= 0 || hq % hkv) return 0;
   const int group = hq / hkv;
-  const bool dim_ok = head_dim == 16 || head_dim == 32 || head_dim == 64 || head_dim == 96 || head_dim == 128 ||
-                      head_dim == 256;
+  const bool dim_ok = head_dim % 16 == 0 && ((head_dim >= 16 && head_dim <= 128) || head_dim == 160 || head_dim == 192 ||
+                                             head_dim == 256);
   const size_t smem = sizeof(float) * (8 * group + 4 * static_cast<size_t>(group) * head_dim);
   return dim_ok && group <= 64 && smem <= 64 * 1024 && hq <= 65535 && hkv <= 65535;
 }
@@ -1204,9 +1204,14 @@ int psamd_attention_prefill(void* stream, const void* qkv, int q_stride, void* o
   switch (head_dim / 16) {
     case 1: PSAMD_PF(1);
     case 2: PSAMD_PF(2);
+    case 3: PSAMD_PF(3);
     case 4: PSAMD_PF(4);
+    case 5: PSAMD_PF(5);
     case 6: PSAMD_PF(6);
+    case 7: PSAMD_PF(7);
     case 8: PSAMD_PF(8);
+    case 10: PSAMD_PF(10);
+    case 12: PSAMD_PF(12);
     default: PSAMD_PF(16);
   }
 #undef PSAMD_PF
@@ -1271,9 +1276,14 @@ int psamd_attention_decode(void* stream, const void* qkv, int q_stride, void* ou
   switch (head_dim / 16) {
     case 1: PSAMD_DEC_NS(1);
     case 2: PSAMD_DEC_NS(2);
+    case 3: PSAMD_DEC_NS(3);
     case 4: PSAMD_DEC_NS(4);
+    case 5: PSAMD_DEC_NS(5);
     case 6: PSAMD_DEC_NS(6);
+    case 7: PSAMD_DEC_NS(7);
     case 8: PSAMD_DEC_NS(8);
+    case 10: PSAMD_DEC_NS(10);
+    case 12: PSAMD_DEC_NS(12);
     default: PSAMD_DEC_NS(16);
   }
 #undef PSAMD_DEC_NS

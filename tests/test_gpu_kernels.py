@@ -543,7 +543,10 @@ def paged_case(ops, act, hq, hkv, d, lens_new, lens_old, window=None, seed=0, nu
 
 
 SHAPES = [(4, 2, 16), (3, 1, 32), (8, 2, 64), (32, 8, 64), (6, 6, 96), (8, 1, 128), (40, 2, 64), (2, 2, 256), (6, 3, 48), (2, 1, 80),
-          (6, 2, 256), (12, 4, 128), (5, 1, 32), (9, 3, 96)]
+          (6, 2, 256), (12, 4, 128), (5, 1, 32), (9, 3, 96),
+          # head sizes that are no multiple of 32 (the last step of 32 half used) and the sizes above 128
+          (8, 2, 48), (10, 2, 80), (8, 2, 112), (4, 1, 160), (6, 2, 192),
+          (4, 2, 144)]      # one the matrix-core kernels do not take: the generic kernel
 
 
 @pytest.mark.parametrize("hq,hkv,d", SHAPES)
@@ -562,7 +565,9 @@ def test_paged_attention_mixed_batch(ops, act, hq, hkv, d):
     (32, 8, 64, 700, 150),         # the same with a window whose first pages were given back
     (16, 8, 128, 3300, None),      # head size 128, long contexts
     (16, 8, 128, 700, None),       # and short ones
-    (6, 3, 48, 300, None),         # a head size the matrix-core kernels do not take: the generic kernel
+    (6, 3, 48, 300, None),         # a head size that is no multiple of 32
+    (10, 2, 80, 700, None),        # the same with five heads per kv head
+    (4, 2, 144, 300, None),        # a head size the matrix-core kernels do not take: the generic kernel
 ])
 def test_decode_attention_of_many_requests(ops, hq, hkv, d, longest, window):
     """Forty requests decode together, their contexts from 0 to ``longest`` tokens (empty, one
@@ -687,6 +692,10 @@ def test_skewed_decode_attention_finds_one_planted_key(ops, hq, hkv, d, short, l
     (16, 8, 128, [500], [600], None),            # the same with few workgroups: the per-head kernel
     (16, 4, 64, [2048, 2100], [0, 0], None),     # two prompts from position 0 in one step, 4 workgroups per tile
     (32, 8, 64, [512], [1536], None),            # 128 workgroups on 2,048 keys: grouped, two runs
+    (16, 4, 48, [2048], [0], None),              # head size 48: grouped, the second 32 dimensions half used
+    (24, 8, 80, [2100], [0], None),              # head size 80, three heads per kv head
+    (8, 8, 112, [700], [500], None),             # head size 112: the per-head kernel
+    (12, 4, 192, [600], [500], None),            # head size 192: grouped, one workgroup per compute unit
     (32, 8, 64, [512], [1000], None),            # 128 workgroups on fewer keys: the per-head kernel at this head size
     (32, 8, 64, [512], [7680], None),            # a portion of a long prompt: each tile's keys in four runs
     (32, 8, 128, [40], [16000], None),           # a short tail behind a long context: sixteen workgroups, fifteen runs each
@@ -723,6 +732,9 @@ def test_prefill_attention_in_each_form(ops, hq, hkv, d, new, old, window):
     (32, 8, 64, [700], [1330], None),               # grouped on a cached prefix
     (32, 8, 64, [300], [5000], None),               # grouped, the keys of a tile in five runs
     (24, 8, 128, [20, 300], [9000, 100], None),     # runs left empty
+    (24, 8, 112, [20, 300], [9000, 100], None),     # the same at head size 112
+    (32, 8, 48, [300], [5000], None),               # head size 48 in runs
+    (8, 2, 160, [100, 40], [5000, 300], None),      # head size 160 in runs
     (8, 8, 128, [100, 40], [5000, 300], None),      # the per-head kernel with runs
     (24, 8, 128, [2100, 1], [0, 77], None),
     (8, 2, 64, [70, 1, 1, 9], [0, 40, 130, 64], 33),        # windows whose first pages were given back
