@@ -209,9 +209,11 @@ py::tuple pack_step(py::array_t<int32_t, py::array::c_style> buffer, const py::s
     py::list group_offsets;
     for (const GroupLayout& g : lay.groups) group_offsets.append(py::make_tuple(g.table_off, g.write_slot, g.block_ids));
     return py::make_tuple(fits, lay.total, lay.tokens, lay.items, lay.logit_rows, lay.decode_items,
-                          lay.prefill_tiles, lay.pages, lay.max_kv_len, lay.decode_max_kv, lay.decode_sum_kv,
+                          lay.prefill_tiles, lay.prefill_blocks, lay.pages, lay.max_kv_len, lay.decode_max_kv,
+                          lay.decode_sum_kv,
                           py::make_tuple(lay.token_ids, lay.positions, lay.tok_item, lay.item_start, lay.item_pos0,
-                                         lay.item_end, lay.slots, lay.logit_rows_off, lay.dec_items, lay.pf_tiles),
+                                         lay.item_end, lay.slots, lay.logit_rows_off, lay.dec_items, lay.pf_tiles,
+                                         lay.pf_blocks),
                           group_offsets);
   } catch (const PackError& e) {
     std::string who;

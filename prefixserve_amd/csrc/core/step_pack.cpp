@@ -52,6 +52,7 @@ PackLayout plan_step(const std::vector<PackItem>& items, const std::vector<PackG
       lay.decode_sum_kv += end;
     } else {
       lay.prefill_tiles += ceil_div(n, lim.prefill_tile);
+      lay.prefill_blocks += ceil_div(n, lim.prefill_tile * kTilesPerBlock);
     }
     lay.pages += lim.static_pages >= 0 ? lim.static_pages : pages;
     lay.max_kv_len = std::max(lay.max_kv_len, end);
@@ -72,6 +73,7 @@ PackLayout plan_step(const std::vector<PackItem>& items, const std::vector<PackG
   lay.logit_rows_off = take(lay.logit_rows);
   lay.dec_items = take(lay.decode_items);
   lay.pf_tiles = take(2 * lay.prefill_tiles);
+  lay.pf_blocks = take(lay.prefill_blocks);
   lay.groups.resize(groups.size());
   for (GroupLayout& g : lay.groups) {
     g.table_off = take(lay.items + 1);
@@ -95,6 +97,8 @@ void fill_step(const std::vector<PackItem>& items, const std::vector<PackGroup>&
   int32_t* rows = buf + lay.logit_rows_off;
   int32_t* dec = buf + lay.dec_items;
   int32_t* tiles = buf + lay.pf_tiles;
+  int32_t* blocks = buf + lay.pf_blocks;
+  int64_t tile_count = 0;
 
   int64_t t0 = 0;
   item_start[0] = 0;
@@ -115,8 +119,10 @@ void fill_step(const std::vector<PackItem>& items, const std::vector<PackGroup>&
       *dec++ = static_cast<int32_t>(i);
     } else {
       for (int64_t q = 0; q < n; q += lim.prefill_tile) {
+        if (q % (lim.prefill_tile * kTilesPerBlock) == 0) *blocks++ = static_cast<int32_t>(tile_count);
         *tiles++ = static_cast<int32_t>(i);
         *tiles++ = static_cast<int32_t>(q);
+        ++tile_count;
       }
     }
     for (int64_t w = 0; w < it.want.size; ++w) *rows++ = static_cast<int32_t>(t0 + it.want.data[w]);

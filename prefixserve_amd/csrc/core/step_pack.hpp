@@ -45,6 +45,8 @@ struct PackLimits {
   int64_t static_pages = -1;  // >= 0: every item's table takes exactly this many entries
 };
 
+inline constexpr int64_t kTilesPerBlock = 4;   // tiles of queries in a block of the prefill list
+
 struct GroupLayout {
   int64_t table_off = 0, write_slot = 0, block_ids = 0;
 };
@@ -52,12 +54,15 @@ struct GroupLayout {
 struct PackLayout {
   int64_t total = 0;
   int64_t tokens = 0, items = 0, logit_rows = 0, decode_items = 0, prefill_tiles = 0, pages = 0;
+  // runs of up to kTilesPerBlock consecutive tiles of one item (a kernel whose workgroups take
+  // several tiles of queries at once finds its tiles through them)
+  int64_t prefill_blocks = 0;
   int64_t max_kv_len = 0;
   // over the items that bring one token: the longest context after the step and the sum of them
   int64_t decode_max_kv = 0, decode_sum_kv = 0;
   // offsets into the buffer, in 32-bit words
   int64_t token_ids = 0, positions = 0, tok_item = 0, item_start = 0, item_pos0 = 0, item_end = 0, slots = 0;
-  int64_t logit_rows_off = 0, dec_items = 0, pf_tiles = 0;
+  int64_t logit_rows_off = 0, dec_items = 0, pf_tiles = 0, pf_blocks = 0;
   std::vector<GroupLayout> groups;
 };
 

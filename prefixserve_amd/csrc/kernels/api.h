@@ -85,10 +85,13 @@ int psamd_attention_mfma_supports(int hq, int hkv, int head_dim);
 // part_o [32 * n_tiles * hq * nsplit * head_dim] and part_ml [32 * n_tiles * hq * nsplit * 2] carry
 // to a merge kernel.
 int psamd_attention_prefill_nsplit(int n_tiles, int max_kv_len, int hq, int hkv, int head_dim);
+// pf_tiles: (item, first query) of every tile of 32 queries; pf_blocks: the first tile of every run
+// of up to four consecutive tiles of one item, in the order of the tiles (n_blocks = 0: no such
+// list; steps with one or two query heads per kv head then run a slower form).
 // The most rows (32 * n_tiles * nsplit) of part_o / part_ml any step of this shape needs.
 int psamd_attention_prefill_part_rows(int hq, int hkv, int head_dim);
 int psamd_attention_prefill(void* stream, const void* qkv, int q_stride, void* out, const void* kv,
-                            const int32_t* pf_tiles, int n_tiles, int max_kv_len,
+                            const int32_t* pf_tiles, int n_tiles, const int32_t* pf_blocks, int n_blocks, int max_kv_len,
                             const int32_t* item_start, const int32_t* item_pos0,
                             const int32_t* table_off, const int32_t* block_ids, int hq, int hkv, int head_dim,
                             float scale, int window, float* part_o, float* part_ml, int nsplit);

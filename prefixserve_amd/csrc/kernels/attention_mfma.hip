@@ -354,7 +354,8 @@ __global__ __launch_bounds__(256 * KP, NS <= 4 ? 4 : 2) void attn_prefill_groupe
     const int32_t* __restrict__ pf_tiles, const int32_t* __restrict__ item_start,
     const int32_t* __restrict__ item_pos0, const int32_t* __restrict__ table_off,
     const int32_t* __restrict__ block_ids, int n_tiles, int hq, int hkv, int table_pages, float scale,
-    int window, float* __restrict__ part_o, float* __restrict__ part_ml, int pair_tiles) {
+    int window, float* __restrict__ part_o, float* __restrict__ part_ml, int pair_tiles, int tiles_per_wg,
+    const int32_t* __restrict__ pf_blocks, int n_blocks) {
   constexpr int D = 16 * NS;
   constexpr int DT = (D + 31) / 32;
   constexpr int KS = D + 8;                      // elements per key row in LDS
@@ -369,8 +370,15 @@ __global__ __launch_bounds__(256 * KP, NS <= 4 ? 4 : 2) void attn_prefill_groupe
   bf16_t* v_lds = k_lds + 2 * K_STAGE;
   int32_t* table = reinterpret_cast<int32_t*>(v_lds + 2 * V_STAGE);
 
+  // A workgroup's four head slots (wave & 3) are four query heads of the kv head on one tile of
+  // queries, or, with fewer query heads per kv head, two heads on two consecutive tiles or one
+  // head on four (tiles_per_wg = 1, 2, 4): the keys and values a workgroup stages are then still
+  // used by four waves. Its tiles are those of one item: pf_blocks lists the first tile of every
+  // run of up to four consecutive tiles of an item, and gridDim.y is the number of those runs
+  // times the workgroups that share one (two with two tiles each).
   const int group = hq / hkv;
-  const int wg_per_kv = (group + 3) >> 2;
+  const int heads_per_wg = 4 / tiles_per_wg;
+  const int wg_per_kv = (group + heads_per_wg - 1) / heads_per_wg;
   // Grid: x = (kv head, block of 4 query heads), y = tile, the late tiles (which see the most
   // keys) first. Workgroups are handed out in the order x + gridDim.x * y and go round robin over
   // the dies: the heaviest tiles of every head start first, so no head's long tiles are left
@@ -380,30 +388,52 @@ __global__ __launch_bounds__(256 * KP, NS <= 4 ? 4 : 2) void attn_prefill_groupe
   const int kvh = blockIdx.x / wg_per_kv;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int part = wave >> 2;                           // which of the iteration's KP runs of keys
-  const int head_in_group = (blockIdx.x - kvh * wg_per_kv) * 4 + (wave & 3);
-  const bool head_valid = head_in_group < group;       // a spare wave repeats the last head and writes nothing
+  const int slot = wave & 3;
+  const int head_in_group = (blockIdx.x - kvh * wg_per_kv) * heads_per_wg + slot % heads_per_wg;
+  const int tile_in_wg = slot / heads_per_wg;
+  bool head_valid = head_in_group < group;             // a spare wave repeats the last head and writes nothing
   const int h = kvh * group + min(head_in_group, group - 1);
   // pair_tiles (the whole grid runs at once, two workgroups to a compute unit): the second half
   // of the workgroups, which join the first half's on their compute units, take the early tiles in
   // ascending order, so that the longest tile shares its compute unit with the shortest and every
   // compute unit has about the same number of keys to go through.
   const int by = static_cast<int>(blockIdx.y), first_half = (n_tiles + 1) >> 1;
-  const int tile = (pair_tiles && by >= first_half) ? by - first_half : n_tiles - 1 - by;
-  const int item = pf_tiles[2 * tile];
-  const int q_off = pf_tiles[2 * tile + 1];
+  int wg_tile = (pair_tiles && by >= first_half) ? by - first_half : n_tiles - 1 - by;
+  int wg_q_off_more = 0;
+  if (tiles_per_wg > 1) {
+    const int sub = 4 / tiles_per_wg;                  // workgroups per run of four tiles
+    const int at = n_blocks * sub - 1 - by;            // late tiles first
+    wg_tile = pf_blocks[at / sub] + tiles_per_wg * (at % sub);
+    wg_q_off_more = 32 * tiles_per_wg * (at % sub);
+  }
+  const int item = pf_tiles[2 * (wg_tile - (wg_q_off_more >> 5))];
+  const int wg_q_off = pf_tiles[2 * (wg_tile - (wg_q_off_more >> 5)) + 1] + wg_q_off_more;
   const int t0 = item_start[item];
   const int n = item_start[item + 1] - t0;
+  if (wg_q_off >= n) return;                           // the run ends before this workgroup's tiles
   const int pos0 = item_pos0[item];
   const int col = lane & 31, hi = lane >> 5;
 
+  // This wave's tile: a block's tiles past the end of the item do not exist, the wave then
+  // repeats the block's first tile and writes nothing.
+  int tile = wg_tile, q_off = wg_q_off;
+  if (tile_in_wg > 0) {
+    if (wg_q_off + 32 * tile_in_wg < n) {
+      tile = wg_tile + tile_in_wg;
+      q_off = wg_q_off + 32 * tile_in_wg;
+    } else {
+      head_valid = false;
+    }
+  }
   const int qi = min(q_off + col, n - 1);          // lanes past the end repeat the last query
   const bool q_valid = q_off + col < n;
   const int q_pos = pos0 + qi;
-  const int first_pos = pos0 + q_off;
+  const int first_pos = pos0 + q_off;                          // of this wave's tile
   const int last_pos = pos0 + min(q_off + 31, n - 1);
+  const int wg_last_pos = pos0 + min(wg_q_off + 32 * tiles_per_wg - 1, n - 1);   // of the block
   const int k_lo_q = window > 0 ? max(0, q_pos - window + 1) : 0;
   const int max_key = pos0 + n - 1;
-  const int k_begin_vis = window > 0 ? max(0, first_pos - window + 1) : 0;   // the first key any query of the tile sees
+  const int k_begin_vis = window > 0 ? max(0, pos0 + wg_q_off - window + 1) : 0;   // the first key any query of the block sees
   const int k_begin = k_begin_vis & ~(KEYS - 1);
   const float c = scale * 1.44269504088896340736f;  // scores are exponentiated in base 2
   // With gridDim.z > 1 the tile's keys are dealt out to that many workgroups in runs of whole
@@ -411,16 +441,16 @@ __global__ __launch_bounds__(256 * KP, NS <= 4 ? 4 : 2) void attn_prefill_groupe
   // maximum and its unnormalized output in part_ml / part_o for the merge kernel. A tile with
   // too few keys for all of them leaves the last ones nothing: they write an empty sum.
   const int nsplit = gridDim.z;
-  int k_first = k_begin, k_last = last_pos;
+  int k_first = k_begin, k_last = wg_last_pos;
   int64_t part_slot = 0;
   if (nsplit > 1) {
     constexpr int PAIR = 2 * KEYS;
-    const int pairs = (last_pos - k_begin) / PAIR + 1;
+    const int pairs = (wg_last_pos - k_begin) / PAIR + 1;
     const int per = max((pairs + nsplit - 1) / nsplit, kMinSplitKeys / PAIR);
     k_first = k_begin + static_cast<int>(blockIdx.z) * per * PAIR;
-    k_last = min(last_pos, k_first + per * PAIR - 1);
+    k_last = min(wg_last_pos, k_first + per * PAIR - 1);
     part_slot = (static_cast<int64_t>(tile * 32 + col) * hq + h) * nsplit + blockIdx.z;
-    if (k_first > last_pos) {
+    if (k_first > wg_last_pos) {
       if (part == 0 && head_valid && q_valid && hi == 0) {
         part_ml[2 * part_slot] = -INFINITY;
         part_ml[2 * part_slot + 1] = 0.f;
@@ -430,7 +460,7 @@ __global__ __launch_bounds__(256 * KP, NS <= 4 ? 4 : 2) void attn_prefill_groupe
   }
   {
     const int32_t* gtable = block_ids + table_off[item];
-    for (int i = threadIdx.x; i <= (last_pos >> 4); i += blockDim.x) table[i] = gtable[i];
+    for (int i = threadIdx.x; i <= (wg_last_pos >> 4); i += blockDim.x) table[i] = gtable[i];
   }
   __syncthreads();
 
@@ -462,7 +492,7 @@ __global__ __launch_bounds__(256 * KP, NS <= 4 ? 4 : 2) void attn_prefill_groupe
       const int p = threadIdx.x + THREADS * i;
       if (CHUNKS % THREADS == 0 || p < CHUNKS) {
         const int page = p / (2 * D), rem = p - page * 2 * D;
-        const int64_t base = static_cast<int64_t>(table[min(k0 + 16 * page, last_pos) >> 4]) * page_elems;
+        const int64_t base = static_cast<int64_t>(table[min(k0 + 16 * page, wg_last_pos) >> 4]) * page_elems;
         const bf16_t* src = kv + base + 8 * rem;
         r.k[i] = *reinterpret_cast<const u32x4*>(src + khead);
         r.v[i] = *reinterpret_cast<const u32x4*>(src + vhead);
@@ -1009,13 +1039,14 @@ static bool lds_allowed(Kernel kernel, size_t bytes) {
 // prefix.
 enum class PrefillForm { kPerHead, kGrouped };
 
+// With one or two query heads per kv head a workgroup of the grouped kernel takes four or two
+// consecutive tiles of queries, so that four waves still share the keys and values it stages.
+static int prefill_tiles_per_wg(int group) { return group == 1 ? 4 : (group == 2 ? 2 : 1); }
+
 static PrefillForm prefill_form(int n_tiles, int hq, int hkv, int head_dim) {
   const int group = hq / hkv;
-  const int64_t workgroups = static_cast<int64_t>(n_tiles) * hkv * ((group + 3) / 4);
-  // Two query heads per kv head leave half of the grouped kernel's waves idle; sharing the keys
-  // and values still pays above head size 64 from one workgroup per compute unit on (16 heads on
-  // 8 at head size 128: 2,048 tokens 71 -> 55 us, 8,192 tokens 779 -> 647; at head size 64 a tie).
-  if (group < 2 || (group == 2 && (head_dim <= 64 || workgroups < 256))) return PrefillForm::kPerHead;
+  const int tiles = prefill_tiles_per_wg(group), heads = 4 / tiles;
+  const int64_t workgroups = ceil_div(n_tiles, tiles) * hkv * ceil_div(group, heads);
   return workgroups <= (head_dim <= 64 ? 128 : 80) ? PrefillForm::kPerHead : PrefillForm::kGrouped;
 }
 
@@ -1071,22 +1102,26 @@ static int prefill_nsplit(int n_tiles, int max_kv_len, int hq, int hkv, int head
 
 template <int NS>
 static int launch_prefill(hipStream_t s, const void* qkv, int q_stride, void* out, const void* kv,
-                          const int32_t* pf_tiles, int n_tiles, int table_pages,
+                          const int32_t* pf_tiles, int n_tiles, const int32_t* pf_blocks, int n_blocks, int table_pages,
                           const int32_t* item_start, const int32_t* item_pos0,
                           const int32_t* table_off, const int32_t* block_ids, int hq, int hkv, float scale, int window,
                           float* part_o, float* part_ml, int nsplit) {
   const int group = hq / hkv;
-  const PrefillForm form = nsplit > 1 ? (group <= 2 ? PrefillForm::kPerHead : PrefillForm::kGrouped)
-                                      : prefill_form(n_tiles, hq, hkv, 16 * NS);
+  // Without the list of runs of tiles, one or two query heads per kv head go to the per-head kernel.
+  const PrefillForm form = nsplit > 1 || (group <= 2 && n_blocks == 0)
+                               ? (group <= 2 ? PrefillForm::kPerHead : PrefillForm::kGrouped)
+                               : prefill_form(n_tiles, hq, hkv, 16 * NS);
   // The heads of a kv head share its keys and values through LDS, two waves per head (each its
   // own run of keys) if the stages fit, else one.
   if (form != PrefillForm::kPerHead) {
-    const dim3 grid(hkv * ((group + 3) / 4), n_tiles, nsplit);
+    const int tiles_per_wg = nsplit == 1 ? prefill_tiles_per_wg(group) : 1, heads_per_wg = 4 / tiles_per_wg;
+    const dim3 grid(hkv * ((group + heads_per_wg - 1) / heads_per_wg), tiles_per_wg == 1 ? n_tiles : n_blocks * heads_per_wg,
+                    nsplit);
     // More than one workgroup per compute unit but no more than run at once (two of eight waves
     // up to head size 64): see pair_tiles in the kernel.
     const int64_t wgs = static_cast<int64_t>(grid.x) * grid.y;
     // (2,048 tokens at head size 64, 32 heads on 8: 37.6 -> 35.1 us; on 2,048 cached keys 80 -> 74.)
-    const int pair = (NS <= 4 && nsplit == 1 && wgs > 256 && wgs <= 512 && grid.x % 8 == 0) ? 1 : 0;
+    const int pair = (NS <= 4 && nsplit == 1 && tiles_per_wg == 1 && wgs > 256 && wgs <= 512 && grid.x % 8 == 0) ? 1 : 0;
 #define PSAMD_GROUPED(KP_)                                                                                         \
   {                                                                                                               \
     const size_t smem = grouped_smem(16 * NS, 1, KP_, table_pages);                                               \
@@ -1094,7 +1129,7 @@ static int launch_prefill(hipStream_t s, const void* qkv, int q_stride, void* ou
       attn_prefill_grouped_kernel<NS, 1, KP_><<<grid, dim3(256 * KP_), smem, s>>>(                                \
           static_cast<const bf16_t*>(qkv), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(kv),   \
           pf_tiles, item_start, item_pos0, table_off, block_ids, n_tiles, hq, hkv, table_pages, scale, window,   \
-          part_o, part_ml, pair);                                                                                 \
+          part_o, part_ml, pair, tiles_per_wg, pf_blocks, n_blocks);                                              \
       const int rc = check_launch("psamd_attention_prefill");                                                     \
       if (rc != 0 || nsplit == 1) return rc;                                                                      \
       return launch_prefill_merge(s, part_o, part_ml, out, pf_tiles, item_start, n_tiles, hq, 16 * NS, nsplit);   \
@@ -1104,7 +1139,7 @@ static int launch_prefill(hipStream_t s, const void* qkv, int q_stride, void* ou
     // workgroups per compute unit's worth of tiles run 5% faster as two workgroups of four waves
     // (one wave per head): two barriers' worth of waves that do not wait for each other
     // (head size 128: 4,096 tokens 181 -> 171 us, 8,192 tokens 657 -> 623 us; 2,048 tokens 56 -> 67).
-    if (NS < 6 || static_cast<int64_t>(grid.x) * grid.y * grid.z < 1024) PSAMD_GROUPED(2)
+    if (NS < 6 || wgs * grid.z < 1024) PSAMD_GROUPED(2)
     PSAMD_GROUPED(1)
 #undef PSAMD_GROUPED
   }
@@ -1181,11 +1216,14 @@ int psamd_attention_prefill_part_rows(int hq, int hkv, int head_dim) {
   return 32 * tiles_times_runs;
 }
 
+// pf_tiles: (item, first query) of every tile of 32 queries; pf_blocks: the first tile of every run
+// of up to four consecutive tiles of one item, in the order of the tiles (n_blocks = 0: no such
+// list; steps with one or two query heads per kv head then run a slower form).
 // max_kv_len: the longest request of the step after it (sizes the block table staged in LDS).
 // nsplit: 1, or what psamd_attention_prefill_nsplit gave for these sizes (or less); part_o then
 // has room for 32 * n_tiles * hq * nsplit * head_dim floats and part_ml for 32 * n_tiles * hq * nsplit * 2.
 int psamd_attention_prefill(void* stream, const void* qkv, int q_stride, void* out, const void* kv,
-                            const int32_t* pf_tiles, int n_tiles, int max_kv_len,
+                            const int32_t* pf_tiles, int n_tiles, const int32_t* pf_blocks, int n_blocks, int max_kv_len,
                             const int32_t* item_start,
                             const int32_t* item_pos0, const int32_t* table_off, const int32_t* block_ids, int hq,
                             int hkv, int head_dim, float scale, int window, float* part_o, float* part_ml, int nsplit) {
@@ -1194,12 +1232,14 @@ int psamd_attention_prefill(void* stream, const void* qkv, int q_stride, void* o
   PSAMD_REQUIRE(max_kv_len >= 1 && max_kv_len <= 8192 * kPage, "context too long for the block table staged in LDS");
   if (n_tiles == 0) return 0;
   PSAMD_REQUIRE(n_tiles <= 65535, "too many query tiles for one launch");
+  PSAMD_REQUIRE(n_blocks >= 0 && n_blocks <= n_tiles && (n_blocks == 0 || (pf_blocks != nullptr && 4LL * n_blocks >= n_tiles)),
+                "the runs of tiles must cover the tiles, four at most each");
   PSAMD_REQUIRE(nsplit >= 1 && nsplit <= kMaxPrefillSplit, "nsplit must be in [1, 16]");
   PSAMD_REQUIRE(nsplit == 1 || (part_o != nullptr && part_ml != nullptr), "split keys need part_o and part_ml");
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int table_pages = static_cast<int>(ceil_div(max_kv_len, kPage));
 #define PSAMD_PF(NS_)                                                                                           \
-  return launch_prefill<NS_>(s, qkv, q_stride, out, kv, pf_tiles, n_tiles, table_pages, item_start, \
+  return launch_prefill<NS_>(s, qkv, q_stride, out, kv, pf_tiles, n_tiles, pf_blocks, n_blocks, table_pages, item_start, \
                              item_pos0, table_off, block_ids, hq, hkv, scale, window, part_o, part_ml, nsplit)
   switch (head_dim / 16) {
     case 1: PSAMD_PF(1);

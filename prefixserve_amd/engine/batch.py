@@ -62,6 +62,7 @@ class StepContext:
     num_logit_rows: int
     num_decode: int            # items with exactly one token (served by the decode kernel)
     num_prefill_tiles: int
+    num_prefill_blocks: int
     max_kv_len: int
     decode_skewed: bool        # the kernels' verdict on the single-token items' context lengths (one far longer than the rest)
     token_ids: torch.Tensor    # [T]
@@ -74,6 +75,7 @@ class StepContext:
     logit_rows: torch.Tensor   # [S] flat token rows
     dec_items: torch.Tensor    # [num_decode] item indices
     pf_tiles: torch.Tensor     # [num_prefill_tiles, 2] (item, first query of the tile within the item)
+    pf_blocks: torch.Tensor    # [num_prefill_blocks] the first tile of each run of up to four consecutive tiles of an item
     groups: list[GroupArrays]
     keys: list[Hashable]
     want_counts: list[int]
@@ -128,21 +130,21 @@ class StepPacker:
                                       self.num_slots, self.prefill_tile, static_pages)
         except ValueError as e:
             raise EngineError(str(e)) from None
-        _, total, t_n, b, s_n, n_dec, n_tiles, p_total, max_kv_len, dec_max_kv, dec_sum_kv, offs, group_offs = res
-        o_ids, o_pos, o_item, o_start, o_pos0, o_end, o_slots, o_rows, o_dec, o_tiles = offs
+        _, total, t_n, b, s_n, n_dec, n_tiles, n_blocks, p_total, max_kv_len, dec_max_kv, dec_sum_kv, offs, group_offs = res
+        o_ids, o_pos, o_item, o_start, o_pos0, o_end, o_slots, o_rows, o_dec, o_tiles, o_blocks = offs
 
         if self.on_gpu:
             self._dev[:total].copy_(self._host[:total], non_blocking=True)
             assert self._copied is not None
             self._copied.record()
         # The views depend on the layout only, and a decoding batch keeps its layout for many steps.
-        sig = (self.version, t_n, b, s_n, n_dec, n_tiles, p_total, offs, tuple(group_offs))
+        sig = (self.version, t_n, b, s_n, n_dec, n_tiles, n_blocks, p_total, offs, tuple(group_offs))
         if self._views is None or self._views[0] != sig:
             dev, buf = self._dev, self._host_np
             named = {"token_ids": (o_ids, t_n), "positions": (o_pos, t_n), "tok_item": (o_item, t_n),
                      "item_start": (o_start, b + 1), "item_pos0": (o_pos0, b), "item_end": (o_end, b),
                      "slots": (o_slots, b), "logit_rows": (o_rows, s_n), "dec_items": (o_dec, n_dec),
-                     "pf_tiles": (o_tiles, 2 * n_tiles)}
+                     "pf_tiles": (o_tiles, 2 * n_tiles), "pf_blocks": (o_blocks, n_blocks)}
             on_dev = {k: dev[o:o + n] for k, (o, n) in named.items()}
             on_dev["pf_tiles"] = on_dev["pf_tiles"].view(n_tiles, 2)
             host = {k: buf[o:o + n] for k, (o, n) in named.items()}
@@ -153,7 +155,7 @@ class StepPacker:
         skewed = bool(self._skew_rule(n_dec, dec_max_kv, dec_sum_kv)) if self._skew_rule is not None and n_dec > 1 else False
         return StepContext(
             num_tokens=t_n, num_items=b, num_logit_rows=s_n, num_decode=n_dec, num_prefill_tiles=n_tiles,
-            max_kv_len=max_kv_len, decode_skewed=skewed, groups=groups,
+            num_prefill_blocks=n_blocks, max_kv_len=max_kv_len, decode_skewed=skewed, groups=groups,
             keys=[it.key for it in items],
             want_counts=[len(it.want) for it in items], host=host, **on_dev,
         )

@@ -63,8 +63,8 @@ _SIGNATURES = {
     "psamd_attention_decode_skewed": [_i32, _i32, _i64],
     "psamd_attention_decode_plan": [_i32, _i32, _i32, _i32, _i32, _vp, _vp],
     "psamd_attention_decode_max_parts": [_i32],
-    "psamd_attention_prefill": [_vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _f32,
-                                _i32, _vp, _vp, _i32],
+    "psamd_attention_prefill": [_vp, _vp, _i32, _vp, _vp, _vp, _i32, _vp, _i32, _i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32,
+                                _f32, _i32, _vp, _vp, _i32],
     "psamd_attention_decode": [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32,
                                _i32, _f32, _i32, _i32],
     "psamd_sample": [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32],
@@ -428,7 +428,7 @@ class HipOps:
                     self._need(32 * ctx.num_prefill_tiles * nsplit <= rows, "attention: more split tiles than planned for")
                 self._ok(self.lib.psamd_attention_prefill(
                     s, qkv.data_ptr(), stride, out.data_ptr(), kv.data_ptr(), ctx.pf_tiles.data_ptr(),
-                    ctx.num_prefill_tiles, kv_len,
+                    ctx.num_prefill_tiles, ctx.pf_blocks.data_ptr(), ctx.num_prefill_blocks, kv_len,
                     ctx.item_start.data_ptr(), ctx.item_pos0.data_ptr(),
                     g.table_off.data_ptr(), g.block_ids.data_ptr(), hq, hkv, d, scale, win,
                     part_o.data_ptr() if nsplit > 1 else None, part_ml.data_ptr() if nsplit > 1 else None, nsplit))

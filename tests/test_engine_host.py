@@ -87,6 +87,12 @@ def test_packer_layout():
     assert ctx.positions[:20].tolist() == list(range(30, 50)) and ctx.positions[20].item() == 16   # absolute
     assert ctx.logit_rows.tolist() == [19, 20] and ctx.dec_items.tolist() == [1]
     assert ctx.pf_tiles.tolist() == [[0, 0], [2, 0], [2, 128]]
+    assert ctx.num_prefill_blocks == 2 and ctx.pf_blocks.tolist() == [0, 1]     # runs of up to four tiles, one item each
+    small = StepPacker(torch.device("cpu"), [GroupMeta(32)], vocab_size=200, max_position=256, num_slots=4, prefill_tile=8)
+    many = small.pack([StepItem("a", [1] * 70, 0, [list(range(5))], slot=0), StepItem("b", [1], 3, [[9]], slot=1),
+                       StepItem("c", [1] * 33, 0, [list(range(10, 13))], slot=2), StepItem("d", [1] * 2, 40, [[20, 21, 22]], slot=3)])
+    assert many.num_prefill_tiles == 9 + 5 + 1 and many.pf_blocks.tolist() == [0, 4, 8, 9, 13, 14]
+    assert [many.pf_tiles[t].tolist() for t in many.pf_blocks.tolist()] == [[0, 0], [0, 32], [0, 64], [2, 0], [2, 32], [3, 0]]
     g = ctx.groups[0]
     assert g.table_off.tolist() == [0, 4, 6, 15] and g.block_ids[:6].tolist() == [5, 6, 7, 8, 9, 3]
     assert g.write_slot[0].item() == 6 * 16 + 14 and g.write_slot[2].item() == 7 * 16 + 0   # pos 30 -> page 1 (id 6)

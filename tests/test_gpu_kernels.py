@@ -715,6 +715,16 @@ def test_skewed_decode_attention_finds_one_planted_key(ops, hq, hkv, d, short, l
     (32, 8, 64, [2048], [0], 300),               # a long prompt with a window
     (32, 8, 64, [100], [1948], None),            # few tiles: grouped, four runs of 512 keys
     (32, 8, 64, [100], [600], None),             # few tiles on few keys: the per-head kernel
+    # One or two query heads per kv head: a workgroup of the grouped kernel takes four or two
+    # consecutive tiles of an item; items that end inside such a run, beside single tokens
+    (32, 32, 64, [300, 70, 1, 2, 129], [0, 500, 77, 40, 1000], None),
+    (32, 16, 128, [300, 70, 1, 2, 129], [0, 500, 77, 40, 1000], None),
+    (16, 16, 128, [2100], [0], None),            # a last run of two tiles, the second of 20 queries
+    (16, 8, 64, [2048 + 33], [0], None),         # a last run of one tile
+    (32, 32, 48, [1000, 600], [24, 0], None),
+    (32, 32, 64, [700, 300, 1], [150, 0, 900], 100),     # with a window
+    (32, 16, 64, [2048], [300], 300),
+    (8, 8, 128, [700], [500], None),             # too few workgroups for that: the per-head kernel
 ])
 def test_prefill_attention_in_each_form(ops, hq, hkv, d, new, old, window):
     """The portions of a step go to the per-head or to the grouped kernel by their number of tiles
@@ -737,6 +747,8 @@ def test_prefill_attention_in_each_form(ops, hq, hkv, d, new, old, window):
     (8, 2, 160, [100, 40], [5000, 300], None),      # head size 160 in runs
     (8, 8, 128, [100, 40], [5000, 300], None),      # the per-head kernel with runs
     (24, 8, 128, [2100, 1], [0, 77], None),
+    (32, 32, 64, [300, 70, 1, 2, 129], [0, 500, 77, 40, 1000], None),     # grouped, four tiles per workgroup
+    (32, 16, 128, [700, 300, 1], [150, 0, 900], 100),                      # two tiles per workgroup, a window
     (8, 2, 64, [70, 1, 1, 9], [0, 40, 130, 64], 33),        # windows whose first pages were given back
     (16, 4, 64, [700, 300, 1], [150, 0, 900], 100),
     (32, 8, 64, [2040], [300], 300),
