@@ -1043,11 +1043,21 @@ enum class PrefillForm { kPerHead, kGrouped };
 // consecutive tiles of queries, so that four waves still share the keys and values it stages.
 static int prefill_tiles_per_wg(int group) { return group == 1 ? 4 : (group == 2 ? 2 : 1); }
 
-static PrefillForm prefill_form(int n_tiles, int hq, int hkv, int head_dim) {
+// Workgroups of the grouped kernel for a step of n_tiles tiles (a run of tiles that ends early
+// adds one per item: the estimate is for choosing a form, not for a grid).
+static int64_t grouped_workgroups(int n_tiles, int hq, int hkv) {
   const int group = hq / hkv;
   const int tiles = prefill_tiles_per_wg(group), heads = 4 / tiles;
-  const int64_t workgroups = ceil_div(n_tiles, tiles) * hkv * ceil_div(group, heads);
-  return workgroups <= (head_dim <= 64 ? 128 : 80) ? PrefillForm::kPerHead : PrefillForm::kGrouped;
+  return ceil_div(n_tiles, tiles) * hkv * ceil_div(group, heads);
+}
+
+// Few enough of them that the per-head kernel, with four times as many, does better.
+static bool few_grouped_workgroups(int n_tiles, int hq, int hkv, int head_dim) {
+  return grouped_workgroups(n_tiles, hq, hkv) <= (head_dim <= 64 ? 128 : 80);
+}
+
+static PrefillForm prefill_form(int n_tiles, int hq, int hkv, int head_dim) {
+  return few_grouped_workgroups(n_tiles, hq, hkv, head_dim) ? PrefillForm::kPerHead : PrefillForm::kGrouped;
 }
 
 static int launch_prefill_merge(hipStream_t s, const float* part_o, const float* part_ml, void* out,
@@ -1072,18 +1082,8 @@ static int launch_prefill_merge(hipStream_t s, const float* part_o, const float*
 // compute unit itself (256 on 1,792: 17 -> 20 with four); where the grouped kernel would run
 // without a cut, two runs pay from 4,096 keys on (512 on 3,584 at head size 128: 78 -> 58) and,
 // above 128 workgroups, from 8,192 on (1,024 on 3,072: 56 -> 60; on 15,000: 199 -> 183).
-static int prefill_nsplit(int n_tiles, int max_kv_len, int hq, int hkv, int head_dim) {
-  const int group = hq / hkv;
-  if (group <= 2) {
-    // The per-head kernel, a workgroup per (tile, query head): runs of 1,024 keys or more, up to
-    // one workgroup per compute unit (more lost again). 32 heads on 32 at head size 128: 64 tokens
-    // on 4,032 cached 51 -> 26 us, 20 on 16,000 172 -> 56; 16 heads on 8: 256 on 7,936 93 -> 57,
-    // 256 on 60,000 622 -> 323.
-    const int64_t workgroups = static_cast<int64_t>(n_tiles) * hq;
-    if (2 * workgroups > 256) return 1;
-    return static_cast<int>(std::max<int64_t>(1, std::min<int64_t>({256 / workgroups, max_kv_len / 1024, 16})));
-  }
-  const int64_t workgroups = static_cast<int64_t>(n_tiles) * hkv * ((group + 3) / 4);
+static int grouped_nsplit(int n_tiles, int max_kv_len, int hq, int hkv, int head_dim) {
+  const int64_t workgroups = grouped_workgroups(n_tiles, hq, hkv);
   const int at_once = head_dim <= 64 ? 512 : 256;
   if (2 * workgroups > at_once) return 1;
   if (grouped_smem(head_dim, 1, 1, static_cast<int>(ceil_div(max_kv_len, kPage))) > 160 * 1024) return 1;
@@ -1091,7 +1091,7 @@ static int prefill_nsplit(int n_tiles, int max_kv_len, int hq, int hkv, int head
   // 64 / 128: 43 -> 36 / 70 -> 54 us; on 1,536 cached 30 -> 28 / 44 -> 41).
   if (workgroups > 64 && workgroups <= 128 && max_kv_len >= 2048 && max_kv_len < 4096) return 2;
   const int nsplit = static_cast<int>(std::min<int64_t>({at_once / workgroups, max_kv_len / kMinSplitKeys, kMaxPrefillSplit}));
-  const bool per_head_else = workgroups <= (head_dim <= 64 ? 128 : 80);
+  const bool per_head_else = few_grouped_workgroups(n_tiles, hq, hkv, head_dim);
   if (per_head_else) {
     if (nsplit < 4 || (static_cast<int64_t>(n_tiles) * hq >= 256 && max_kv_len < 4096)) return 1;
   } else if (max_kv_len < (workgroups <= 128 ? 4096 : 8192)) {
@@ -1100,21 +1100,42 @@ static int prefill_nsplit(int n_tiles, int max_kv_len, int hq, int hkv, int head
   return std::max(nsplit, 1);
 }
 
+// The same for the per-head kernel, a workgroup per (tile, query head), which takes the steps
+// with one or two query heads per kv head that the grouped kernel (four or two tiles of queries
+// per workgroup then) neither cuts nor has enough workgroups for: runs of 1,024 keys or more, up
+// to one workgroup per compute unit (more lost again). 32 heads on 32 at head size 128: 64 tokens
+// on 4,032 cached 51 -> 26 us, 20 on 16,000 172 -> 56; 16 heads on 8: 256 on 7,936 93 -> 57,
+// 256 on 60,000 622 -> 323.
+static int per_head_nsplit(int n_tiles, int max_kv_len, int hq) {
+  const int64_t workgroups = static_cast<int64_t>(n_tiles) * hq;
+  if (2 * workgroups > 256) return 1;
+  return static_cast<int>(std::max<int64_t>(1, std::min<int64_t>({256 / workgroups, max_kv_len / 1024, 16})));
+}
+
+static int prefill_nsplit(int n_tiles, int max_kv_len, int hq, int hkv, int head_dim) {
+  const int cut = grouped_nsplit(n_tiles, max_kv_len, hq, hkv, head_dim);
+  if (hq / hkv > 2 || cut > 1 || !few_grouped_workgroups(n_tiles, hq, hkv, head_dim)) return cut;
+  return per_head_nsplit(n_tiles, max_kv_len, hq);
+}
+
 template <int NS>
 static int launch_prefill(hipStream_t s, const void* qkv, int q_stride, void* out, const void* kv,
-                          const int32_t* pf_tiles, int n_tiles, const int32_t* pf_blocks, int n_blocks, int table_pages,
+                          const int32_t* pf_tiles, int n_tiles, const int32_t* pf_blocks, int n_blocks, int max_kv_len,
                           const int32_t* item_start, const int32_t* item_pos0,
                           const int32_t* table_off, const int32_t* block_ids, int hq, int hkv, float scale, int window,
                           float* part_o, float* part_ml, int nsplit) {
   const int group = hq / hkv;
-  // Without the list of runs of tiles, one or two query heads per kv head go to the per-head kernel.
-  const PrefillForm form = nsplit > 1 || (group <= 2 && n_blocks == 0)
-                               ? (group <= 2 ? PrefillForm::kPerHead : PrefillForm::kGrouped)
-                               : prefill_form(n_tiles, hq, hkv, 16 * NS);
+  const int table_pages = static_cast<int>(ceil_div(max_kv_len, kPage));
+  // One or two query heads per kv head: the per-head kernel without the list of runs of tiles, and
+  // where the keys are cut by its rule and not by the grouped kernel's.
+  const bool small_per_head =
+      group <= 2 && (n_blocks == 0 || (nsplit > 1 && grouped_nsplit(n_tiles, max_kv_len, hq, hkv, 16 * NS) == 1));
+  const PrefillForm form = nsplit > 1 || small_per_head ? (small_per_head ? PrefillForm::kPerHead : PrefillForm::kGrouped)
+                                                        : prefill_form(n_tiles, hq, hkv, 16 * NS);
   // The heads of a kv head share its keys and values through LDS, two waves per head (each its
   // own run of keys) if the stages fit, else one.
   if (form != PrefillForm::kPerHead) {
-    const int tiles_per_wg = nsplit == 1 ? prefill_tiles_per_wg(group) : 1, heads_per_wg = 4 / tiles_per_wg;
+    const int tiles_per_wg = prefill_tiles_per_wg(group), heads_per_wg = 4 / tiles_per_wg;
     const dim3 grid(hkv * ((group + heads_per_wg - 1) / heads_per_wg), tiles_per_wg == 1 ? n_tiles : n_blocks * heads_per_wg,
                     nsplit);
     // More than one workgroup per compute unit but no more than run at once (two of eight waves
@@ -1212,7 +1233,10 @@ int psamd_attention_prefill_part_rows(int hq, int hkv, int head_dim) {
   const int group = hq / hkv;
   // grouped kernel: tiles * runs * hkv * ceil(group / 4) <= 512 (256 above head size 64; two runs
   // for up to 128 workgroups stay below it too); per-head kernel: tiles * runs * hq <= 256.
-  const int tiles_times_runs = group <= 2 ? std::max(1, 256 / hq) : std::max(1, 512 / (hkv * ((group + 3) / 4)));
+  // With one or two query heads per kv head the grouped kernel's workgroups take four or two tiles:
+  // tiles * runs * hq <= 4 * 512 (4 * 256 above head size 64).
+  const int tiles_times_runs = group <= 2 ? std::max(1, 4 * (head_dim <= 64 ? 512 : 256) / hq)
+                                          : std::max(1, 512 / (hkv * ((group + 3) / 4)));
   return 32 * tiles_times_runs;
 }
 
@@ -1237,9 +1261,8 @@ int psamd_attention_prefill(void* stream, const void* qkv, int q_stride, void* o
   PSAMD_REQUIRE(nsplit >= 1 && nsplit <= kMaxPrefillSplit, "nsplit must be in [1, 16]");
   PSAMD_REQUIRE(nsplit == 1 || (part_o != nullptr && part_ml != nullptr), "split keys need part_o and part_ml");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const int table_pages = static_cast<int>(ceil_div(max_kv_len, kPage));
 #define PSAMD_PF(NS_)                                                                                           \
-  return launch_prefill<NS_>(s, qkv, q_stride, out, kv, pf_tiles, n_tiles, pf_blocks, n_blocks, table_pages, item_start, \
+  return launch_prefill<NS_>(s, qkv, q_stride, out, kv, pf_tiles, n_tiles, pf_blocks, n_blocks, max_kv_len, item_start, \
                              item_pos0, table_off, block_ids, hq, hkv, scale, window, part_o, part_ml, nsplit)
   switch (head_dim / 16) {
     case 1: PSAMD_PF(1);

@@ -725,6 +725,11 @@ def test_skewed_decode_attention_finds_one_planted_key(ops, hq, hkv, d, short, l
     (32, 32, 64, [700, 300, 1], [150, 0, 900], 100),     # with a window
     (32, 16, 64, [2048], [300], 300),
     (8, 8, 128, [700], [500], None),             # too few workgroups for that: the per-head kernel
+    (32, 32, 128, [512], [7680], None),          # four tiles per workgroup, each run of tiles' keys in two runs
+    (32, 32, 64, [500], [7680], None),           # the same in four runs, a last run of tiles that ends early
+    (32, 16, 128, [20, 300], [9000, 100], None), # two tiles per workgroup, runs of keys that a short request leaves empty
+    (16, 16, 64, [64], [5000], 1500),            # runs of keys inside a window
+    (16, 8, 64, [90], [4100], None),             # few workgroups: the per-head kernel, with its own runs
 ])
 def test_prefill_attention_in_each_form(ops, hq, hkv, d, new, old, window):
     """The portions of a step go to the per-head or to the grouped kernel by their number of tiles
@@ -749,6 +754,7 @@ def test_prefill_attention_in_each_form(ops, hq, hkv, d, new, old, window):
     (24, 8, 128, [2100, 1], [0, 77], None),
     (32, 32, 64, [300, 70, 1, 2, 129], [0, 500, 77, 40, 1000], None),     # grouped, four tiles per workgroup
     (32, 16, 128, [700, 300, 1], [150, 0, 900], 100),                      # two tiles per workgroup, a window
+    (32, 32, 64, [500], [7690], None),                                     # four tiles per workgroup, keys in runs
     (8, 2, 64, [70, 1, 1, 9], [0, 40, 130, 64], 33),        # windows whose first pages were given back
     (16, 4, 64, [700, 300, 1], [150, 0, 900], 100),
     (32, 8, 64, [2040], [300], 300),
