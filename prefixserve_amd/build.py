@@ -141,7 +141,7 @@ def build_core() -> Path:
     return out
 
 
-def build_core_program(main_source: Path, out: Path, sanitize: bool = False) -> Path:
+def build_core_program(main_source: Path, out: Path, sanitize: bool = False, what: str = "core check program") -> Path:
     """A standalone program from ``main_source`` and the core's sources without the Python
     bindings, for checks of the core that run without an interpreter: with ``sanitize`` the
     address and undefined-behaviour sanitizers are compiled in (host code only; a sanitized
@@ -150,7 +150,7 @@ def build_core_program(main_source: Path, out: Path, sanitize: bool = False) -> 
     sources = [str(CSRC / s) for s in CORE_SOURCES if not s.endswith("bindings.cpp")]
     cmd = [gxx, "-std=c++17", *CORE_WARNINGS, *(SANITIZE_FLAGS if sanitize else ["-O2"]), f"-I{CSRC / 'core'}",
            str(main_source), *sources, "-o", str(out)]
-    _run(cmd, f"core check program{' (sanitizers)' if sanitize else ''}")
+    _run(cmd, f"{what}{' (sanitizers)' if sanitize else ''}")
     return out
 
 

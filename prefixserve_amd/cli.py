@@ -8,6 +8,7 @@ The reference's entry is an HTTP server; this one generates from token ids and p
 
   generate       run prompts (given ids or random ids) to completion, print tokens and stats
   random-model   write a model folder (config.json, model.safetensors) from a config and a seed
+  bench-core     time the host cache core's calls alone (prefix lookup, pages, step packing)
 """
 
 from __future__ import annotations
@@ -92,6 +93,19 @@ def _random_model(args: argparse.Namespace) -> int:
     return 0
 
 
+def _bench_core(args: argparse.Namespace) -> int:
+    """Builds the cache core's micro-benchmark (csrc/core/core_bench.cpp: the reference's
+    bench/micro_core.cpp workload and three more) and runs it."""
+    import subprocess
+    import tempfile
+
+    from prefixserve_amd import build
+
+    with tempfile.TemporaryDirectory() as tmp:
+        exe = build.build_core_program(build.CSRC / "core" / "core_bench.cpp", Path(tmp) / "core_bench", what="core benchmark")
+        return subprocess.run([str(exe)], check=False).returncode
+
+
 def main(argv: list[str] | None = None) -> int:
     parser = argparse.ArgumentParser(prog="prefixserve_amd", description=__doc__,
                                      formatter_class=argparse.RawDescriptionHelpFormatter)
@@ -121,6 +135,9 @@ def main(argv: list[str] | None = None) -> int:
     r.add_argument("--norm-std", type=float, default=0.1)
     r.add_argument("--store-dtype", choices=["bfloat16", "float32"], default="bfloat16")
     r.set_defaults(run=_random_model)
+
+    c = sub.add_parser("bench-core", help="time the host cache core's calls (no GPU)")
+    c.set_defaults(run=_bench_core)
 
     args = parser.parse_args(argv)
     logging.basicConfig(level=getattr(logging, args.log_level.upper(), logging.WARNING))

@@ -26,3 +26,18 @@ def test_core_check_program(sanitize, tmp_path):
     assert "the counter counts" in out and "allocated 0 times" in out and "all core checks passed" in out
     assert out.count("ok: random workload") == 5
     assert "runtime error" not in run.stderr and "AddressSanitizer" not in run.stderr
+
+
+def test_core_benchmark_runs_and_meets_the_reference_bar(tmp_path):
+    """The core's micro-benchmark (the reference: bench/micro_core.cpp, whose bar for looking up a
+    held 2,048-token prompt is 10 microseconds): it builds with every warning an error, runs, and
+    the lookup is under the bar (the program's exit status says so); the figures it prints parse."""
+    from prefixserve_amd.build import CSRC
+
+    exe = build_core_program(CSRC / "core" / "core_bench.cpp", tmp_path / "core_bench", what="core benchmark")
+    run = subprocess.run([str(exe)], capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stdout + run.stderr
+    lines = run.stdout.strip().splitlines()
+    assert len(lines) == 4 and lines[0].startswith("lookup of 2048 held tokens")
+    figures = [float(line.split(": ")[1].split(" ns/call")[0]) for line in lines]
+    assert all(0 < f < 1e6 for f in figures) and figures[0] < 10000
