@@ -187,6 +187,22 @@ def build_kernels() -> Path:
     return out
 
 
+def build_extension(sources: list[Path], out: Path) -> Path:
+    """A shared library of device kernels from HIP sources of one's own, compiled with the flags
+    the package's kernels are compiled with (``csrc/kernels`` is on the include path, so
+    ``common.h`` may be used): what a part that brings a kernel of its own builds and then hands
+    to ``HipOps.load_extension``. Its entry points are ``extern "C"``, take the stream first
+    and return 0 or an error code."""
+    hipcc = _find("hipcc", ["/opt/rocm/bin/hipcc"])
+    out = Path(out)
+    out.parent.mkdir(parents=True, exist_ok=True)
+    tmp = out.with_suffix(f".tmp{os.getpid()}")
+    _run([hipcc, *HIPCC_FLAGS, f"-I{CSRC / 'kernels'}", "-shared", *[str(s) for s in sources], "-o", str(tmp)],
+         f"hipcc {' '.join(Path(s).name for s in sources)} -> {out.name}")
+    os.replace(tmp, out)
+    return out
+
+
 def build_all(force: bool = True) -> None:
     if force or _existing(core_module_name()) is None:
         build_core()

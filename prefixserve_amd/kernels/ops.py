@@ -13,6 +13,7 @@ from __future__ import annotations
 import contextlib
 import ctypes
 import logging
+import os
 from typing import Any, Sequence
 
 import torch
@@ -128,6 +129,37 @@ class HipOps:
     def _ok(self, rc: int) -> None:
         if rc != 0:
             raise KernelError(self.lib.psamd_last_error().decode())
+
+    # ------------------------------------------------- kernels a part brings itself
+
+    def load_extension(self, path: "str | os.PathLike[str]", signatures: dict[str, list]) -> ctypes.CDLL:
+        """Loads a library of device kernels built with ``build.build_extension`` and declares
+        its entry points (``name -> ctypes argument types``; each returns 0 or an error code):
+        how a part with a kernel of its own gets at it without a change to this file. The part
+        calls ``lib.entry(ops.stream_pointer(), tensor.data_ptr(), ...)`` and hands the result to
+        ``ops.check``; the stream is the step's, so the call may be captured like any other."""
+        try:
+            lib = ctypes.CDLL(os.fspath(path))
+        except OSError as e:
+            raise KernelError(f"cannot load the kernel library {path}: {e}") from None
+        for name, argtypes in signatures.items():
+            try:
+                fn = getattr(lib, name)
+            except AttributeError:
+                raise KernelError(f"{path} has no entry point {name}") from None
+            fn.argtypes = list(argtypes)
+            fn.restype = ctypes.c_int
+        return lib
+
+    def stream_pointer(self) -> int:
+        """The stream this step's kernels are launched on, as a kernel library takes it."""
+        return self._stream()
+
+    @staticmethod
+    def check(rc: int, what: str) -> None:
+        """Raises if an entry point of an extension returned an error code."""
+        if rc != 0:
+            raise KernelError(f"{what} failed with code {rc}")
 
     @staticmethod
     def _need(cond: bool, msg: str) -> None:

@@ -5,6 +5,8 @@ registered, built into a model and stepped without touching the package's files.
 from __future__ import annotations
 
 import math
+import tempfile
+from pathlib import Path
 
 import numpy as np
 import pytest
@@ -587,3 +589,98 @@ def test_toy_transforms_and_a_block_with_more_norms(tmp_path):
                 assert err.max() < tol, f"{dtype} positions {p0}..{p0 + c}: {err.max():.3e}"
                 p0 += c
         assert (1, 1, False) in runner._graphs                    # the single tokens went through a captured graph
+
+
+def toy_kernel_library():
+    """The test's own kernel library, compiled on first use (the build entry point compiles it
+    beforehand together with the package's)."""
+    from prefixserve_amd.build import build_extension
+
+    here = Path(__file__).resolve().parent / "toy_kernels"
+    out = here / "_lib" / "libtoy_soft_cap.so"
+    if not out.exists() or out.stat().st_mtime < (here / "soft_cap.hip").stat().st_mtime:
+        try:
+            build_extension([here / "soft_cap.hip"], out)
+        except OSError:                                           # a tree that cannot be written to
+            out = Path(tempfile.mkdtemp()) / out.name
+            build_extension([here / "soft_cap.hip"], out)
+    return out
+
+
+def test_a_part_with_a_kernel_of_its_own(tmp_path):
+    """A part that brings its own device kernel, from test files alone: a transform of the logits
+    whose HIP source lies beside this test, built with the package's flags
+    (``build.build_extension``) and loaded through ``HipOps.load_extension``; no file of the
+    package is touched. The architecture is the Llama builder's specification with that transform
+    behind the output matrix. Compared with the plain model's logits, capped, whole and token by
+    token through graphs (the kernel is launched on the step's stream, so it is captured with it),
+    in both dtypes; and the library's refusals and a missing entry point come back as errors."""
+    import ctypes
+    import dataclasses
+    import json
+
+    from configs import INIT_STD, TINY
+    from plain.llama_plain import PlainLlama
+    from prefixserve_amd.config import register_architecture, registered_architectures
+    from prefixserve_amd.config.llama import LlamaConfig
+    from prefixserve_amd.engine.replay import TraceReplayer
+    from prefixserve_amd.engine.runner import ModelRunner
+    from prefixserve_amd.kernels.ops import KernelError
+    from prefixserve_amd.models.llama import build_llama_spec
+    from prefixserve_amd.parts import PartSpec, Transform, register_transform
+    from prefixserve_amd.weights import write_random_model
+
+    CAP = 2.0
+    lib_path = toy_kernel_library()
+
+    class KernelSoftCap(Transform):
+        def __init__(self, hidden_size, vocab_size, cap):
+            self.cap = float(cap)
+
+        def bind(self, tensors, rt):
+            super().bind(tensors, rt)
+            self.ops = rt.ops
+            self.lib = rt.ops.load_extension(lib_path, {"toy_soft_cap": [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_float]})
+
+        def apply(self, t, ctx, rows):
+            assert t.dtype == torch.float32 and t.is_contiguous()
+            self.ops.check(self.lib.toy_soft_cap(self.ops.stream_pointer(), t.data_ptr(), t.numel(), self.cap), "toy_soft_cap")
+
+    def build(cfg):
+        return dataclasses.replace(build_llama_spec(cfg), logit_transforms=(PartSpec("test_kernel_softcap", {"cap": CAP}),))
+
+    if "ToyCappedLlamaForCausalLM" not in registered_architectures():
+        register_transform("test_kernel_softcap", KernelSoftCap)
+        register_architecture("ToyCappedLlamaForCausalLM", LlamaConfig, build)
+    raw = dict(TINY["B"])
+    write_random_model(tmp_path / "llama", raw, seed=12, std=INIT_STD)
+    plain = PlainLlama(tmp_path / "llama")
+    capped = tmp_path / "capped"
+    capped.mkdir()
+    (capped / "config.json").write_text(json.dumps({**raw, "architectures": ["ToyCappedLlamaForCausalLM"]}))
+    (capped / "model.safetensors").write_bytes((tmp_path / "llama" / "model.safetensors").read_bytes())
+
+    toks = np.random.default_rng(3).integers(0, raw["vocab_size"], 60).tolist()
+    n = len(toks)
+    want = CAP * np.tanh(plain.logits(toks) / CAP)
+    assert np.abs(plain.logits(toks)).max() > CAP                  # the cap is felt
+    for dtype, tol in (("float32", 2e-5), ("bfloat16", 4e-2)):
+        runner = ModelRunner(capped, dtype=dtype, device="cuda:0", num_blocks=16, max_seq_len=128, max_num_seqs=2, use_graphs=True)
+        for cuts in ([n], [25] + [1] * 35):
+            rp = TraceReplayer(runner)
+            p0 = 0
+            for kk, c in enumerate(cuts):
+                got = rp.run_step({"step": kk, "entries": [{"id": "a", "tokens": toks[p0:p0 + c], "want": list(range(c))}],
+                                   "end": ["a"] if p0 + c == n else []})
+                err = np.abs(got - want[p0:p0 + c]).max(-1) / np.abs(want[p0:p0 + c]).max(-1)
+                assert err.max() < tol, f"{dtype} positions {p0}..{p0 + c}: {err.max():.3e}"
+                p0 += c
+        assert (1, 1, False) in runner._graphs                    # the single tokens went through a captured graph
+        ops = runner.rt.ops
+    lib = ops.load_extension(lib_path, {"toy_soft_cap": [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_float]})
+    with pytest.raises(KernelError, match="code 1"):
+        ops.check(lib.toy_soft_cap(ops.stream_pointer(), None, 4, 1.0), "toy_soft_cap")
+    with pytest.raises(KernelError, match="no entry point"):
+        ops.load_extension(lib_path, {"toy_missing": [ctypes.c_void_p]})
+    with pytest.raises(KernelError, match="cannot load"):
+        ops.load_extension(tmp_path / "nothing.so", {})
