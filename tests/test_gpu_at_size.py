@@ -5,6 +5,8 @@ tiles of q/k/v columns, the grouped prefill attention at head sizes 64 and 128 w
 query heads per kv head, decode attention split over thousands of keys and merged, and the
 output matrix over 128,256 columns. Fewer layers than the real models, the same layers
 (the reference tests its attention at real head shapes, tests/gpu/test_flashinfer_vs_ref.py:48,60-67).
+And long prompts through two small models with one and with two query heads per kv head, whose
+prefill attention takes several tiles of queries per workgroup.
 """
 
 from __future__ import annotations
@@ -272,3 +274,58 @@ def test_the_pool_sized_from_free_memory_leaves_room_for_the_largest_step(sized)
         del eng, runner
         gc.collect()
         torch.cuda.empty_cache()
+
+
+FEW_HEADS_PER_KV = {
+    # one query head per kv head at head size 64, two at head size 128: long prompts then go to the
+    # form of the prefill attention in which a workgroup takes four or two consecutive tiles of queries
+    "one": dict(architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=2000, hidden_size=512,
+                intermediate_size=1024, num_hidden_layers=2, num_attention_heads=16, num_key_value_heads=16, head_dim=64,
+                rms_norm_eps=1e-5, rope_theta=10000.0, max_position_embeddings=4096, tie_word_embeddings=True),
+    "two": dict(architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=1500, hidden_size=384,
+                intermediate_size=800, num_hidden_layers=2, num_attention_heads=12, num_key_value_heads=6, head_dim=128,
+                rms_norm_eps=1e-6, rope_theta=500000.0, rope_scaling=dict(LLAMA3, factor=8.0, original_max_position_embeddings=512),
+                max_position_embeddings=4096, tie_word_embeddings=False),
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("heads", list(FEW_HEADS_PER_KV))
+def test_long_prompts_with_one_or_two_query_heads_per_kv_head(dtype, heads, tmp_path):
+    """Two prompts of 1,500 and 1,107 tokens in one step (47 + 35 tiles of queries: runs of four
+    tiles, the last of each prompt shorter, the second prompt's last tile of 19 queries), a third
+    in portions on top of what it cached, then all of them decoding together; logits at places
+    all over the prompts against the plain model."""
+    from plain.llama_plain import PlainLlama
+    from prefixserve_amd.weights import write_random_model
+
+    cfg = FEW_HEADS_PER_KV[heads]
+    write_random_model(tmp_path, cfg, seed=7, std=0.05)
+    plain = PlainLlama(tmp_path)
+    rng = np.random.default_rng(12)
+    yardstick, row_bar = plain_bf16_bars(tmp_path, plain, [rng.integers(0, cfg["vocab_size"], 130).tolist() for _ in range(3)])
+    lengths, new = (1500, 1107, 1300), 4
+    seqs = [rng.integers(0, cfg["vocab_size"], n + new).tolist() for n in lengths]
+    places = [[0, 31, 32, 127, 128, 129, 700, 1471, 1472, 1499], [5, 1087, 1088, 1106], [1299]]
+    truth = [plain.logits_at(s, list(p) + list(range(n, n + new))) for s, n, p in zip(seqs, lengths, places)]
+    runner = ModelRunner(tmp_path, dtype=dtype, device="cuda:0", num_blocks=260, max_seq_len=1536, max_num_seqs=4, use_graphs=True)
+    rp = TraceReplayer(runner)
+    errors = []
+
+    def judge(got, want):
+        errors.extend((np.abs(got - want).max(-1) / np.abs(want).max(-1)).tolist())
+
+    got = rp.run_step({"step": 0, "entries": [{"id": "r0", "tokens": seqs[0][:1500], "want": places[0]},
+                                              {"id": "r1", "tokens": seqs[1][:1107], "want": places[1]}], "end": []})
+    judge(got, np.concatenate([truth[0][:len(places[0])], truth[1][:len(places[1])]]))
+    for k, (a, b) in enumerate(((0, 600), (600, 1150), (1150, 1300))):
+        got = rp.run_step({"step": 1 + k, "entries": [{"id": "r2", "tokens": seqs[2][a:b], "want": [b - a - 1] if b == 1300 else []}], "end": []})
+    judge(got, truth[2][:1])
+    for k in range(new):
+        entries = [{"id": f"r{i}", "tokens": [s[n + k]], "want": [0]} for i, (s, n) in enumerate(zip(seqs, lengths))]
+        got = rp.run_step({"step": 10 + k, "entries": entries, "end": []})
+        judge(got, np.stack([truth[i][len(places[i]) + k] for i in range(3)]))
+    print(heads, dtype, f"worst {max(errors):.2e} mean {np.mean(errors):.2e} (plain bf16 {yardstick:.2e}, bar for a row {row_bar:.2e})", flush=True)
+    assert max(errors) < (2e-5 if dtype == "float32" else row_bar)
+    if dtype == "bfloat16":
+        assert np.mean(errors) <= yardstick
