@@ -45,11 +45,14 @@ def _llama3(hidden, inter, layers, heads, kv, dim, factor, tied):
     return cfg
 
 
-# The default is the 1B shape; the two larger ones show the kernels at another head size and width.
+# The default is the 1B shape; the larger ones show the kernels at another head size and width and with other head counts.
 SHAPES = {
     "llama-3.2-1b": LLAMA_1B,
     "llama-3.2-3b": _llama3(3072, 8192, 28, 24, 8, 128, 32.0, True),
     "llama-3.1-8b": _llama3(4096, 14336, 32, 32, 8, 128, 8.0, False),
+    # every query head with keys and values of its own, a vocabulary of 32,000, no rope scaling
+    "llama-2-7b": {**_llama3(4096, 11008, 32, 32, 32, 128, 1.0, False), "vocab_size": 32000, "rope_theta": 10000.0,
+                   "rope_scaling": None},
 }
 
 
