@@ -255,6 +255,8 @@ def main() -> int:
                                           args.context)["tok_s"]
         if args.prompt_len > 512:
             points["prefill_portions_of_512"] = prefill_run(reps=3, warm=1, portion=512)["value"]
+        if args.prompt_len > 1024:
+            points["prefill_portions_of_1024"] = prefill_run(reps=3, warm=1, portion=1024)["value"]
 
     peaks = {} if args.no_peaks else measured_peaks()      # last: a long product changes the clocks of what follows
 

@@ -28,7 +28,8 @@ def _add_engine_options(p: argparse.ArgumentParser) -> None:
     p.add_argument("--num-blocks", type=int, default=None, help="KV blocks; default: sized from free GPU memory")
     p.add_argument("--max-waiting", type=int, default=256)
     p.add_argument("--max-running-requests", type=int, default=64)
-    p.add_argument("--chunked-prefill-size", type=int, default=512)
+    p.add_argument("--chunked-prefill-size", type=int, default=2048,
+                   help="prompt tokens per step and per portion of one prompt (the reference's default is 512)")
     p.add_argument("--disable-prefix-cache", action="store_true")
     p.add_argument("--no-graphs", action="store_true", help="do not capture decode steps as HIP graphs")
     p.add_argument("--decode-steps", type=int, default=1,

@@ -39,7 +39,7 @@ def _make_ops(device: torch.device, workspace: Workspace) -> Any:
 class ModelRunner:
     def __init__(self, model_dir: str | Path, dtype: str | torch.dtype = "bfloat16", device: str = "cuda:0",
                  num_blocks: int | Sequence[int] | None = None, max_seq_len: int = 8192, max_num_seqs: int = 64,
-                 max_prefill_tokens: int = 512, reserve_bytes: int = 1 << 30, use_graphs: bool = True,
+                 max_prefill_tokens: int = 2048, reserve_bytes: int = 1 << 30, use_graphs: bool = True,
                  ops: Any = None) -> None:
         self.device = torch.device(device)
         self.dtype = DTYPES[dtype] if isinstance(dtype, str) else dtype

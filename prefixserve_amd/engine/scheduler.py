@@ -50,6 +50,8 @@ __all__ = ["AddResult", "Batch", "FinishReason", "ReqState", "Request", "Schedul
 
 log = logging.getLogger(__name__)
 
+# As the reference's scheduler (prefixserve/scheduler.py:149); an Engine hands its own
+# EngineConfig.max_prefill_tokens to the scheduler it makes, which is larger.
 DEFAULT_CHUNK_SIZE = 512
 _SLOW_PLAN_MS = 1.0
 
