@@ -44,7 +44,7 @@ int psamd_linear(void* stream, const void* x, int x_dtype, const void* w, int w_
 // psamd_gemm_lt returns 2, not an error, if the library has no algorithm for the shape.
 int psamd_gemm_lt_available();
 int psamd_gemm_lt(void* stream, const void* x, const void* w, void* out, int out_dtype, int64_t M, int N, int K,
-                  int use_workspace);
+                  int use_workspace, int accumulate);
 
 
 // bfloat16 product for M <= 64 on the matrix cores. epilogue 1: w = [gate; up], out = silu(gate) * up.

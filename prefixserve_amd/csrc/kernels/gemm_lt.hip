@@ -158,7 +158,7 @@ int psamd_gemm_lt_available() {
 }
 
 int psamd_gemm_lt(void* stream, const void* x, const void* w, void* out, int out_dtype, int64_t M, int N, int K,
-                  int use_workspace) {
+                  int use_workspace, int accumulate) {
   PSAMD_REQUIRE(M > 0 && N > 0 && K > 0 && M <= INT32_MAX, "bad sizes");
   PSAMD_REQUIRE(out_dtype == kBF16 || out_dtype == kF32, "the output is bfloat16 or float32");
   const bool float_out = out_dtype == kF32;
@@ -183,7 +183,7 @@ int psamd_gemm_lt(void* stream, const void* x, const void* w, void* out, int out
   const Plan& p = it->second;
   if (p.desc == nullptr) return 2;                         // the message of make_plan is the last error
   const float one = 1.f, zero = 0.f;
-  const hipblasStatus_t st = a.matmul(dev.handle, p.desc, &one, w, p.w, x, p.x, &zero, out, p.out, out, p.out, &p.algo,
+  const hipblasStatus_t st = a.matmul(dev.handle, p.desc, &one, w, p.w, x, p.x, accumulate ? &one : &zero, out, p.out, out, p.out, &p.algo,
                                       roomy ? dev.workspace : nullptr, roomy ? kWorkspaceBytes : 0,
                                       static_cast<hipStream_t>(stream));
   if (st != HIPBLAS_STATUS_SUCCESS) return fail("psamd_gemm_lt: hipblasLtMatmul returned " + std::to_string(st));

@@ -49,7 +49,7 @@ _SIGNATURES = {
     "psamd_swiglu": [_vp, _vp, _vp, _i32, _i64, _i32],
     "psamd_rope_kv_append": [_vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp, _vp, _vp, _vp],
     "psamd_linear": [_vp, _vp, _i32, _vp, _i32, _vp, _i32, _i64, _i32, _i32],
-    "psamd_gemm_lt": [_vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32],
+    "psamd_gemm_lt": [_vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _i32],
     "psamd_linear_skinny": [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32],
     "psamd_linear_skinny_ksplit": [_i32, _i32, _i32],
     "psamd_qkv_rope_append": [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp],
@@ -76,6 +76,7 @@ class HipOps:
     PREFILL_TILE_Q = 32    # queries per workgroup of the prefill attention kernel (its 4 waves split the keys)
     SKINNY_MAX_ROWS = 64
     FUSED_SWIGLU_MAX_ROWS = 32      # above it (to SKINNY_MAX_ROWS) gate/up goes to the library, where there is one
+    LIBRARY_ADD_MIN_ROWS = 1024     # from here on a product that feeds the residual stream adds into it in the library
     name = "hip"
 
     def __init__(self, device: torch.device | str, workspace: Any = None) -> None:
@@ -326,7 +327,7 @@ class HipOps:
             if m > self.SKINNY_MAX_ROWS and self._direct_library:
                 # Library product, as in the reference (float32 output for more than 64 rows of logits).
                 rc = self.lib.psamd_gemm_lt(self._stream(), x.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out.dtype),
-                                            m, n, k, 0 if self.fixed_kv_len else 1)
+                                            m, n, k, 0 if self.fixed_kv_len else 1, 0)
                 if rc != 2:                      # 2: no algorithm for this shape (without a workspace): the paths below
                     self._ok(rc)
                     return
@@ -357,6 +358,19 @@ class HipOps:
             self._need(w.shape[1] == k and x.is_contiguous() and w.is_contiguous(), "linear_to_residual: operands")
             self._ok(self.lib.psamd_linear_skinny_add(self._stream(), x.data_ptr(), w.data_ptr(), residual.data_ptr(), m, n, k))
             return None
+        if (residual is not None and m >= self.LIBRARY_ADD_MIN_ROWS and x.dtype == torch.bfloat16 and k % 8 == 0
+                and residual.shape == (m, n) and residual.dtype == torch.float32 and self._direct_library):
+            # A large step: the library's product adds into the float32 stream itself (out = x w^T + out),
+            # so the sum is not rounded to bfloat16 on its way there and the norm that follows reads the
+            # stream alone (2,048 rows of the 1B shape: o + norm 32.9 -> 30.2 us, down + norm 78.5 -> 76.7;
+            # at 512 rows down lost, 37.3 -> 40.7, hence the bound).
+            self._need(w.shape[1] == k and x.is_contiguous() and w.is_contiguous() and residual.is_contiguous(),
+                       "linear_to_residual: operands")
+            rc = self.lib.psamd_gemm_lt(self._stream(), x.data_ptr(), w.data_ptr(), residual.data_ptr(), _F32, m, n, k,
+                                        0 if self.fixed_kv_len else 1, 1)
+            if rc != 2:                          # 2: no algorithm for this shape: the ways below
+                self._ok(rc)
+                return None
         if x.dtype == torch.bfloat16 and k % 8 == 0 and 0 < m <= self.SKINNY_MAX_ROWS:
             ksplit = self.lib.psamd_linear_skinny_ksplit(m, n, k)
             if ksplit > 1:
@@ -396,7 +410,7 @@ class HipOps:
             # take less time than the fused form, which streams the weights with too few rows a wave.
             gu = self.ws.get("mlp.gate_up", (m, 2 * inter), x.dtype)
             rc = self.lib.psamd_gemm_lt(self._stream(), x.data_ptr(), w_gate_up.data_ptr(), gu.data_ptr(), _BF16,
-                                        m, 2 * inter, k, 0 if self.fixed_kv_len else 1)
+                                        m, 2 * inter, k, 0 if self.fixed_kv_len else 1, 0)
             if rc != 2:                          # 2: no algorithm for this shape: the fused form below
                 self._ok(rc)
                 self.swiglu(gu, out)

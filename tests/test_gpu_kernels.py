@@ -305,6 +305,30 @@ def test_linear_to_residual_adds_into_the_stream(ops, m, n, k):
     assert out is not None and rel(out.sum(0) if out.dim() == 3 else out, big.double() @ w.double().T) < 5e-3
 
 
+@pytest.mark.parametrize("m,n,k", [(1024, 2048, 2048), (2100, 2048, 8192), (1030, 200, 96), (1500, 3072, 8192)])
+def test_linear_to_residual_of_a_large_step_adds_in_the_library(ops, m, n, k):
+    """From 1,024 tokens on the library's product adds into the float32 residual itself (its sums
+    reach the stream unrounded); twice in a row adds twice, rows behind the step stay as they
+    were, and without the stream, or without the library, the product is handed back."""
+    x, w = rnd(m, k, dtype=torch.bfloat16, seed=1), rnd(n, k, dtype=torch.bfloat16, seed=2, scale=0.05)
+    start = rnd(m + 1, n, seed=3)
+    resid = start.clone()
+    prod = x.double() @ w.double().T
+    assert ops.linear_to_residual(x, w, "test.big", resid[:m]) is None
+    assert rel(resid[:m].double() - start[:m].double(), prod) < 2e-6
+    assert ops.linear_to_residual(x, w, "test.big", resid[:m]) is None
+    assert rel(resid[:m].double() - start[:m].double(), 2 * prod) < 2e-6
+    assert torch.equal(resid[m], start[m])
+    out = ops.linear_to_residual(x, w, "test.big", None)
+    assert out is not None and out.dtype == torch.bfloat16 and rel(out, prod) < 5e-3
+    ops._direct_library = False
+    try:
+        out = ops.linear_to_residual(x, w, "test.big", resid[:m])
+    finally:
+        ops._direct_library = True
+    assert out is not None and rel(out, prod) < 5e-3
+
+
 @pytest.mark.parametrize("m", [1, 2, 5, 8, 9, 16])
 @pytest.mark.parametrize("n,k,epilogue,out_dtype,wdt", [
     (8192, 2048, 1, torch.bfloat16, torch.bfloat16),      # gate/up of the 1B shape: 512 pairs of tiles
