@@ -142,6 +142,44 @@ def test_rope_kv_append(ops, act, hq, hkv, d):
     assert torch.equal(q2.float(), src.to(act).float())
 
 
+@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 64), (6, 3, 48), (24, 8, 128), (2, 1, 16)])
+def test_rope_kv_append_of_whole_pages(ops, hq, hkv, d):
+    """The tokens of prompts as a step brings them: one of 53 tokens over pages 4, 1, 5, 2 (three
+    whole pages in order and five tokens), one of 30 tokens that starts three slots into page 3
+    and so lies across the groups of 16 tokens the kernel works in, 13 tokens, then a whole page
+    again; every slot nobody wrote keeps what it held."""
+    from prefixserve_amd.parts.rope import rope_inv_freq
+
+    blocks = 9
+    slots = [16 * [4, 1, 5, 2][p // 16] + p % 16 for p in range(53)] + \
+            [16 * [3, 6, 7][(p + 3) // 16] + (p + 3) % 16 for p in range(30)] + [16 * 8 + p for p in range(16)]
+    pos = list(range(53)) + list(range(3, 33)) + list(range(16))
+    # 13 more tokens in front of the last page, so that it starts a group of 16 of the step's tokens
+    slots = slots[:83] + [16 * 0 + p for p in range(13)] + slots[83:]
+    pos = pos[:83] + list(range(13)) + pos[83:]
+    t = len(slots)
+    assert t == 112 and len(set(slots)) == t
+    qkv = rnd(t, (hq + 2 * hkv) * d, dtype=torch.bfloat16, seed=3)
+    src = qkv.clone().float()
+    inv = rope_inv_freq(d, 10000.0, None)
+    ang = torch.outer(torch.arange(64, dtype=torch.float32), inv).double()
+    table = torch.stack((ang.cos(), ang.sin()), -1).float().to(DEV).contiguous()
+    kv = torch.full((blocks, 2, hkv, 16 * d), 7.0, dtype=torch.bfloat16, device=DEV)
+    pos_t = torch.tensor(pos, dtype=torch.int32, device=DEV)
+    slots_t = torch.tensor(slots, dtype=torch.int32, device=DEV)
+    ops.rope_kv_append(qkv, hq, hkv, d, pos_t, table, kv, slots_t)
+    got = qkv[:, : (hq + hkv) * d].view(t, hq + hkv, d)
+    kp = kv[:, 0].view(blocks, hkv, 16, d)
+    vp = kv[:, 1].view(blocks, hkv, d, 16)
+    page, off = (slots_t // 16).long(), (slots_t % 16).long()
+    assert torch.equal(kp[page, :, off, :], got[:, hq:])
+    assert torch.equal(vp[page, :, :, off].float(), src[:, (hq + hkv) * d:].view(t, hkv, d))
+    untouched = torch.ones(blocks, 16, dtype=torch.bool)
+    untouched[page.cpu(), off.cpu()] = False
+    assert untouched.sum() == blocks * 16 - t
+    assert torch.all(kp.permute(0, 2, 1, 3)[untouched.to(DEV)] == 7.0) and torch.all(vp.permute(0, 3, 1, 2)[untouched.to(DEV)] == 7.0)
+
+
 @pytest.mark.parametrize("m", [1, 8, 17, 40, 64])
 @pytest.mark.parametrize("hq,hkv,d,k", [(6, 3, 48, 72), (4, 2, 16, 64), (32, 8, 64, 2048), (3, 1, 32, 96), (2, 2, 128, 200),
                                         (32, 8, 128, 264), (50, 1, 128, 72)])   # enough tiles for two per workgroup
